@@ -1,0 +1,53 @@
+"""ctypes binding of libfmscan_hip.so (interface: include/fmscan.h).
+
+There is no other implementation behind these calls: if the library cannot
+be loaded the import of `fm_amd.scan.fm_scan` fails, and tensors that are not
+on a GPU are rejected.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_int, c_int64, c_uint, c_void_p
+
+from . import build as _build
+
+ABI_VERSION = 1
+
+DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
+FLAG_PLAIN = 0x1
+FLAG_WAVES_SHIFT = 8
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the built library; builds it first only when no build exists."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not _build.LIB.exists():
+        _build.build(verbose=False)
+    lib = ctypes.CDLL(str(_build.LIB))
+    lib.fmscan_abi_version.restype = c_int
+    lib.fmscan_abi_version.argtypes = []
+    lib.fmscan_last_error.restype = c_char_p
+    lib.fmscan_last_error.argtypes = []
+    lib.fmscan_forward.restype = c_int
+    lib.fmscan_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_int64, c_int64, c_int64, c_int64, c_int, c_uint, c_void_p]
+    lib.fmscan_backward.restype = c_int
+    lib.fmscan_backward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_void_p,
+                                    c_int64, c_int64, c_int64, c_int64, c_int, c_uint, c_void_p]
+    got = lib.fmscan_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError(f"libfmscan_hip.so has ABI version {got}, this package needs {ABI_VERSION}; "
+                           "rebuild with `python -m fm_amd.build`")
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = load().fmscan_last_error().decode("utf-8", "replace")
+        raise RuntimeError(msg or f"libfmscan_hip.so returned {rc}")

@@ -1,0 +1,189 @@
+// Device-side building blocks of the gfx950 scan kernels: 16-byte packed I/O,
+// dtype <-> fp32 conversion, and the 64-lane wavefront scan of the recurrence
+// operator. Everything here is written for CDNA4 wave64 directly.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fmscan {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// ---- 16 bytes <-> E fp32 values -------------------------------------------------
+// One lane always moves 16 bytes per tensor per tile: 4 fp32 or 8 fp16/bf16
+// consecutive sequence positions. Narrow types are widened to fp32 on load and
+// rounded to nearest-even on store (the reference casts the same way,
+// fm/scan/fm_scan.cuh:14-40).
+template <typename T> struct Elem;
+
+template <> struct Elem<float> {
+    static constexpr int E = 4;
+    static constexpr uint32_t kOnes = 0x3f800000u;  // 1.0f
+    static __device__ __forceinline__ void unpack(u32x4 r, float (&f)[4]) {
+        f[0] = u2f(r.x); f[1] = u2f(r.y); f[2] = u2f(r.z); f[3] = u2f(r.w);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[4]) {
+        u32x4 r; r.x = f2u(f[0]); r.y = f2u(f[1]); r.z = f2u(f[2]); r.w = f2u(f[3]);
+        return r;
+    }
+    static __device__ __forceinline__ float widen(float v) { return v; }
+};
+
+template <> struct Elem<__bf16> {
+    static constexpr int E = 8;
+    static constexpr uint32_t kOnes = 0x3f803f80u;  // two bf16 1.0
+    static __device__ __forceinline__ void unpack(u32x4 r, float (&f)[8]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f[2 * j] = u2f(r[j] << 16);
+            f[2 * j + 1] = u2f(r[j] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f32x2 v = {f[2 * j], f[2 * j + 1]};
+            bf16x2 b = __builtin_convertvector(v, bf16x2);  // v_cvt_pk_bf16_f32, RNE
+            r[j] = __builtin_bit_cast(uint32_t, b);
+        }
+        return r;
+    }
+    static __device__ __forceinline__ float widen(__bf16 v) { return (float)v; }
+};
+
+template <> struct Elem<_Float16> {
+    static constexpr int E = 8;
+    static constexpr uint32_t kOnes = 0x3c003c00u;  // two fp16 1.0
+    static __device__ __forceinline__ void unpack(u32x4 r, float (&f)[8]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t word = r[j];  // a copy: bit_cast straight from the vector element reads element 0
+            f16x2 h = __builtin_bit_cast(f16x2, word);
+            f[2 * j] = (float)h.x;
+            f[2 * j + 1] = (float)h.y;
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f32x2 v = {f[2 * j], f[2 * j + 1]};
+            f16x2 h = __builtin_convertvector(v, f16x2);  // RNE
+            r[j] = __builtin_bit_cast(uint32_t, h);
+        }
+        return r;
+    }
+    static __device__ __forceinline__ float widen(_Float16 v) { return (float)v; }
+};
+
+// Chunk = the E consecutive elements one lane owns in a tile, starting at
+// sequence position t0 of a row. VEC: the row base and L*sizeof(T) are 16-byte
+// multiples, so a chunk is either wholly inside [0, L) or wholly outside and
+// moves as one 16-byte access. !VEC: element accesses with a bound check each;
+// `fill` is the 32-bit pattern for positions at or beyond L.
+template <typename T, bool VEC>
+__device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t0, int64_t L,
+                                            uint32_t fill) {
+    constexpr int E = Elem<T>::E;
+    u32x4 r = {fill, fill, fill, fill};
+    if constexpr (VEC) {
+        if (t0 < L) r = *reinterpret_cast<const u32x4*>(row + t0);
+    } else {
+        if (t0 < L) {
+            if constexpr (sizeof(T) == 4) {
+                const uint32_t* p = reinterpret_cast<const uint32_t*>(row);
+#pragma unroll
+                for (int i = 0; i < E; ++i)
+                    if (t0 + i < L) r[i] = p[t0 + i];
+            } else {
+                const uint16_t* p = reinterpret_cast<const uint16_t*>(row);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t lo = fill & 0xffffu, hi = fill >> 16;
+                    if (t0 + 2 * j < L) lo = p[t0 + 2 * j];
+                    if (t0 + 2 * j + 1 < L) hi = p[t0 + 2 * j + 1];
+                    r[j] = lo | (hi << 16);
+                }
+            }
+        }
+    }
+    return r;
+}
+
+template <typename T, bool VEC>
+__device__ __forceinline__ void store_chunk(T* __restrict__ row, int64_t t0, int64_t L, u32x4 r) {
+    constexpr int E = Elem<T>::E;
+    if (t0 >= L) return;
+    if constexpr (VEC) {
+#if FMSCAN_NT_STORE
+        __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(row + t0));
+#else
+        *reinterpret_cast<u32x4*>(row + t0) = r;
+#endif
+    } else {
+        if constexpr (sizeof(T) == 4) {
+            uint32_t* p = reinterpret_cast<uint32_t*>(row);
+#pragma unroll
+            for (int i = 0; i < E; ++i)
+                if (t0 + i < L) p[t0 + i] = r[i];
+        } else {
+            uint16_t* p = reinterpret_cast<uint16_t*>(row);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (t0 + 2 * j < L) p[t0 + 2 * j] = (uint16_t)(r[j] & 0xffffu);
+                if (t0 + 2 * j + 1 < L) p[t0 + 2 * j + 1] = (uint16_t)(r[j] >> 16);
+            }
+        }
+    }
+}
+
+// ---- wavefront scan ---------------------------------------------------------------
+// DPP lane permutes (data-parallel primitives: the permute happens in the VALU
+// operand path, no LDS traffic). A lane whose source lane does not exist, or
+// that the row mask switches off, receives `old`.
+constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
+constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+constexpr int kWaveShl1 = 0x130;  // lane i <- lane i+1
+constexpr int kWaveShr1 = 0x138;  // lane i <- lane i-1
+
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp(float old, float v) {
+    return u2f((uint32_t)__builtin_amdgcn_update_dpp((int)f2u(old), (int)f2u(v), CTRL, ROW_MASK,
+                                                      0xf, false));
+}
+
+// The recurrence step "h -> a*h + b" composes as (a1,b1) then (a2,b2) =
+// (a1*a2, b1*a2 + b2) (the combine at reference fm/scan/fm_scan.cuh:139-140).
+// On entry lane l holds the pair of its own chunk; on exit it holds the
+// composition of chunks 0..l: four shifted steps inside each 16-lane row, then
+// the row totals are broadcast into rows 1,3 and finally into rows 2,3.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void scan_step(float& a, float& b) {
+    const float pa = dpp<CTRL, ROW_MASK>(1.0f, a);
+    const float pb = dpp<CTRL, ROW_MASK>(0.0f, b);
+    b = __builtin_fmaf(pb, a, b);
+    a = pa * a;
+}
+
+__device__ __forceinline__ void wave_scan_inclusive(float& a, float& b) {
+    scan_step<kRowShr1, 0xf>(a, b);
+    scan_step<kRowShr2, 0xf>(a, b);
+    scan_step<kRowShr4, 0xf>(a, b);
+    scan_step<kRowShr8, 0xf>(a, b);
+    scan_step<kRowBcast15, 0xa>(a, b);
+    scan_step<kRowBcast31, 0xc>(a, b);
+}
+
+__device__ __forceinline__ float lane63(float v) {
+    return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(v), 63));
+}
+
+}  // namespace fmscan

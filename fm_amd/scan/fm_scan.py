@@ -1,0 +1,218 @@
+"""Factorization-Memory scan on MI355X: the module that stands where the reference's
+`fm/scan/fm_scan.py` stands.
+
+Exports, with the reference's names and positional signatures:
+
+    fm_scan_forward(gates, tokens, initial_state, out) -> out        fm_scan.py:9,34 / fm_scan.cuh:344-358
+    fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut,
+                     cached_output, input_tokens, gateGradOut)        fm_scan.py:11-15,35 / fm_scan.cuh:361-381
+    FM_Scan (torch.autograd.Function)                                fm_scan.py:37-81
+    fm_scan(gates, tokens, initial_state=None)                       fm_scan.py:84-99
+    fm_memory(alpha, update_scale, output_scale, inputs, ...)        fm_scan.py:102-133
+
+The two extension functions call libfmscan_hip.so through ctypes with raw device
+pointers and the current HIP stream; there is no CPU implementation behind them.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+__all__ = ["fm_scan_forward", "fm_scan_backward", "FM_Scan", "fm_scan", "fm_memory", "module"]
+
+_DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16,
+           torch.bfloat16: _lib.DTYPE_BF16}
+
+# the library is loaded when this module is imported, as the reference builds and
+# loads its extension at import (fm_scan.py:18-33); a missing library is an error here
+module = _lib.load()
+
+
+def _require(cond: bool, what: str) -> None:
+    # the reference's TORCH_CHECKs surface as RuntimeError
+    if not cond:
+        raise RuntimeError(what)
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    _require(t.dtype in _DTYPES,
+             f"Unsupported tensor dtype {t.dtype}: expecting bfloat16, float16 or float32")
+    return _DTYPES[t.dtype]
+
+
+def _on_gpu(name: str, t: torch.Tensor, dev: torch.device) -> None:
+    _require(t.is_cuda, f"{name} must be a GPU tensor (got device {t.device}); "
+                        "this scan has no CPU implementation")
+    _require(t.device == dev, f"{name} is on {t.device}, expected {dev}")
+
+
+def _flags(plain: bool, waves_per_row: int) -> int:
+    return (_lib.FLAG_PLAIN if plain else 0) | (int(waves_per_row) << _lib.FLAG_WAVES_SHIFT)
+
+
+def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per_row=0):
+    """Writes the scan states into `out` (B, M, D, L) and returns `out`.
+
+    gates (B, M, L), tokens (B, D, L), initial_state (B, M, D); everything
+    contiguous, on one GPU, of one dtype. Sizes are read from `out`, as the
+    reference launcher does (fm_scan.cuh:265-269). `plain=True` drops the
+    (1 - gate) input scaling (h_t = g_t h_{t-1} + x_t).
+    """
+    dev = out.device
+    for name, t in (("gates", gates), ("tokens", tokens), ("initial_state", initial_state),
+                    ("out", out)):
+        _on_gpu(name, t, dev)
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        _require(t.dtype == gates.dtype, f"{name} has dtype {t.dtype}, gates has {gates.dtype}")
+    _require(out.dim() == 4, "out must be (B, M, D, L)")
+    B, M, D, L = out.shape
+    _require(tuple(gates.shape) == (B, M, L), f"gates must be {(B, M, L)}, got {tuple(gates.shape)}")
+    _require(tuple(tokens.shape) == (B, D, L), f"tokens must be {(B, D, L)}, got {tuple(tokens.shape)}")
+    _require(initial_state.numel() == B * M * D, f"initial_state must hold {B * M * D} elements")
+    code = _dtype_code(gates)
+    if out.numel() == 0:
+        return out
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _lib.check(module.fmscan_forward(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+                                         out.data_ptr(), B, M, D, L, code,
+                                         _flags(plain, waves_per_row), stream))
+    return out
+
+
+def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output, input_tokens,
+                     gateGradOut, *, initial_state=None, plain=False, waves_per_row=0):
+    """Reverse scan of `outGrad` (B, M, D, L); fills `tokenGradOut` and `gateGradOut`
+    (both (B, M, D, L), one contribution per (m, d) pair) and returns None.
+
+    With the seven positional arguments alone this computes what the reference
+    extension computes, including its use of `firstPropGrad` as the state before
+    the first step in the gate gradient (fm_scan.cuh:196,380). `initial_state`
+    (B, M, D), when given, is used there instead.
+    """
+    dev = gates.device
+    named = [("gates", gates), ("outGrad", outGrad), ("firstPropGrad", firstPropGrad),
+             ("tokenGradOut", tokenGradOut), ("cached_output", cached_output),
+             ("input_tokens", input_tokens), ("gateGradOut", gateGradOut)]
+    if initial_state is not None:
+        named.append(("initial_state", initial_state))
+    for name, t in named:
+        _on_gpu(name, t, dev)
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        _require(t.dtype == gates.dtype, f"{name} has dtype {t.dtype}, gates has {gates.dtype}")
+    _require(cached_output.dim() == 4, "cached_output must be (B, M, D, L)")
+    B, M, D, L = cached_output.shape
+    full = (B, M, D, L)
+    _require(tuple(gates.shape) == (B, M, L), f"gates must be {(B, M, L)}, got {tuple(gates.shape)}")
+    _require(tuple(input_tokens.shape) == (B, D, L),
+             f"input_tokens must be {(B, D, L)}, got {tuple(input_tokens.shape)}")
+    for name, t in (("outGrad", outGrad), ("tokenGradOut", tokenGradOut), ("gateGradOut", gateGradOut)):
+        _require(tuple(t.shape) == full, f"{name} must be {full}, got {tuple(t.shape)}")
+    _require(firstPropGrad.numel() == B * M * D, f"firstPropGrad must hold {B * M * D} elements")
+    if initial_state is not None:
+        _require(initial_state.numel() == B * M * D, f"initial_state must hold {B * M * D} elements")
+    code = _dtype_code(gates)
+    if cached_output.numel() == 0:
+        return None
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _lib.check(module.fmscan_backward(
+            gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), tokenGradOut.data_ptr(),
+            cached_output.data_ptr(), input_tokens.data_ptr(), gateGradOut.data_ptr(),
+            None if initial_state is None else initial_state.data_ptr(),
+            B, M, D, L, code, _flags(plain, waves_per_row), stream))
+    return None
+
+
+class FM_Scan(torch.autograd.Function):
+    """states = FM_Scan.apply(gates, tokens, initial_state=None)
+
+    gates (B, M, L), tokens (B, D, L) -> states (B, M, D, L) in gates.dtype;
+    backward returns (d_gates (B, M, L), d_tokens (B, D, L), None)
+    (reference fm_scan.py:37-81).
+    """
+
+    @staticmethod
+    def forward(ctx, gates, tokens, initial_state=None):
+        B_g, M, L_g = gates.shape
+        B, D, L = tokens.shape
+        assert L_g == L
+        assert B_g == B
+        assert gates.is_contiguous()
+        assert tokens.is_contiguous()
+
+        given_state = initial_state is not None
+        if given_state:
+            assert initial_state.shape == (B, M, D)
+            assert initial_state.is_contiguous()
+        else:
+            initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
+
+        states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
+        fm_scan_forward(gates, tokens, initial_state, states)
+        # The state before the first step enters the gate gradient at t = 0. The
+        # reference does not keep it (fm_scan.py:55) and its kernel uses zero there;
+        # its per-timestep PyTorch path differentiates the true recurrence. Kept
+        # here only when the caller supplied one, so both agree in every case.
+        ctx.save_for_backward(tokens, gates, states, initial_state if given_state else None)
+        return states
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        tokens, gates, states, initial_state = ctx.saved_tensors
+        B, M, D, L = states.shape
+        assert states.is_contiguous()
+        assert gates.is_contiguous()
+
+        first_prop_grad = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
+        grad_output = grad_output.contiguous()
+        per_pair_gates = torch.empty_like(states)   # (B, M, D, L)
+        per_pair_tokens = torch.empty_like(states)  # (B, M, D, L)
+        fm_scan_backward(gates, grad_output, first_prop_grad, per_pair_tokens, states, tokens,
+                         per_pair_gates, initial_state=initial_state)
+
+        # (B, M, D, L) -> (B, M, L) and (B, D, L); a sum over an axis of length one
+        # is the same tensor, so it is returned as a view without another pass
+        d_gates = per_pair_gates.view(B, M, L) if D == 1 else per_pair_gates.sum(dim=2)
+        d_tokens = per_pair_tokens.view(B, D, L) if M == 1 else per_pair_tokens.sum(dim=1)
+        return d_gates, d_tokens, None
+
+
+def fm_scan(gates, tokens, initial_state=None):
+    """First-order recurrence h_t = g_t * h_{t-1} + (1 - g_t) * x_t along the last axis.
+
+    Arguments:
+        gates (torch.Tensor): (B, M, L), contiguous, on the GPU.
+        tokens (torch.Tensor): (B, D, L), contiguous, same dtype and device.
+        initial_state (torch.Tensor, optional): (B, M, D), contiguous; zeros if omitted.
+    Any L >= 1 is accepted (the reference needs a power of two in 32..131072).
+
+    Returns:
+        torch.Tensor: (B, M, D, L), the state after every step.
+    """
+    return FM_Scan.apply(gates, tokens, initial_state)
+
+
+def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True,
+              norm_eps=1e-6):
+    """The Factorization-Memory layer around the scan (reference fm_scan.py:102-133).
+
+        alpha:        (B, L, M)  mixing weights over the M memory slots
+        update_scale: (B, L, 1)
+        output_scale: (B, L, 1)
+        inputs:       (B, L, D)
+        initial_state (B, M, D), optional
+    Returns (output (B, L, D), memory_states (B, M, D, L)).
+    """
+    write = (alpha * update_scale).transpose(1, 2).contiguous()  # (B, M, L)
+    tokens = inputs.transpose(1, 2).contiguous()                 # (B, D, L)
+    memory_states = fm_scan(1.0 - write, tokens, initial_state)  # decay gate = 1 - write weight
+
+    if mem_norm:  # RMS norm over the D axis of every memory slot
+        inv_rms = torch.rsqrt(memory_states.pow(2).mean(dim=2, keepdim=True) + norm_eps)
+        memory_states = memory_states * inv_rms
+
+    read = alpha * output_scale  # (B, L, M)
+    output = torch.einsum("blm,bmdl->bld", read, memory_states).contiguous()
+    return output, memory_states

@@ -1,0 +1,117 @@
+/*
+ * fmscan.h -- C ABI of libfmscan_hip.so: the Factorization-Memory first-order
+ * linear-recurrence scan for AMD MI355X (gfx950), forward and backward.
+ *
+ *   forward :  h[b,m,d,t] = g[b,m,t] * h[b,m,d,t-1] + (1 - g[b,m,t]) * x[b,d,t]
+ *              h[b,m,d,-1] = h0[b,m,d]            (zeros when h0 == NULL)
+ *   backward:  delta[t]    = G[t] + g[t+1] * delta[t+1],  delta[L] = first_prop_grad
+ *              token_grad  = (1 - g[t]) * delta[t]
+ *              gate_grad   = (h[t-1] - x[t]) * delta[t]
+ *
+ * Every pointer is a device pointer on the GPU that is current when the call
+ * is made; all tensors are dense, row-major, sequence (L) innermost. The
+ * library owns no memory and keeps no state between calls: the caller
+ * allocates inputs and outputs, the calls enqueue kernels on `stream`
+ * (a hipStream_t, NULL = the default stream) and return without waiting.
+ *
+ * These entry points stand where the reference's two extension functions
+ * stand (reference fm/scan/fm_scan.cuh:344-358 `fm_scan_forward`, :361-381
+ * `fm_scan_backward`, with the launcher :248-331 and dtype dispatch :333-342
+ * behind them); the torch::Tensor arguments of those functions become plain
+ * pointers plus the four sizes the launcher reads from `out.sizes()` (:265-269).
+ *
+ * Return value of every int function: 0 on success, a negative FMSCAN_E_*
+ * code for a rejected argument (nothing was launched), a positive hipError_t
+ * when the HIP runtime refused the launch. fmscan_last_error() gives the text.
+ */
+#ifndef FMSCAN_H_
+#define FMSCAN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FMSCAN_ABI_VERSION 1
+
+/* element type of every tensor in one call (reference fm_scan.cuh:333-342) */
+#define FMSCAN_DTYPE_F32  0
+#define FMSCAN_DTYPE_F16  1
+#define FMSCAN_DTYPE_BF16 2
+
+/* flags */
+#define FMSCAN_FLAG_PLAIN        0x1u /* core operator h_t = g_t h_{t-1} + x_t: no (1-g) input
+                                         scaling; backward: token_grad = delta,
+                                         gate_grad = h[t-1] * delta (input_tokens unused) */
+#define FMSCAN_FLAG_WAVES_SHIFT  8    /* bits 8..11: waves cooperating on one row (1,2,4,8);
+                                         0 = let the library choose */
+#define FMSCAN_FLAG_WAVES_MASK   0xF00u
+
+/* error codes (negative returns) */
+#define FMSCAN_E_NULL      (-1) /* a required pointer is NULL */
+#define FMSCAN_E_SHAPE     (-2) /* B, M, D or L is < 1, or a size overflows */
+#define FMSCAN_E_DTYPE     (-3) /* dtype is not one of FMSCAN_DTYPE_* */
+#define FMSCAN_E_FLAGS     (-4) /* unknown flag bit or unsupported waves-per-row value */
+#define FMSCAN_E_ALIAS     (-5) /* an output overlaps an input it must not overlap */
+
+/* Version of this interface; equals FMSCAN_ABI_VERSION of the header the
+ * library was built from. No counterpart in the reference (its extension is
+ * JIT-built from source at import, fm/scan/fm_scan.py:18-33). */
+int fmscan_abi_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none).
+ * Replaces the c10::Error text of the reference's TORCH_CHECKs
+ * (fm/scan/fm_scan.cuh:329,341,346-354,367-378). */
+const char* fmscan_last_error(void);
+
+/*
+ * Forward scan. Replaces fm_scan_forward (reference fm/scan/fm_scan.cuh:344-358)
+ * and the forward instantiation of its kernel (:42-218 with reverse=false,
+ * backward=false).
+ *   gates          (B, M, L)     in
+ *   tokens         (B, D, L)     in
+ *   initial_state  (B, M, D)     in, may be NULL (= zeros)
+ *   out            (B, M, D, L)  out; must not overlap gates or tokens
+ * Any L >= 1 is accepted (the reference accepts powers of two in 32..131072,
+ * fm_scan.cuh:275-329); 16-byte vector access is used when the pointers and
+ * L * sizeof(element) are multiples of 16, element access otherwise.
+ */
+int fmscan_forward(const void* gates, const void* tokens, const void* initial_state,
+                   void* out,
+                   int64_t B, int64_t M, int64_t D, int64_t L,
+                   int dtype, unsigned flags, void* stream);
+
+/*
+ * Backward scan. Replaces fm_scan_backward (reference fm/scan/fm_scan.cuh:361-381)
+ * and the backward instantiation of its kernel (:42-218 with reverse=true,
+ * backward=true; gate shift :103-108, epilogues :184-185 and :188-208).
+ *   gates            (B, M, L)     in
+ *   out_grad         (B, M, D, L)  in   dL/dh
+ *   first_prop_grad  (B, M, D)     in, may be NULL (= zeros): gradient flowing in
+ *                                       from beyond the last step (:360)
+ *   token_grad_out   (B, M, D, L)  out  (1 - g) * delta per (m, d)
+ *   cached_output    (B, M, D, L)  in   h saved by the forward call
+ *   input_tokens     (B, D, L)     in   (ignored with FMSCAN_FLAG_PLAIN)
+ *   gate_grad_out    (B, M, D, L)  out  (h[t-1] - x[t]) * delta per (m, d)
+ *   initial_state    (B, M, D)     in, may be NULL: h[-1] used by gate_grad at t = 0.
+ *                    NULL reproduces the reference kernel, which reads its own
+ *                    `initial_state` argument there and is handed first_prop_grad
+ *                    (:196 with :380), i.e. h[-1] := first_prop_grad (zeros if that
+ *                    is NULL too). Pass the forward call's initial_state to get the
+ *                    mathematically exact gate gradient at t = 0.
+ * The two outputs must not overlap any input or each other.
+ */
+int fmscan_backward(const void* gates, const void* out_grad, const void* first_prop_grad,
+                    void* token_grad_out,
+                    const void* cached_output, const void* input_tokens,
+                    void* gate_grad_out,
+                    const void* initial_state,
+                    int64_t B, int64_t M, int64_t D, int64_t L,
+                    int dtype, unsigned flags, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FMSCAN_H_ */
