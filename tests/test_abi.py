@@ -1,0 +1,87 @@
+"""The C-ABI library loads and exports exactly what include/fmscan.h declares; rejected
+arguments come back as error codes with a message, before anything touches a GPU."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = (ROOT / "include" / "fmscan.h").read_text()
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from fm_amd import _lib
+
+    return _lib.load()
+
+
+def declared_functions():
+    code = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmscan_[a-z0-9_]+)\s*\(", code)))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_forward",
+                                    "fmscan_last_error"]
+
+
+def test_every_declared_symbol_is_exported(lib):
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+
+
+def test_abi_version_matches_header(lib):
+    want = int(re.search(r"#define\s+FMSCAN_ABI_VERSION\s+(\d+)", HEADER).group(1))
+    assert lib.fmscan_abi_version() == want
+
+
+def _const(name):
+    return int(re.search(r"#define\s+%s\s+\(?(-?\w+)\)?" % name, HEADER).group(1), 0)
+
+
+def test_python_constants_match_header():
+    from fm_amd import _lib
+
+    assert _lib.DTYPE_F32 == _const("FMSCAN_DTYPE_F32")
+    assert _lib.DTYPE_F16 == _const("FMSCAN_DTYPE_F16")
+    assert _lib.DTYPE_BF16 == _const("FMSCAN_DTYPE_BF16")
+    assert _lib.FLAG_WAVES_SHIFT == _const("FMSCAN_FLAG_WAVES_SHIFT")
+    assert _lib.FLAG_PLAIN == int(re.search(r"FMSCAN_FLAG_PLAIN\s+(0x[0-9a-f]+)u", HEADER).group(1), 16)
+
+
+P = 0x10000  # never dereferenced: every call below is rejected by the argument checks
+
+
+def fwd(lib, g=P, x=2 * P, h0=None, out=3 * P, B=1, M=1, D=1, L=8, dtype=0, flags=0):
+    return lib.fmscan_forward(g, x, h0, out, B, M, D, L, dtype, flags, None)
+
+
+def bwd(lib, g=P, G=2 * P, fpg=None, dx=3 * P, h=4 * P, x=5 * P, dg=6 * P, h0=None, B=1, M=1, D=1, L=8,
+        dtype=0, flags=0):
+    return lib.fmscan_backward(g, G, fpg, dx, h, x, dg, h0, B, M, D, L, dtype, flags, None)
+
+
+def test_rejected_arguments(lib):
+    E_NULL, E_SHAPE, E_DTYPE, E_FLAGS, E_ALIAS = (_const("FMSCAN_E_" + n) for n in
+                                                  ("NULL", "SHAPE", "DTYPE", "FLAGS", "ALIAS"))
+    assert fwd(lib, g=None) == E_NULL
+    assert b"NULL" in lib.fmscan_last_error()
+    assert fwd(lib, out=None) == E_NULL
+    assert fwd(lib, L=0) == E_SHAPE
+    assert fwd(lib, B=-1) == E_SHAPE
+    assert fwd(lib, B=1 << 20, M=1 << 20, D=1 << 20) == E_SHAPE
+    assert fwd(lib, dtype=3) == E_DTYPE
+    assert b"dtype" in lib.fmscan_last_error()
+    assert fwd(lib, flags=0x2) == E_FLAGS
+    assert fwd(lib, flags=3 << 8) == E_FLAGS          # 3 waves per row is not offered
+    assert fwd(lib, out=P) == E_ALIAS                 # out on top of gates
+    assert fwd(lib, out=2 * P + 16) == E_ALIAS        # out inside tokens
+    assert bwd(lib, h=None) == E_NULL
+    assert bwd(lib, x=None) == E_NULL                 # tokens are needed unless plain
+    assert bwd(lib, L=0) == E_SHAPE
+    assert bwd(lib, dtype=-1) == E_DTYPE
+    assert bwd(lib, dx=4 * P) == E_ALIAS              # token_grad_out on top of cached_output
+    assert bwd(lib, dg=3 * P) == E_ALIAS              # the two outputs on top of each other
+    assert b"overlaps" in lib.fmscan_last_error()

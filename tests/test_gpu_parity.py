@@ -1,0 +1,421 @@
+"""Parity of the HIP scan (through the C ABI, as fm_scan_forward / fm_scan_backward /
+FM_Scan call it) with the float64 CPU oracle, on an MI355X.
+
+Tolerance (stated by the benchmark definition): normwise error against the float64
+sequential oracle evaluated on the same, already quantised inputs,
+    max|y - ref| / max|ref| <= tol   and   ||y - ref||_2 / ||ref||_2 <= tol,
+tol = 1e-5 for float32, 1e-2 for bfloat16 / float16. Backward is checked against
+the oracle fed with the states the GPU stored, which is what the kernel reads.
+Where the arithmetic allows it the checks are bit-exact (resets, scaling by two,
+row permutation, run-to-run determinism).
+"""
+import numpy as np
+import pytest
+import torch
+
+import fm_scan_oracle as O
+import fmscan_cpu as C
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def scan():
+    import fm.scan.fm_scan as m
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return m
+
+
+def errs(y, ref):
+    y = y.detach().double().cpu().numpy().reshape(ref.shape)
+    d = y - ref
+    return (float(np.abs(d).max() / max(np.abs(ref).max(), 1e-300)),
+            float(np.linalg.norm(d.ravel()) / max(np.linalg.norm(ref.ravel()), 1e-300)))
+
+
+def check(name, y, ref, tol):
+    e_max, e_l2 = errs(y, ref)
+    assert e_max <= tol and e_l2 <= tol, f"{name}: max-norm {e_max:.3e}, l2 {e_l2:.3e} > {tol:g}"
+
+
+# ----------------------------------------------------------------------------- inputs
+
+def gpu_gen(seed=0):
+    return torch.Generator(device=DEV).manual_seed(seed)
+
+
+def baseline_inputs(cfg, dtype=None):
+    """(gates, tokens, out_grad) of BASELINE config `cfg` as (rows, 1, L) / (rows, 1, 1, L)
+    tensors: a (B, C, T) problem is the zero-copy fold B' = B*C, M = D = 1."""
+    gen = gpu_gen(0)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    ru = lambda *s: torch.rand(*s, device=DEV, generator=gen)
+    if cfg == 1:
+        B, Cn, T, dt = 2, 64, 1024, torch.float32
+        x, g, G = rn(B * Cn, 1, T), torch.sigmoid(rn(B * Cn, 1, T) + 2.0), rn(B * Cn, 1, 1, T)
+    elif cfg == 2:
+        B, Cn, T, dt = 8, 1024, 4096, torch.float32
+        x, g, G = rn(B * Cn, 1, T), 0.9 + 0.1 * ru(B * Cn, 1, T), rn(B * Cn, 1, 1, T)
+    elif cfg == 3:
+        B, Cn, T, dt = 16, 2048, 16384, torch.bfloat16
+        g = 1.0 - torch.exp(-torch.nn.functional.softplus(rn(B * Cn, 1, T)))
+        x, G = rn(B * Cn, 1, T), rn(B * Cn, 1, 1, T)
+    elif cfg == 4:
+        B, Cn, T, dt = 4, 1024, 65536, torch.bfloat16
+        g = 0.99 + 0.01 * ru(B * Cn, 1, T)
+        g[ru(B * Cn, 1, T) < 0.01] = 0.0
+        x, G = 0.1 * rn(B * Cn, 1, T), rn(B * Cn, 1, 1, T)
+    elif cfg == 5:
+        B, Cn, T, dt = 32, 4096, 2048, torch.bfloat16
+        decay = torch.exp(-torch.exp(-6.0 * ru(1, Cn, 1)))
+        g = decay.expand(B, Cn, T).reshape(B * Cn, 1, T)
+        x = (rn(B * Cn, 1, T) * rn(B * Cn, 1, T)) / 128.0
+        G = rn(B * Cn, 1, 1, T)
+    else:
+        raise ValueError(cfg)
+    dt = dtype or dt
+    return g.to(dt).contiguous(), x.to(dt).contiguous(), G.to(dt).contiguous()
+
+
+def run_fwd_bwd(scan, g, x, G, h0=None, fpg=None, **kw):
+    rows, M, L = g.shape
+    D = x.shape[1]
+    z = torch.zeros(rows, M, D, dtype=g.dtype, device=g.device)
+    out = torch.empty(rows, M, D, L, dtype=g.dtype, device=g.device)
+    scan.fm_scan_forward(g, x, z if h0 is None else h0, out, **kw)
+    dx, dg = torch.empty_like(out), torch.empty_like(out)
+    scan.fm_scan_backward(g, G, z if fpg is None else fpg, dx, out, x, dg,
+                          initial_state=z if h0 is None else h0, **kw)
+    return out, dx, dg
+
+
+def oracle_rows(g, x, G, out, idx, h0=None, fpg=None, plain=False):
+    """float64 oracle on the rows `idx` of a fold-mapped (rows, 1, L) problem."""
+    sel = lambda t: None if t is None else t[idx]
+    h_ref = C.forward_f64(sel(g), sel(x), sel(h0), plain)
+    tg, gg = C.backward_f64(sel(g), sel(G), sel(out), sel(x), sel(fpg),
+                            sel(h0) if h0 is not None else np.zeros((len(idx), 1, 1)), plain)
+    return h_ref, tg, gg
+
+
+# ----------------------------------------------------------------------------- BASELINE configs
+
+@pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
+def test_baseline_config(scan, cfg):
+    g, x, G = baseline_inputs(cfg)
+    out, dx, dg = run_fwd_bwd(scan, g, x, G)
+    torch.cuda.synchronize()
+    rows = g.shape[0]
+    if cfg in (1, 2):
+        idx = torch.arange(rows, device=DEV)
+    else:
+        pick = torch.randperm(rows, device=DEV, generator=gpu_gen(1))[:254]
+        idx = torch.cat([torch.tensor([0, rows - 1], device=DEV), pick])
+    h_ref, tg, gg = oracle_rows(g, x, G, out, idx)
+    tol = TOL[g.dtype]
+    check(f"cfg{cfg} states", out[idx], h_ref, tol)
+    check(f"cfg{cfg} token grad", dx[idx], tg, tol)
+    check(f"cfg{cfg} gate grad", dg[idx], gg, tol)
+
+    # full-size properties, bit-exact
+    out2, dx2, dg2 = run_fwd_bwd(scan, g, x, G)
+    assert torch.equal(out, out2) and torch.equal(dx, dx2) and torch.equal(dg, dg2), "not deterministic"
+    del out2, dx2, dg2
+    # doubling tokens and upstream gradient: states and token gradient double, the gate
+    # gradient (h_prev - x) * delta quadruples; scaling by two is exact in every dtype
+    o3, dx3, dg3 = run_fwd_bwd(scan, g, x * 2, G * 2)
+    assert torch.equal(o3, out * 2), "states not linear in tokens"
+    del o3
+    assert torch.equal(dx3, dx * 2)
+    assert torch.equal(dg3, dg * 4)
+    del dx3, dg3
+    if cfg == 4:  # exact resets: g == 0 -> h == x
+        zero = (g.view(rows, -1) == 0)
+        assert zero.any()
+        assert torch.equal(out.view(rows, -1)[zero], x.view(rows, -1)[zero])
+        assert torch.isfinite(out).all() and torch.isfinite(dx).all() and torch.isfinite(dg).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16])
+def test_baseline_config5_float16(scan, dtype):
+    g, x, G = baseline_inputs(5, dtype)
+    out, dx, dg = run_fwd_bwd(scan, g, x, G)
+    rows = g.shape[0]
+    idx = torch.randperm(rows, device=DEV, generator=gpu_gen(2))[:256]
+    h_ref, tg, gg = oracle_rows(g, x, G, out, idx)
+    check("states", out[idx], h_ref, TOL[dtype])
+    check("token grad", dx[idx], tg, TOL[dtype])
+    check("gate grad", dg[idx], gg, TOL[dtype])
+
+
+def test_config5_native_shape_through_autograd(scan):
+    """Config 5 read as the layer shapes it: M = 32 memory rows, D = 128 state
+    channels; gates (B, 32, T), tokens (B, 128, T), states (B, 32, 128, T)."""
+    B, M, D, L, dt = 32, 32, 128, 2048, torch.bfloat16
+    gen = gpu_gen(3)
+    decay = torch.exp(-torch.exp(-6.0 * torch.rand(1, M, 1, device=DEV, generator=gen)))
+    g = decay.expand(B, M, L).contiguous().to(dt).requires_grad_()
+    x = (torch.randn(B, D, L, device=DEV, generator=gen) *
+         torch.randn(B, D, L, device=DEV, generator=gen) / 128.0).to(dt).requires_grad_()
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    states = scan.fm_scan(g, x)
+    states.backward(G)
+    for b in (0, B - 1):
+        gb, xb, Gb = g[b:b + 1].detach(), x[b:b + 1].detach(), G[b:b + 1]
+        h_ref = C.forward_f64(gb, xb)
+        check("states", states[b:b + 1], h_ref, TOL[dt])
+        tg, gg = C.backward_f64(gb, Gb, states[b:b + 1], xb, None, np.zeros((1, M, D)))
+        check("d_gates", g.grad[b:b + 1], gg.sum(axis=2), TOL[dt])
+        check("d_tokens", x.grad[b:b + 1], tg.sum(axis=1), TOL[dt])
+
+
+# ----------------------------------------------------------------------------- shapes, dtypes, variants
+
+SHAPES = [(1, 1, 1, 1), (1, 1, 1, 7), (2, 1, 1, 32), (1, 2, 3, 33), (2, 3, 5, 512), (3, 1, 2, 1000),
+          (1, 1, 2, 4096), (2, 2, 1, 5000), (1, 1, 1, 131072), (5, 1, 1, 2048)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("waves", [0, 1, 2, 4, 8])
+@pytest.mark.parametrize("plain", [False, True])
+def test_shapes_and_variants(scan, dtype, waves, plain):
+    for (B, M, D, L) in SHAPES:
+        gen = torch.Generator().manual_seed(B * 1000 + L)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        out, dx, dg = run_fwd_bwd(scan, g, x, G, h0, fpg, plain=plain, waves_per_row=waves)
+        h_ref = C.forward_f64(g, x, h0, plain)
+        tg, gg = C.backward_f64(g, G, out, x, fpg, h0, plain)
+        tag = f"{(B, M, D, L)} {dtype} waves={waves} plain={plain}"
+        check(tag + " states", out, h_ref, TOL[dtype])
+        check(tag + " token grad", dx, tg, TOL[dtype])
+        check(tag + " gate grad", dg, gg, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_unaligned_pointers_take_the_element_path(scan, dtype):
+    """Tensors that start one element past a 16-byte boundary (still contiguous)."""
+    B, M, D, L = 2, 2, 3, 520
+    gen = torch.Generator().manual_seed(5)
+
+    def shifted(*shape):
+        n = int(np.prod(shape))
+        buf = torch.randn(n + 1, generator=gen).to(dtype).to(DEV)
+        t = buf[1:].view(*shape)
+        assert t.data_ptr() % 16 != 0 and t.is_contiguous()
+        return t
+
+    g = shifted(B, M, L).sigmoid_()
+    x, G, h0 = shifted(B, D, L), shifted(B, M, D, L), shifted(B, M, D)
+    out, dx, dg = shifted(B, M, D, L), shifted(B, M, D, L), shifted(B, M, D, L)
+    scan.fm_scan_forward(g, x, h0, out)
+    scan.fm_scan_backward(g, G, torch.zeros_like(h0), dx, out, x, dg, initial_state=h0)
+    check("states", out, C.forward_f64(g, x, h0), TOL[dtype])
+    tg, gg = C.backward_f64(g, G, out, x, None, h0)
+    check("token grad", dx, tg, TOL[dtype])
+    check("gate grad", dg, gg, TOL[dtype])
+
+
+def test_reset_and_hold_gates_are_exact(scan):
+    """g = 0 restarts the row at the token, bit-exactly in every dtype; g = 1 passes no
+    gradient to its token, exactly; long runs of exact ones and zeros give no NaN / Inf
+    and stay within tolerance of the oracle."""
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        rows, L = 64, 8192
+        gen = gpu_gen(6)
+        r = torch.rand(rows, 1, L, device=DEV, generator=gen)
+        g = torch.where(r < 0.3, torch.zeros_like(r), torch.where(r < 0.8, torch.ones_like(r), r)).to(dtype)
+        x = torch.randn(rows, 1, L, device=DEV, generator=gen).to(dtype)
+        G = torch.randn(rows, 1, 1, L, device=DEV, generator=gen).to(dtype)
+        out, dx, dg = run_fwd_bwd(scan, g, x, G)
+        g2, x2, o2 = g.view(rows, L), x.view(rows, L), out.view(rows, L)
+        assert torch.equal(o2[g2 == 0], x2[g2 == 0])
+        assert (dx.view(rows, L)[g2 == 1] == 0).all()
+        for t in (out, dx, dg):
+            assert torch.isfinite(t).all()
+        idx = torch.arange(rows, device=DEV)
+        h_ref, tg, gg = oracle_rows(g, x, G, out, idx)
+        check("states", out, h_ref, TOL[dtype])
+        check("token grad", dx, tg, TOL[dtype])
+        check("gate grad", dg, gg, TOL[dtype])
+
+
+def test_row_permutation_is_bit_exact(scan):
+    rows, L, dt = 1000, 4096, torch.bfloat16
+    gen = gpu_gen(7)
+    g = torch.rand(rows, 1, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(rows, 1, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(rows, 1, 1, L, device=DEV, generator=gen).to(dt)
+    perm = torch.randperm(rows, device=DEV, generator=gen)
+    a = run_fwd_bwd(scan, g, x, G)
+    b = run_fwd_bwd(scan, g[perm].contiguous(), x[perm].contiguous(), G[perm].contiguous())
+    for ta, tb in zip(a, b):
+        assert torch.equal(ta[perm], tb)
+
+
+def test_broadcast_rows_equal_explicit_rows(scan):
+    """(B, M, D) broadcasting equals the fold-mapped problem with gates and tokens
+    expanded by hand, bit for bit."""
+    B, M, D, L, dt = 2, 3, 4, 2048, torch.bfloat16
+    gen = gpu_gen(8)
+    g = torch.rand(B, M, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(B, D, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    out, dx, dg = run_fwd_bwd(scan, g, x, G, waves_per_row=1)
+    ge = g[:, :, None, :].expand(B, M, D, L).reshape(B * M * D, 1, L).contiguous()
+    xe = x[:, None, :, :].expand(B, M, D, L).reshape(B * M * D, 1, L).contiguous()
+    oe, dxe, dge = run_fwd_bwd(scan, ge, xe, G.view(B * M * D, 1, 1, L), waves_per_row=1)
+    assert torch.equal(out.view(-1), oe.view(-1))
+    assert torch.equal(dx.view(-1), dxe.view(-1)) and torch.equal(dg.view(-1), dge.view(-1))
+
+
+def test_segment_chaining(scan):
+    """scan(L) == scan(first part) followed by scan(rest, initial_state = last state),
+    and backward chains through first_prop_grad the same way."""
+    rows, L, k, dt = 256, 8192, 3000 // 8 * 8, torch.float32
+    gen = gpu_gen(9)
+    g = (0.9 + 0.09 * torch.rand(rows, 1, L, device=DEV, generator=gen)).to(dt)
+    x = torch.randn(rows, 1, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(rows, 1, 1, L, device=DEV, generator=gen).to(dt)
+    out, dx, dg = run_fwd_bwd(scan, g, x, G)
+    cut = lambda t, a, b: t[..., a:b].contiguous()
+    o1, _, _ = run_fwd_bwd(scan, cut(g, 0, k), cut(x, 0, k), cut(G, 0, k))
+    h_mid = o1[..., -1].contiguous()
+    o2, dx2, dg2 = run_fwd_bwd(scan, cut(g, k, L), cut(x, k, L), cut(G, k, L), h0=h_mid)
+    ref = out.double().cpu().numpy()
+    check("chained states", torch.cat([o1, o2], dim=3), ref, 1e-5)
+    # gradient crossing the cut: g[k] * delta[k]; delta[k] = dx2[k] / (1 - g[k])
+    delta_k = dx2[..., 0] / (1 - g[:, :, k].view(rows, 1, 1))
+    cross = (g[:, :, k].view(rows, 1, 1) * delta_k).contiguous()
+    _, dx1, dg1 = run_fwd_bwd(scan, cut(g, 0, k), cut(x, 0, k), cut(G, 0, k), fpg=cross)
+    check("chained token grad", torch.cat([dx1, dx2], dim=3), dx.double().cpu().numpy(), 1e-4)
+    check("chained gate grad", torch.cat([dg1, dg2], dim=3), dg.double().cpu().numpy(), 1e-4)
+
+
+# ----------------------------------------------------------------------------- autograd level
+
+def test_notebook_design(scan):
+    """The reference's only check (fm_test.ipynb:63-101): batch 1, D 5, L 32, M 1,
+    gates 0.5 + 0.5 rand, tokens rand, loss = states.sum(); kernel in bfloat16 and in
+    float32 against the per-timestep PyTorch form. Here with a seed and thresholds."""
+    from fm.scan.fm_pytorch import fm_scan_pytorch
+
+    torch.manual_seed(0)
+    gates0 = 0.5 + 0.5 * torch.rand(1, 1, 32, device=DEV)
+    tokens0 = torch.rand(1, 5, 32, device=DEV)
+    res = {}
+    for name, dt, fn in (("bf16", torch.bfloat16, scan.fm_scan), ("fp32", torch.float32, scan.fm_scan),
+                         ("loop", torch.float32, fm_scan_pytorch)):
+        g = gates0.to(dt).clone().requires_grad_()
+        x = tokens0.to(dt).clone().requires_grad_()
+        states = fn(g, x)
+        states.sum().backward()
+        res[name] = (states.detach().float().clone(), x.grad.float().clone(), g.grad.float().clone())
+    for a, b, tol in (("fp32", "loop", 1e-5), ("bf16", "loop", 2e-2), ("bf16", "fp32", 2e-2)):
+        for ta, tb, what in zip(res[a], res[b], ("states", "token grad", "gate grad")):
+            scale = tb.abs().max().item()
+            assert (ta - tb).abs().max().item() <= tol * scale, (a, b, what)
+    # and the float32 run against the float64 oracle's summed gradients
+    d_g, d_x, _ = O.backward(gates0, tokens0, np.ones((1, 1, 5, 32)))
+    check("d_gates", res["fp32"][2], d_g, 1e-5)
+    check("d_tokens", res["fp32"][1], d_x, 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_autograd_with_initial_state(scan, dtype):
+    """FM_Scan with a non-zero initial state: gradients equal the derivative of the
+    recurrence (what autograd gives through the per-timestep form), third gradient
+    is None as in the reference."""
+    B, M, D, L = 2, 3, 4, 256
+    gen = torch.Generator().manual_seed(11)
+    g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 1).to(dtype).to(DEV).requires_grad_()
+    x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV).requires_grad_()
+    h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV).requires_grad_()
+    G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+    states = scan.fm_scan(g, x, h0)
+    assert states.shape == (B, M, D, L) and states.dtype == dtype
+    states.backward(G)
+    assert h0.grad is None
+    tg, gg = C.backward_f64(g, G, states, x, None, h0)
+    check("states", states, C.forward_f64(g, x, h0), TOL[dtype])
+    check("d_gates", g.grad, gg.sum(axis=2), TOL[dtype])
+    check("d_tokens", x.grad, tg.sum(axis=1), TOL[dtype])
+
+
+def test_seven_argument_backward_reproduces_reference_kernel(scan):
+    """fm_scan_backward with the reference's seven arguments uses firstPropGrad as the
+    state before the first step (reference fm_scan.cuh:196,380)."""
+    B, M, D, L, dt = 2, 2, 2, 64, torch.float32
+    gen = torch.Generator().manual_seed(12)
+    g = torch.rand(B, M, L, generator=gen).to(DEV)
+    x = torch.randn(B, D, L, generator=gen).to(DEV)
+    G = torch.randn(B, M, D, L, generator=gen).to(DEV)
+    h0 = torch.randn(B, M, D, generator=gen).to(DEV)
+    fpg = torch.randn(B, M, D, generator=gen).to(DEV)
+    out = torch.empty(B, M, D, L, device=DEV)
+    assert scan.fm_scan_forward(g, x, h0, out) is out
+    dx, dg = torch.empty_like(out), torch.empty_like(out)
+    assert scan.fm_scan_backward(g, G, fpg, dx, out, x, dg) is None
+    tg, gg, _ = O.backward_per_row(g, G, out, x, fpg, None)
+    check("token grad", dx, tg, 1e-5)
+    check("gate grad", dg, gg, 1e-5)
+
+
+def test_fm_memory_layer(scan):
+    """The layer on top of the scan, forward and backward, against the same layer
+    built on the per-timestep PyTorch form in float64."""
+    from fm.scan.fm_pytorch import fm_scan_pytorch
+
+    B, L, M, D = 2, 512, 4, 16
+    gen = torch.Generator().manual_seed(13)
+    mk = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float64)
+    alpha64 = torch.softmax(mk(B, L, M), dim=-1)
+    us64, os64, inp64 = torch.rand(B, L, 1, generator=gen, dtype=torch.float64), \
+        torch.rand(B, L, 1, generator=gen, dtype=torch.float64), mk(B, L, D)
+    outs = {}
+    for name, dt, dev in (("gpu", torch.float32, DEV), ("ref", torch.float64, "cpu")):
+        a, u, o, i = (t.to(dt).to(dev).requires_grad_() for t in (alpha64, us64, os64, inp64))
+        if name == "gpu":
+            y, mem = scan.fm_memory(a, u, o, i)
+        else:
+            tok = i.transpose(1, 2).contiguous()
+            gate = 1.0 - (a * u).transpose(1, 2).contiguous()
+            mem = fm_scan_pytorch(gate, tok)
+            mem = mem * torch.rsqrt((mem ** 2).mean(dim=2, keepdim=True) + 1e-6)
+            y = torch.einsum("blm,bmdl->bld", a * o, mem)
+        y.square().sum().backward()
+        outs[name] = [y.detach(), mem.detach(), a.grad, u.grad, o.grad, i.grad]
+    for t_gpu, t_ref, what in zip(outs["gpu"], outs["ref"], ("output", "memory", "d_alpha", "d_update_scale",
+                                                            "d_output_scale", "d_inputs")):
+        check(what, t_gpu, t_ref.numpy(), 1e-4)
+
+
+# ----------------------------------------------------------------------------- errors on the GPU
+
+def test_argument_errors_on_gpu(scan):
+    g = torch.rand(2, 2, 64, device=DEV)
+    x = torch.rand(2, 3, 64, device=DEV)
+    z = torch.zeros(2, 2, 3, device=DEV)
+    out = torch.empty(2, 2, 3, 64, device=DEV)
+    with pytest.raises(RuntimeError, match="dtype"):
+        scan.fm_scan_forward(g, x.half(), z, out)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        scan.fm_scan_forward(g, torch.rand(2, 64, 3, device=DEV).transpose(1, 2), z, out)
+    with pytest.raises(RuntimeError, match="Unsupported tensor dtype"):
+        scan.fm_scan_forward(g.double(), x.double(), z.double(), out.double())
+    with pytest.raises(RuntimeError, match="gates must be"):
+        scan.fm_scan_forward(g[:, :1].contiguous(), x, z, out)
+    with pytest.raises(RuntimeError, match="overlaps"):
+        scan.fm_scan_forward(out.view(-1)[:256].view(2, 2, 64), x, z, out)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        scan.fm_scan_forward(g.cpu(), x, z, out)
+    # the calls above launched nothing; a valid call still works afterwards
+    scan.fm_scan_forward(g, x, z, out)
+    check("states", out, C.forward_f64(g, x), 1e-5)

@@ -1,0 +1,82 @@
+"""Host-side behaviour that needs no GPU: import paths, argument checks of the
+extension functions and of FM_Scan, and the layer arithmetic of fm_memory around
+the scan (with the scan itself replaced by the per-timestep PyTorch form)."""
+import numpy as np
+import pytest
+import torch
+
+import fm_scan_oracle as O
+
+
+def test_reference_import_paths():
+    from fm.scan.fm_pytorch import fm_scan_pytorch  # noqa: F401
+    from fm.scan.fm_scan import (FM_Scan, fm_memory, fm_scan, fm_scan_backward,  # noqa: F401
+                                 fm_scan_forward, module)
+    import fm_amd.scan.fm_scan as impl
+
+    assert fm_scan is impl.fm_scan and FM_Scan is impl.FM_Scan
+
+
+def test_product_does_not_import_the_oracle():
+    import sys
+    import subprocess
+
+    code = ("import sys; import fm.scan.fm_scan, fm.scan.fm_pytorch; "
+            "bad=[m for m in sys.modules if 'oracle' in m or m=='fmscan_cpu']; print(bad); sys.exit(bool(bad))")
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    res = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True)
+    assert res.returncode == 0, res.stdout + res.stderr
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    from fm.scan.fm_scan import fm_scan, fm_scan_backward, fm_scan_forward
+
+    g, x = torch.rand(1, 1, 32), torch.rand(1, 1, 32)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fm_scan(g, x)
+    out = torch.empty(1, 1, 1, 32)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fm_scan_forward(g, x, torch.zeros(1, 1, 1), out)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fm_scan_backward(g, out, torch.zeros(1, 1, 1), out.clone(), out, x, out.clone())
+
+
+def test_fm_scan_shape_asserts_match_reference_behaviour():
+    from fm.scan.fm_scan import fm_scan
+
+    with pytest.raises(AssertionError):  # sequence lengths differ
+        fm_scan(torch.rand(2, 1, 32), torch.rand(2, 1, 64))
+    with pytest.raises(AssertionError):  # batch sizes differ
+        fm_scan(torch.rand(2, 1, 32), torch.rand(3, 1, 32))
+    with pytest.raises(AssertionError):  # gates not contiguous
+        fm_scan(torch.rand(2, 32, 2).transpose(1, 2), torch.rand(2, 1, 32))
+    with pytest.raises(AssertionError):  # initial state of the wrong shape
+        fm_scan(torch.rand(2, 3, 32), torch.rand(2, 4, 32), torch.zeros(2, 4, 3))
+
+
+def test_fm_memory_layer_arithmetic(monkeypatch):
+    """fm_memory = gates 1 - alpha*update_scale, scan, RMS norm over D, read-out
+    einsum (reference fm_scan.py:117-131). Checked against a direct numpy
+    statement, with the scan served by the per-timestep PyTorch form."""
+    import fm_amd.scan.fm_scan as impl
+    from fm_amd.scan.fm_pytorch import fm_scan_pytorch
+
+    monkeypatch.setattr(impl, "fm_scan", fm_scan_pytorch)
+    gen = torch.Generator().manual_seed(0)
+    B, L, M, D = 2, 16, 3, 5
+    alpha = torch.softmax(torch.randn(B, L, M, generator=gen, dtype=torch.float64), dim=-1)
+    us = torch.rand(B, L, 1, generator=gen, dtype=torch.float64)
+    os_ = torch.rand(B, L, 1, generator=gen, dtype=torch.float64)
+    inp = torch.randn(B, L, D, generator=gen, dtype=torch.float64)
+    h0 = torch.randn(B, M, D, generator=gen, dtype=torch.float64)
+    for norm in (True, False):
+        out, states = impl.fm_memory(alpha, us, os_, inp, h0, mem_norm=norm, norm_eps=1e-6)
+        assert out.shape == (B, L, D) and states.shape == (B, M, D, L)
+        g = 1.0 - (alpha * us).numpy().transpose(0, 2, 1)
+        h = O.forward(g, inp.numpy().transpose(0, 2, 1), h0.numpy())
+        if norm:
+            h = h / np.sqrt((h ** 2).mean(axis=2, keepdims=True) + 1e-6)
+        ref = np.einsum("blm,bmdl->bld", (alpha * os_).numpy(), h)
+        np.testing.assert_allclose(states.numpy(), h, rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(out.numpy(), ref, rtol=1e-12, atol=1e-12)

@@ -1,0 +1,264 @@
+"""Pins the CPU oracle (oracle/fm_scan_oracle.py, oracle/fmscan_cpu.c) without the
+reference: exact rational vectors, closed forms, library routines, finite
+differences and structural identities. Each check is chosen so that a plausible
+slip (dropped (1-g) factor, gate shifted the wrong way, h[t] in place of h[t-1],
+wrong reduction axis, transposed row mapping) fails it.
+"""
+import numpy as np
+import pytest
+import torch
+from scipy.signal import lfilter
+
+import fm_scan_oracle as O
+import fmscan_cpu as C
+
+
+def rng(seed=0):
+    return np.random.default_rng(seed)
+
+
+def rand_problem(B, M, D, L, seed=0, state=True):
+    r = rng(seed)
+    g = r.random((B, M, L))
+    x = r.standard_normal((B, D, L))
+    G = r.standard_normal((B, M, D, L))
+    h0 = r.standard_normal((B, M, D)) if state else None
+    fpg = r.standard_normal((B, M, D)) if state else None
+    return g, x, G, h0, fpg
+
+
+# ------------------------------------------------------------------ exact vectors
+
+CASES = ["fm_zero_state", "fm_with_state", "fm_single_row", "fm_length_one", "plain_with_state",
+         "fm_gates_outside_unit_interval"]
+
+
+@pytest.mark.parametrize("name", CASES)
+@pytest.mark.parametrize("impl", ["numpy", "c"])
+def test_exact_rational_vectors(exact_cases, name, impl):
+    c = exact_cases[name]
+    a = lambda k: np.array(c[k], dtype=np.float64)
+    g, x, G, h0, fpg = a("gates"), a("tokens"), a("out_grad"), a("initial_state"), a("first_prop_grad")
+    plain = c["plain"]
+    if impl == "numpy":
+        h = O.forward(g, x, h0, plain)
+        tg, gg, delta = O.backward_per_row(g, G, h, x, fpg, h0, plain)
+    else:
+        h = C.forward_f64(g, x, h0, plain)
+        tg, gg = C.backward_f64(g, G, h, x, fpg, h0, plain)
+    np.testing.assert_allclose(h, a("states"), rtol=1e-14, atol=1e-14)
+    np.testing.assert_allclose(tg, a("token_grad"), rtol=1e-13, atol=1e-13)
+    np.testing.assert_allclose(gg, a("gate_grad"), rtol=1e-13, atol=1e-13)
+    if impl == "numpy":
+        d_g, d_x, d_h0 = O.backward(g, x, G, h0, plain, first_prop_grad=fpg)
+        np.testing.assert_allclose(d_g, a("gate_grad").sum(axis=2), rtol=1e-13, atol=1e-13)
+        np.testing.assert_allclose(d_x, a("token_grad").sum(axis=1), rtol=1e-13, atol=1e-13)
+        np.testing.assert_allclose(d_h0, a("d_initial_state"), rtol=1e-13, atol=1e-13)
+
+
+# ------------------------------------------------------------------ closed forms, forward
+
+def test_constant_gate_unit_input_is_geometric_series():
+    L, a = 40, 0.8
+    h = O.forward(np.full((1, 1, L), a), np.ones((1, 1, L)))
+    np.testing.assert_allclose(h[0, 0, 0], 1.0 - a ** np.arange(1, L + 1), rtol=1e-13)
+
+
+@pytest.mark.parametrize("plain", [False, True])
+def test_constant_gate_matches_iir_filter(plain):
+    L, a = 200, 0.93
+    x = rng(1).standard_normal(L)
+    h0 = 0.7
+    h = O.forward(np.full((1, 1, L), a), x[None, None], np.full((1, 1, 1), h0), plain)[0, 0, 0]
+    b = [1.0] if plain else [1.0 - a]
+    ref, _ = lfilter(b, [1.0, -a], x, zi=[a * h0])
+    np.testing.assert_allclose(h, ref, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(C.forward_f64(np.full((1, 1, L), a), x[None, None], np.full((1, 1, 1), h0), plain)
+                               [0, 0, 0], ref, rtol=1e-12, atol=1e-12)
+
+
+def test_plain_unit_gate_is_cumulative_sum():
+    x = rng(2).standard_normal((2, 3, 50))
+    h = O.forward(np.ones((2, 1, 50)), x, None, plain=True)
+    np.testing.assert_allclose(h[:, 0], np.cumsum(x, axis=2), rtol=1e-13, atol=1e-13)
+
+
+def test_reset_hold_and_fixed_point():
+    r = rng(3)
+    x = r.standard_normal((2, 3, 17))
+    h0 = r.standard_normal((2, 2, 3))
+    # gate 0: the state is the token, for every memory row
+    h = O.forward(np.zeros((2, 2, 17)), x, h0)
+    assert np.array_equal(h, np.broadcast_to(x[:, None], h.shape))
+    # gate 1: the state never moves
+    h = O.forward(np.ones((2, 2, 17)), x, h0)
+    assert np.array_equal(h, np.broadcast_to(h0[..., None], h.shape))
+    # tokens == state == c: convex combination keeps c whatever the gates are
+    g = r.random((2, 2, 17))
+    h = O.forward(g, np.full((2, 3, 17), 0.25), np.full((2, 2, 3), 0.25))
+    np.testing.assert_allclose(h, 0.25, rtol=1e-14)
+
+
+def test_convexity_bounds():
+    g, x, _, _, _ = rand_problem(2, 2, 3, 64, seed=4, state=False)
+    h = O.forward(g, x)
+    hi = np.maximum.accumulate(np.maximum(x, 0.0), axis=2)[:, None]
+    lo = np.minimum.accumulate(np.minimum(x, 0.0), axis=2)[:, None]
+    assert np.all(h <= hi + 1e-12) and np.all(h >= lo - 1e-12)
+
+
+def test_row_mapping_against_scalar_loops():
+    """(B, M, D) broadcasting: every output row equals the one-row scan of its own
+    gate row b*M+m and token row b*D+d, written as a scalar Python loop."""
+    g, x, _, h0, _ = rand_problem(2, 3, 4, 11, seed=5)
+    h = O.forward(g, x, h0)
+    hc = C.forward_f64(g, x, h0)
+    for b in range(2):
+        for m in range(3):
+            for d in range(4):
+                s = h0[b, m, d]
+                for t in range(11):
+                    s = g[b, m, t] * s + (1.0 - g[b, m, t]) * x[b, d, t]
+                    assert abs(h[b, m, d, t] - s) < 1e-14
+                    assert abs(hc[b, m, d, t] - s) < 1e-14
+
+
+def test_segment_chaining_and_linearity():
+    g, x, _, h0, _ = rand_problem(2, 2, 2, 64, seed=6)
+    h = O.forward(g, x, h0)
+    first = O.forward(g[..., :24], x[..., :24], h0)
+    second = O.forward(g[..., 24:], x[..., 24:], first[..., -1])
+    np.testing.assert_allclose(np.concatenate([first, second], axis=3), h, rtol=1e-14, atol=1e-14)
+    x2 = rng(7).standard_normal(x.shape)
+    h2 = O.forward(g, x2, 0 * h0)
+    np.testing.assert_allclose(O.forward(g, 2 * x - 3 * x2, 2 * h0), 2 * h - 3 * h2, rtol=1e-12, atol=1e-12)
+
+
+# ------------------------------------------------------------------ backward
+
+def fd_grad(f, a, eps=1e-6):
+    out = np.zeros_like(a)
+    it = np.nditer(a, flags=["multi_index"])
+    for _ in it:
+        i = it.multi_index
+        old = a[i]
+        a[i] = old + eps
+        fp = f()
+        a[i] = old - eps
+        fm = f()
+        a[i] = old
+        out[i] = (fp - fm) / (2 * eps)
+    return out
+
+
+@pytest.mark.parametrize("plain", [False, True])
+def test_backward_matches_finite_differences(plain):
+    g, x, G, h0, _ = rand_problem(2, 2, 3, 7, seed=8)
+    loss = lambda: float((G * O.forward(g, x, h0, plain)).sum())
+    d_g, d_x, d_h0 = O.backward(g, x, G, h0, plain)
+    np.testing.assert_allclose(d_g, fd_grad(loss, g), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(d_x, fd_grad(loss, x), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(d_h0, fd_grad(loss, h0), rtol=1e-6, atol=1e-7)
+
+
+def test_backward_constant_gate_closed_form():
+    # G == 1, constant gate a: delta[t] = (1 - a^(L-t)) / (1 - a)
+    L, a = 30, 0.9
+    g = np.full((1, 1, L), a)
+    x = rng(9).standard_normal((1, 1, L))
+    h = O.forward(g, x)
+    tg, gg, delta = O.backward_per_row(g, np.ones((1, 1, 1, L)), h, x)
+    expect = (1.0 - a ** (L - np.arange(L))) / (1.0 - a)
+    np.testing.assert_allclose(delta[0, 0, 0], expect, rtol=1e-12)
+    np.testing.assert_allclose(tg[0, 0, 0], (1.0 - a) * expect, rtol=1e-12)
+    hprev = np.concatenate([[0.0], h[0, 0, 0, :-1]])
+    np.testing.assert_allclose(gg[0, 0, 0], (hprev - x[0, 0]) * expect, rtol=1e-12)
+
+
+def test_adjoint_identity():
+    """Forward is linear in the tokens: <G, J v> == <J^T G, v>."""
+    g, x, G, _, _ = rand_problem(2, 3, 2, 33, seed=10, state=False)
+    v = rng(11).standard_normal(x.shape)
+    _, d_x, _ = O.backward(g, x, G)
+    lhs = float((G * O.forward(g, v)).sum())
+    np.testing.assert_allclose(lhs, float((d_x * v).sum()), rtol=1e-12)
+
+
+def test_first_prop_grad_chains_segments():
+    """Backward over [0, L) equals backward over the second half, then the first half
+    fed with the gradient that crosses the cut (g[k] * delta[k])."""
+    g, x, G, h0, _ = rand_problem(1, 2, 2, 32, seed=12)
+    h = O.forward(g, x, h0)
+    tg, gg, delta = O.backward_per_row(g, G, h, x, None, h0)
+    k = 20
+    tg2, gg2, d2 = O.backward_per_row(g[..., k:], G[..., k:], h[..., k:], x[..., k:], None, h[..., k - 1])
+    cross = g[:, :, k][:, :, None] * d2[..., 0]
+    tg1, gg1, _ = O.backward_per_row(g[..., :k], G[..., :k], h[..., :k], x[..., :k], cross, h0)
+    np.testing.assert_allclose(np.concatenate([tg1, tg2], 3), tg, rtol=1e-13, atol=1e-13)
+    np.testing.assert_allclose(np.concatenate([gg1, gg2], 3), gg, rtol=1e-13, atol=1e-13)
+
+
+def test_kernel_literal_mode_differs_only_at_first_step():
+    """Without an initial state handed to backward the reference kernel takes
+    first_prop_grad as h[-1]: only gate_grad[..., 0] changes, by (h0 - fpg) * delta[0]."""
+    g, x, G, h0, fpg = rand_problem(2, 2, 2, 9, seed=13)
+    h = O.forward(g, x, h0)
+    tg_e, gg_e, delta = O.backward_per_row(g, G, h, x, fpg, h0)
+    tg_k, gg_k, _ = O.backward_per_row(g, G, h, x, fpg, None)
+    assert np.array_equal(tg_e, tg_k)
+    assert np.array_equal(gg_e[..., 1:], gg_k[..., 1:])
+    np.testing.assert_allclose(gg_e[..., 0] - gg_k[..., 0], (h0 - fpg) * delta[..., 0], rtol=1e-13)
+    tc, gc = C.backward_f64(g, G, h, x, fpg, None)
+    np.testing.assert_allclose(gc, gg_k, rtol=1e-14, atol=1e-14)
+
+
+def test_torch_loop_autograd_agrees_with_oracle():
+    """The per-timestep PyTorch form (product module fm_amd.scan.fm_pytorch, the
+    counterpart of the reference's CPU path) differentiated by autograd gives the
+    oracle's analytic gradients, the one for the initial state included."""
+    from fm_amd.scan.fm_pytorch import fm_scan_pytorch
+
+    g, x, G, h0, _ = rand_problem(2, 3, 4, 19, seed=14)
+    tg = torch.tensor(g, requires_grad=True)
+    tx = torch.tensor(x, requires_grad=True)
+    th = torch.tensor(h0, requires_grad=True)
+    states = fm_scan_pytorch(tg, tx, th)
+    np.testing.assert_allclose(states.detach().numpy(), O.forward(g, x, h0), rtol=1e-13, atol=1e-13)
+    (states * torch.tensor(G)).sum().backward()
+    d_g, d_x, d_h0 = O.backward(g, x, G, h0)
+    np.testing.assert_allclose(tg.grad.numpy(), d_g, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(tx.grad.numpy(), d_x, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(th.grad.numpy(), d_h0, rtol=1e-12, atol=1e-12)
+
+
+# ------------------------------------------------------------------ compiled oracle and port
+
+@pytest.mark.parametrize("plain", [False, True])
+def test_c_oracle_equals_numpy_oracle(plain):
+    g, x, G, h0, fpg = rand_problem(3, 2, 5, 257, seed=15)
+    h = O.forward(g, x, h0, plain)
+    np.testing.assert_allclose(C.forward_f64(g, x, h0, plain), h, rtol=1e-14, atol=1e-14)
+    for state in (h0, None):
+        tg, gg, _ = O.backward_per_row(g, G, h, x, fpg, state, plain)
+        tc, gc = C.backward_f64(g, G, h, x, fpg, state, plain)
+        np.testing.assert_allclose(tc, tg, rtol=1e-14, atol=1e-14)
+        np.testing.assert_allclose(gc, gg, rtol=1e-14, atol=1e-14)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+def test_cpu_port_within_tolerance_of_f64(dtype, tol):
+    gen = torch.Generator().manual_seed(16)
+    B, M, D, L = 2, 2, 3, 1000
+    g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype)
+    x = torch.randn(B, D, L, generator=gen).to(dtype)
+    G = torch.randn(B, M, D, L, generator=gen).to(dtype)
+    h0 = torch.randn(B, M, D, generator=gen).to(dtype)
+    out = torch.empty(B, M, D, L, dtype=dtype)
+    C.port_forward(g, x, h0, out)
+    ref = C.forward_f64(g, x, h0)
+    nerr = lambda a, r: np.abs(a.double().numpy() - r).max() / np.abs(r).max()
+    assert nerr(out, ref) <= tol
+    dx, dg = torch.empty_like(out), torch.empty_like(out)
+    C.port_backward(g, G, None, dx, out, x, dg, initial_state=h0)
+    tr, gr = C.backward_f64(g, G, out, x, None, h0)
+    assert nerr(dx, tr) <= tol and nerr(dg, gr) <= tol
