@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the Factorization-Memory scan on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3]
+
+One step = one forward scan + one backward scan over one batch of synthetic
+input that is already resident in HBM, through the extension entry points
+(`fm_scan_forward`, `fm_scan_backward`: ctypes -> C ABI -> HIP kernels) on
+pre-allocated outputs. The default workload is the headline configuration:
+bfloat16, (B, C, T) = (16, 2048, 16384), passed as B' = B*C rows with M = D = 1.
+
+Prints one JSON line. `value` is the effective HBM bandwidth of the step:
+algorithmic bytes (9 * element size per element: forward reads g, x and writes h;
+backward reads g, dL/dh, h, x and writes the two gradients) divided by wall
+time. `roofline` prices the backward kernel, the dominant one, from HIP events
+recorded around it inside the timed region. `cpu_baseline` times the compiled CPU
+port of the same scan (oracle/fmscan_cpu.c) on this host's cores on a bounded
+row sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_HBM_GBPS = 8000.0  # MI355X HBM3E, published
+
+METRIC = "fwd+bwd scan effective HBM GB/s (% of MI355X peak), bf16 B16 C2048 T16384"
+
+# (B, C, T, dtype name, gate law)
+WORKLOADS = {
+    "cfg1": (2, 64, 1024, "float32"),
+    "cfg2": (8, 1024, 4096, "float32"),
+    "cfg3": (16, 2048, 16384, "bfloat16"),
+    "cfg4": (4, 1024, 65536, "bfloat16"),
+    "cfg5": (32, 4096, 2048, "bfloat16"),
+}
+
+# HBM bytes per backward launch read from rocprofv3 counters (FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a copy of known
+# size); the runs are summarised under profiles/. None = not measured.
+MEASURED_BWD_TRAFFIC_BYTES = {}
+
+
+def make_inputs(torch, name, device):
+    B, Cn, T, dtn = WORKLOADS[name]
+    dt = getattr(torch, dtn)
+    rows = B * Cn
+    gen = torch.Generator(device=device).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=device, generator=gen)
+    ru = lambda *s: torch.rand(*s, device=device, generator=gen)
+    if name == "cfg1":
+        g = torch.sigmoid(rn(rows, 1, T) + 2.0)
+        x = rn(rows, 1, T)
+    elif name == "cfg2":
+        g = 0.9 + 0.1 * ru(rows, 1, T)
+        x = rn(rows, 1, T)
+    elif name == "cfg3":
+        g = 1.0 - torch.exp(-torch.nn.functional.softplus(rn(rows, 1, T)))
+        x = rn(rows, 1, T)
+    elif name == "cfg4":
+        g = 0.99 + 0.01 * ru(rows, 1, T)
+        g[ru(rows, 1, T) < 0.01] = 0.0
+        x = 0.1 * rn(rows, 1, T)
+    else:
+        g = torch.exp(-torch.exp(-6.0 * ru(1, Cn, 1))).expand(B, Cn, T).reshape(rows, 1, T)
+        x = rn(rows, 1, T) * rn(rows, 1, T) / 128.0
+    G = rn(rows, 1, 1, T)
+    return g.to(dt).contiguous(), x.to(dt).contiguous(), G.to(dt).contiguous()
+
+
+def cpu_baseline(torch, g, x, G, budget_s=12.0):
+    """Times the CPU port on the first rows of the workload (at most 1/8 of them)."""
+    sys.path.insert(0, str(ROOT / "oracle"))
+    import fmscan_cpu as C
+
+    rows, _, T = g.shape
+    n = max(1, min(rows, max(rows // 8, 128)))
+    gc, xc, Gc = g[:n].cpu().contiguous(), x[:n].cpu().contiguous(), G[:n].cpu().contiguous()
+    out = torch.empty(n, 1, 1, T, dtype=g.dtype)
+    dx, dg = torch.empty_like(out), torch.empty_like(out)
+    threads = C.max_threads()
+
+    def one_pass():
+        C.port_forward(gc, xc, None, out)
+        C.port_backward(gc, Gc, None, dx, out, xc, dg)
+
+    one_pass()  # warm up: thread pool, page faults of the outputs
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        one_pass()
+        passes += 1
+        el = time.perf_counter() - t0
+        if (el >= budget_s and passes >= 3) or el >= 2.5 * budget_s:
+            break
+    s = g.element_size()
+    gbps = 9 * s * n * T * passes / el / 1e9
+    return {"value": round(gbps, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "elements_per_s": round(n * T * passes / el, 1),
+            "sample": f"first {n} of {rows} rows x T={T} ({g.dtype}), fwd+bwd, {passes} passes in "
+                      f"{el:.1f} s, C port oracle/fmscan_cpu.c with OpenMP over rows"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--waves-per-row", type=int, default=0, help="0 = library's choice")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--probe", action="store_true",
+                    help="for rocprofv3 --pmc runs: a few launches of an elementwise copy of known "
+                         "size (torch.neg, reads and writes one tensor), then of the two scan "
+                         "kernels; no timing, no JSON")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; rows are independent, so more GPUs would "
+              "each run the same kernels on a slice of the rows. Use --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the scan has no CPU path to benchmark", file=sys.stderr)
+        return 1
+    from fm.scan.fm_scan import fm_scan_backward, fm_scan_forward
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    B, Cn, T, dtn = WORKLOADS[args.workload]
+    g, x, G = make_inputs(torch, args.workload, dev)
+    rows = B * Cn
+    zeros = torch.zeros(rows, 1, 1, dtype=g.dtype, device=dev)
+    out = torch.empty(rows, 1, 1, T, dtype=g.dtype, device=dev)
+    dx, dg = torch.empty_like(out), torch.empty_like(out)
+    W = args.waves_per_row
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        fm_scan_forward(g, x, zeros, out, waves_per_row=W)
+        if ev:
+            ev[1].record()
+        fm_scan_backward(g, G, zeros, dx, out, x, dg, waves_per_row=W)
+        if ev:
+            ev[2].record()
+
+    if args.probe:
+        for _ in range(4):
+            torch.neg(out, out=dx)
+        for _ in range(4):
+            step()
+        torch.cuda.synchronize()
+        print(f"probe: torch.neg reads and writes {out.numel() * out.element_size()} bytes each; "
+              f"forward algorithmic bytes {3 * g.element_size() * rows * T}, "
+              f"backward {6 * g.element_size() * rows * T}")
+        return 0
+
+    for _ in range(args.warmup):
+        step()
+    # the kernels run on torch's current stream, so torch events bracket them
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    s = g.element_size()
+    N = rows * T
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = 9 * s * N / (ms_per_step * 1e-3) / 1e9
+    bwd_bytes = 6 * s * N
+    achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"bfloat16": "bf16", "float32": "f32", "float16": "f16"}[dtn] + " storage, f32 arithmetic",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: (B,C,T)=({B},{Cn},{T}) {dtn}, fwd+bwd, passed as "
+                               f"{rows} rows with M=D=1, FM form h=g*h+(1-g)*x",
+                   "bytes_per_element": 9 * s, "elements": N},
+        "pct_of_peak": round(100 * value / PEAK_HBM_GBPS, 2),
+        "elements_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "fwd_ms": round(fwd_ms, 4),
+        "bwd_ms": round(bwd_ms, 4),
+        "fwd_GBps": round(3 * s * N / (fwd_ms * 1e-3) / 1e9, 1),
+        "roofline": {"kernel": "scan_backward_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBPS, 4),
+                     "algorithmic_bytes": bwd_bytes,
+                     "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.workload)},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, g, x, G)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
