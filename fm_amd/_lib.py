@@ -16,6 +16,8 @@ ABI_VERSION = 1
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 FLAG_PLAIN = 0x1
 FLAG_WAVES_SHIFT = 8
+FLAG_BLOCKS_SHIFT = 12
+FLAG_DEPTH_SHIFT = 16
 
 _lib = None
 

@@ -28,7 +28,6 @@ HIPCC_FLAGS = [
     "-shared",
     # keep hipcc from forming packed fp32 VALU ops out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-DFMSCAN_NT_STORE=0",
 ]
 
 

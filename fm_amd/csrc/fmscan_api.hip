@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -36,6 +37,8 @@ struct Problem {
     int64_t B, M, D, L, rows;
     int esize;
     unsigned waves;  // requested waves per row, 0 = auto
+    unsigned blocks_per_cu;  // requested cap on resident blocks per CU, 0 = auto
+    unsigned depth;          // requested prefetch depth in tiles, 0 = auto
     bool plain;
 };
 
@@ -48,7 +51,8 @@ int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
     if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16)
         return fail(FMSCAN_E_DTYPE, "fmscan: dtype %d is not float32 (0), float16 (1) or bfloat16 (2)",
                     dtype);
-    if (flags & ~(FMSCAN_FLAG_PLAIN | FMSCAN_FLAG_WAVES_MASK))
+    if (flags & ~(FMSCAN_FLAG_PLAIN | FMSCAN_FLAG_WAVES_MASK | FMSCAN_FLAG_BLOCKS_MASK |
+                  FMSCAN_FLAG_DEPTH_MASK))
         return fail(FMSCAN_E_FLAGS, "fmscan: unknown flag bits 0x%x", flags);
     const unsigned waves = (flags & FMSCAN_FLAG_WAVES_MASK) >> FMSCAN_FLAG_WAVES_SHIFT;
     if (waves != 0 && waves != 1 && waves != 2 && waves != 4 && waves != 8)
@@ -62,22 +66,15 @@ int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
     pb->rows = (int64_t)rows;
     pb->esize = dtype == FMSCAN_DTYPE_F32 ? 4 : 2;
     pb->waves = waves;
+    pb->blocks_per_cu = (flags & FMSCAN_FLAG_BLOCKS_MASK) >> FMSCAN_FLAG_BLOCKS_SHIFT;
+    pb->depth = (flags & FMSCAN_FLAG_DEPTH_MASK) >> FMSCAN_FLAG_DEPTH_SHIFT;
+    if (pb->depth != 0 && (pb->depth < 2 || pb->depth > 4))
+        return fail(FMSCAN_E_FLAGS, "fmscan: prefetch depth must be 0 (auto), 2, 3 or 4 (got %u)", pb->depth);
     pb->plain = (flags & FMSCAN_FLAG_PLAIN) != 0;
     return 0;
 }
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
-
-// Waves per row when the caller leaves the choice to the library. A wave walks
-// its row alone unless there are too few rows to fill the chip that way
-// (256 CUs x 4 SIMDs x several waves) and the row is long enough to share.
-unsigned choose_waves(const Problem& pb) {
-    if (pb.waves) return pb.waves;
-    const int64_t tile1 = (16 / pb.esize) * 64;  // elements one wave covers per tile
-    unsigned w = 1;
-    while (w < 8 && pb.rows * w < 8192 && pb.L >= (int64_t)tile1 * w * 2) w *= 2;
-    return w;
-}
 
 int launched(const char* what) {
     const hipError_t e = hipGetLastError();
@@ -85,42 +82,113 @@ int launched(const char* what) {
     return 0;
 }
 
-template <typename T, int W, int R, bool PLAIN, bool VEC>
-void launch_fwd(const Problem& pb, const void* g, const void* x, const void* h0, void* out,
+// One block per R rows. Each block also asks for a share of the 160 KiB of LDS of a
+// compute unit that it never touches: at most `blocks_per_cu` blocks then fit a unit
+// at a time, which bounds the number of rows that stream concurrently.
+struct Grid {
+    unsigned blocks, lds;
+};
+Grid throttled_grid(const void* kern, int64_t rows, int R, unsigned blocks_per_cu) {
+    Grid g;
+    g.blocks = (unsigned)((rows + R - 1) / R);
+    g.lds = ((160u * 1024u - 2048u) / blocks_per_cu) & ~1023u;
+    static std::atomic<uint64_t> last_set{~0ull};  // (kernel, device, bytes) of the last attribute call
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const uint64_t key = ((uint64_t)(uintptr_t)kern << 24) ^ ((uint64_t)dev << 20) ^ g.lds;
+    if (last_set.load(std::memory_order_relaxed) != key) {
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess) {
+            (void)hipGetLastError();
+            g.lds = 0;
+        } else {
+            last_set.store(key, std::memory_order_relaxed);
+        }
+    }
+    return g;
+}
+
+// Waves per row, resident blocks per compute unit and prefetch depth when the caller
+// leaves the choice to the library. The table comes from sweeps on an MI355X over the
+// benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536 in 16-bit types
+// and 8192 x 4096 in float32. What it encodes: a wave per row streams best when there are
+// many rows of moderate length; long rows want several waves side by side so that fewer
+// rows are open at a time; with few rows a block per row keeps every compute unit busy.
+// About two waves per SIMD is where HBM efficiency peaks; more resident rows lower it.
+struct Tuning {
+    unsigned waves, blocks_per_cu, depth;
+};
+Tuning choose(const Problem& pb) {
+    Tuning t;
+    const int64_t tile1 = (16 / pb.esize) * 64;               // elements one wave covers per tile
+    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;        // tiles per row for one wave
+    unsigned w = pb.waves;
+    if (!w) {
+        if (tiles1 >= 64) w = 4;
+        else if (pb.rows < 16384 && tiles1 >= 8) w = 8;
+        else w = 1;
+        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                                     // row shorter than a tile
+        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;           // very few rows
+    }
+    t.waves = w;
+    if (pb.blocks_per_cu) t.blocks_per_cu = pb.blocks_per_cu;
+    else if (w == 1) t.blocks_per_cu = tiles1 >= 16 ? 2 : 4;
+    else if (w == 4) t.blocks_per_cu = 2;
+    else t.blocks_per_cu = 4;
+    if (pb.depth) t.depth = pb.depth;
+    else if (w == 1) t.depth = tiles1 >= 16 ? 3 : 4;
+    else if (w == 4) t.depth = 4;
+    else t.depth = 3;
+    return t;
+}
+
+template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
+void launch_fwd(const Problem& pb, unsigned bpc, const void* g, const void* x, const void* h0, void* out,
                 hipStream_t s) {
-    const unsigned grid = (unsigned)((pb.rows + R - 1) / R);
-    fmscan::scan_forward_kernel<T, W, R, PLAIN, VEC><<<grid, 64 * W * R, 0, s>>>(
+    auto kern = fmscan::scan_forward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
+    const Grid grid = throttled_grid((const void*)kern, pb.rows, R, bpc);
+    kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>(
         (const T*)g, (const T*)x, (const T*)h0, (T*)out, pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L);
 }
 
-template <typename T, int W, int R, bool PLAIN, bool VEC>
-void launch_bwd(const Problem& pb, const void* g, const void* G, const void* fpg, void* dx,
+template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
+void launch_bwd(const Problem& pb, unsigned bpc, const void* g, const void* G, const void* fpg, void* dx,
                 const void* h, const void* x, void* dg, const void* h0, hipStream_t s) {
-    const unsigned grid = (unsigned)((pb.rows + R - 1) / R);
-    fmscan::scan_backward_kernel<T, W, R, PLAIN, VEC><<<grid, 64 * W * R, 0, s>>>(
+    auto kern = fmscan::scan_backward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
+    const Grid grid = throttled_grid((const void*)kern, pb.rows, R, bpc);
+    kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>(
         (const T*)g, (const T*)G, (const T*)fpg, (T*)dx, (const T*)h, (const T*)x, (T*)dg,
         (const T*)h0, pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L);
 }
 
-// Expands the run-time choices (dtype, waves per row, plain, vector access) into
-// the kernel template arguments. F is a generic lambda called with tag values.
+// Expands the run-time choices (dtype, waves per row, prefetch depth, plain, vector
+// access) into the kernel template arguments. F is a generic lambda called with tags.
 template <typename T> struct TypeTag { using type = T; };
 template <int V> struct IntTag { static constexpr int value = V; };
 template <bool V> struct BoolTag { static constexpr bool value = V; };
 
 template <typename F>
-void dispatch(int dtype, unsigned waves, bool plain, bool vec, F&& f) {
+void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f) {
     auto with_type = [&](auto tt) {
         auto with_waves = [&](auto wt, auto rt) {
-            if (plain) {
-                if (vec) f(tt, wt, rt, BoolTag<true>{}, BoolTag<true>{});
-                else f(tt, wt, rt, BoolTag<true>{}, BoolTag<false>{});
-            } else {
-                if (vec) f(tt, wt, rt, BoolTag<false>{}, BoolTag<true>{});
-                else f(tt, wt, rt, BoolTag<false>{}, BoolTag<false>{});
+            auto with_depth = [&](auto dt, auto vt, auto ft) {
+                if (plain) f(tt, wt, rt, dt, BoolTag<true>{}, vt, ft);
+                else f(tt, wt, rt, dt, BoolTag<false>{}, vt, ft);
+            };
+            if (!vec) {  // element access: the slow path gets one variant
+                with_depth(IntTag<2>{}, BoolTag<false>{}, BoolTag<false>{});
+                return;
+            }
+            auto with_fold = [&](auto dt) {
+                if (fold) with_depth(dt, BoolTag<true>{}, BoolTag<true>{});
+                else with_depth(dt, BoolTag<true>{}, BoolTag<false>{});
+            };
+            switch (t.depth) {
+                case 2: with_fold(IntTag<2>{}); break;
+                case 3: with_fold(IntTag<3>{}); break;
+                default: with_fold(IntTag<4>{}); break;
             }
         };
-        switch (waves) {
+        switch (t.waves) {
             case 1: with_waves(IntTag<1>{}, IntTag<4>{}); break;  // 4 independent rows per block
             case 2: with_waves(IntTag<2>{}, IntTag<1>{}); break;
             case 4: with_waves(IntTag<4>{}, IntTag<1>{}); break;
@@ -156,11 +224,13 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
             return fail(FMSCAN_E_ALIAS, "fmscan_forward: out overlaps %s", in.name);
 
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(tokens) && aligned16(out);
-    const unsigned waves = choose_waves(pb);
-    dispatch(dtype, waves, pb.plain, vec, [&](auto tt, auto wt, auto rt, auto pt, auto vt) {
+    const Tuning tune = choose(pb);
+    const bool fold = M == 1 && D == 1;
+    dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;
-        launch_fwd<T, decltype(wt)::value, decltype(rt)::value, decltype(pt)::value,
-                   decltype(vt)::value>(pb, gates, tokens, initial_state, out, (hipStream_t)stream);
+        launch_fwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
+                   decltype(vt)::value, decltype(ft)::value>(pb, tune.blocks_per_cu, gates, tokens,
+                                                             initial_state, out, (hipStream_t)stream);
     });
     return launched("forward");
 }
@@ -198,13 +268,15 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
                      aligned16(token_grad_out) && aligned16(cached_output) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_out);
-    const unsigned waves = choose_waves(pb);
-    dispatch(dtype, waves, pb.plain, vec, [&](auto tt, auto wt, auto rt, auto pt, auto vt) {
+    const Tuning tune = choose(pb);
+    const bool fold = M == 1 && D == 1;
+    dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;
-        launch_bwd<T, decltype(wt)::value, decltype(rt)::value, decltype(pt)::value,
-                   decltype(vt)::value>(pb, gates, out_grad, first_prop_grad, token_grad_out,
-                                        cached_output, input_tokens, gate_grad_out, h_init,
-                                        (hipStream_t)stream);
+        launch_bwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
+                   decltype(vt)::value, decltype(ft)::value>(pb, tune.blocks_per_cu, gates, out_grad,
+                                                             first_prop_grad, token_grad_out, cached_output,
+                                                             input_tokens, gate_grad_out, h_init,
+                                                             (hipStream_t)stream);
     });
     return launched("backward");
 }

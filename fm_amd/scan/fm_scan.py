@@ -47,11 +47,13 @@ def _on_gpu(name: str, t: torch.Tensor, dev: torch.device) -> None:
     _require(t.device == dev, f"{name} is on {t.device}, expected {dev}")
 
 
-def _flags(plain: bool, waves_per_row: int) -> int:
-    return (_lib.FLAG_PLAIN if plain else 0) | (int(waves_per_row) << _lib.FLAG_WAVES_SHIFT)
+def _flags(plain: bool, waves_per_row: int, blocks_per_cu: int = 0, depth: int = 0) -> int:
+    return ((_lib.FLAG_PLAIN if plain else 0) | (int(waves_per_row) << _lib.FLAG_WAVES_SHIFT)
+            | (int(blocks_per_cu) << _lib.FLAG_BLOCKS_SHIFT) | (int(depth) << _lib.FLAG_DEPTH_SHIFT))
 
 
-def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per_row=0):
+def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per_row=0, blocks_per_cu=0,
+                    depth=0):
     """Writes the scan states into `out` (B, M, D, L) and returns `out`.
 
     gates (B, M, L), tokens (B, D, L), initial_state (B, M, D); everything
@@ -77,12 +79,13 @@ def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per
         stream = torch.cuda.current_stream(dev).cuda_stream
         _lib.check(module.fmscan_forward(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
                                          out.data_ptr(), B, M, D, L, code,
-                                         _flags(plain, waves_per_row), stream))
+                                         _flags(plain, waves_per_row, blocks_per_cu, depth), stream))
     return out
 
 
 def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output, input_tokens,
-                     gateGradOut, *, initial_state=None, plain=False, waves_per_row=0):
+                     gateGradOut, *, initial_state=None, plain=False, waves_per_row=0, blocks_per_cu=0,
+                     depth=0):
     """Reverse scan of `outGrad` (B, M, D, L); fills `tokenGradOut` and `gateGradOut`
     (both (B, M, D, L), one contribution per (m, d) pair) and returns None.
 
@@ -121,7 +124,7 @@ def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output,
             gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), tokenGradOut.data_ptr(),
             cached_output.data_ptr(), input_tokens.data_ptr(), gateGradOut.data_ptr(),
             None if initial_state is None else initial_state.data_ptr(),
-            B, M, D, L, code, _flags(plain, waves_per_row), stream))
+            B, M, D, L, code, _flags(plain, waves_per_row, blocks_per_cu, depth), stream))
     return None
 
 

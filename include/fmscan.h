@@ -48,6 +48,12 @@ extern "C" {
 #define FMSCAN_FLAG_WAVES_SHIFT  8    /* bits 8..11: waves cooperating on one row (1,2,4,8);
                                          0 = let the library choose */
 #define FMSCAN_FLAG_WAVES_MASK   0xF00u
+#define FMSCAN_FLAG_BLOCKS_SHIFT 12   /* bits 12..15: cap on the blocks a compute unit holds at a
+                                         time (1..15); 0 = let the library choose */
+#define FMSCAN_FLAG_BLOCKS_MASK  0xF000u
+#define FMSCAN_FLAG_DEPTH_SHIFT  16   /* bits 16..19: tiles whose loads a wave keeps in flight
+                                         ahead of the one it scans (2, 3 or 4); 0 = library's choice */
+#define FMSCAN_FLAG_DEPTH_MASK   0xF0000u
 
 /* error codes (negative returns) */
 #define FMSCAN_E_NULL      (-1) /* a required pointer is NULL */
