@@ -45,7 +45,10 @@ WORKLOADS = {
 # HBM bytes per backward launch read from rocprofv3 counters (FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the same counter reads for a copy of known
 # size); the runs are summarised under profiles/. None = not measured.
-MEASURED_BWD_TRAFFIC_BYTES = {}
+MEASURED_BWD_TRAFFIC_BYTES = {
+    # FETCH_SIZE 2097469.4 KiB x 2.0 (copy calibration) + WRITE_SIZE 2097154.2 KiB x 1.0
+    "cfg3": int((2097469.4 * 2.0 + 2097154.2) * 1024),
+}
 
 
 def make_inputs(torch, name, device):
