@@ -7,17 +7,18 @@ on a GPU are rejected.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_uint, c_void_p
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_uint, c_void_p
 
 from . import build as _build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 FLAG_PLAIN = 0x1
 FLAG_WAVES_SHIFT = 8
 FLAG_BLOCKS_SHIFT = 12
 FLAG_DEPTH_SHIFT = 16
+FLAG_SEGMENTS_SHIFT = 20
 
 _lib = None
 
@@ -35,12 +36,16 @@ def load() -> ctypes.CDLL:
     lib.fmscan_last_error.restype = c_char_p
     lib.fmscan_last_error.argtypes = []
     lib.fmscan_forward.restype = c_int
+    lib.fmscan_workspace_bytes.restype = c_size_t
+    lib.fmscan_workspace_bytes.argtypes = [c_int64, c_int64, c_int64, c_int64, c_int, c_uint]
     lib.fmscan_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p,
-                                   c_int64, c_int64, c_int64, c_int64, c_int, c_uint, c_void_p]
+                                   c_int64, c_int64, c_int64, c_int64, c_int, c_uint,
+                                   c_void_p, c_size_t, c_void_p]
     lib.fmscan_backward.restype = c_int
     lib.fmscan_backward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                    c_void_p, c_void_p,
-                                    c_int64, c_int64, c_int64, c_int64, c_int, c_uint, c_void_p]
+                                    c_void_p, c_void_p, c_void_p,
+                                    c_int64, c_int64, c_int64, c_int64, c_int, c_uint,
+                                    c_void_p, c_size_t, c_void_p]
     got = lib.fmscan_abi_version()
     if got != ABI_VERSION:
         raise RuntimeError(f"libfmscan_hip.so has ABI version {got}, this package needs {ABI_VERSION}; "

@@ -36,11 +36,15 @@ bool overlap(const Range& a, const Range& b) {
 struct Problem {
     int64_t B, M, D, L, rows;
     int esize;
-    unsigned waves;  // requested waves per row, 0 = auto
+    unsigned waves;          // requested waves per row, 0 = auto
     unsigned blocks_per_cu;  // requested cap on resident blocks per CU, 0 = auto
     unsigned depth;          // requested prefetch depth in tiles, 0 = auto
+    unsigned segments;       // requested segments per row, 0 = auto
     bool plain;
 };
+
+constexpr unsigned kKnownFlags = FMSCAN_FLAG_PLAIN | FMSCAN_FLAG_WAVES_MASK | FMSCAN_FLAG_BLOCKS_MASK |
+                                 FMSCAN_FLAG_DEPTH_MASK | FMSCAN_FLAG_SEGMENTS_MASK;
 
 int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, Problem* pb) {
     if (B < 1 || M < 1 || D < 1 || L < 1)
@@ -51,13 +55,15 @@ int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
     if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16)
         return fail(FMSCAN_E_DTYPE, "fmscan: dtype %d is not float32 (0), float16 (1) or bfloat16 (2)",
                     dtype);
-    if (flags & ~(FMSCAN_FLAG_PLAIN | FMSCAN_FLAG_WAVES_MASK | FMSCAN_FLAG_BLOCKS_MASK |
-                  FMSCAN_FLAG_DEPTH_MASK))
-        return fail(FMSCAN_E_FLAGS, "fmscan: unknown flag bits 0x%x", flags);
+    if (flags & ~kKnownFlags)
+        return fail(FMSCAN_E_FLAGS, "fmscan: unknown flag bits 0x%x", flags & ~kKnownFlags);
     const unsigned waves = (flags & FMSCAN_FLAG_WAVES_MASK) >> FMSCAN_FLAG_WAVES_SHIFT;
     if (waves != 0 && waves != 1 && waves != 2 && waves != 4 && waves != 8)
         return fail(FMSCAN_E_FLAGS, "fmscan: waves per row must be 0 (auto), 1, 2, 4 or 8 (got %u)",
                     waves);
+    const unsigned depth = (flags & FMSCAN_FLAG_DEPTH_MASK) >> FMSCAN_FLAG_DEPTH_SHIFT;
+    if (depth != 0 && (depth < 2 || depth > 4))
+        return fail(FMSCAN_E_FLAGS, "fmscan: prefetch depth must be 0 (auto), 2, 3 or 4 (got %u)", depth);
     // rows*L elements must be addressable and the grid must fit 31 bits
     const __int128 rows = (__int128)B * M * D;
     if (rows > (__int128)INT32_MAX || rows * L > ((__int128)1 << 46))
@@ -67,9 +73,8 @@ int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
     pb->esize = dtype == FMSCAN_DTYPE_F32 ? 4 : 2;
     pb->waves = waves;
     pb->blocks_per_cu = (flags & FMSCAN_FLAG_BLOCKS_MASK) >> FMSCAN_FLAG_BLOCKS_SHIFT;
-    pb->depth = (flags & FMSCAN_FLAG_DEPTH_MASK) >> FMSCAN_FLAG_DEPTH_SHIFT;
-    if (pb->depth != 0 && (pb->depth < 2 || pb->depth > 4))
-        return fail(FMSCAN_E_FLAGS, "fmscan: prefetch depth must be 0 (auto), 2, 3 or 4 (got %u)", pb->depth);
+    pb->depth = depth;
+    pb->segments = (flags & FMSCAN_FLAG_SEGMENTS_MASK) >> FMSCAN_FLAG_SEGMENTS_SHIFT;
     pb->plain = (flags & FMSCAN_FLAG_PLAIN) != 0;
     return 0;
 }
@@ -82,15 +87,16 @@ int launched(const char* what) {
     return 0;
 }
 
-// One block per R rows. Each block also asks for a share of the 160 KiB of LDS of a
-// compute unit that it never touches: at most `blocks_per_cu` blocks then fit a unit
-// at a time, which bounds the number of rows that stream concurrently.
+// One block per R slots (a slot is a row, or a segment of a row). Each block also asks
+// for a share of the 160 KiB of LDS of a compute unit that it never touches: at most
+// `blocks_per_cu` blocks then fit a unit at a time, which bounds the number of rows
+// that stream concurrently.
 struct Grid {
     unsigned blocks, lds;
 };
-Grid throttled_grid(const void* kern, int64_t rows, int R, unsigned blocks_per_cu) {
+Grid throttled_grid(const void* kern, int64_t slots, int R, unsigned blocks_per_cu) {
     Grid g;
-    g.blocks = (unsigned)((rows + R - 1) / R);
+    g.blocks = (unsigned)((slots + R - 1) / R);
     g.lds = ((160u * 1024u - 2048u) / blocks_per_cu) & ~1023u;
     static std::atomic<uint64_t> last_set{~0ull};  // (kernel, device, bytes) of the last attribute call
     int dev = 0;
@@ -107,68 +113,133 @@ Grid throttled_grid(const void* kern, int64_t rows, int R, unsigned blocks_per_c
     return g;
 }
 
-// Waves per row, resident blocks per compute unit and prefetch depth when the caller
-// leaves the choice to the library. The table comes from sweeps on an MI355X over the
-// benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536 in 16-bit types
-// and 8192 x 4096 in float32. What it encodes: a wave per row streams best when there are
-// many rows of moderate length; long rows want several waves side by side so that fewer
-// rows are open at a time; with few rows a block per row keeps every compute unit busy.
-// About two waves per SIMD is where HBM efficiency peaks; more resident rows lower it.
+// Waves per row, resident blocks per compute unit, prefetch depth and segments per row
+// when the caller leaves the choice to the library. The table comes from sweeps on an
+// MI355X over the benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536
+// in 16-bit types and 8192 x 4096 in float32. What it encodes: a wave per row streams
+// best when there are many rows of moderate length; long rows want several waves side
+// by side so that fewer rows are open at a time; with few rows a block per row keeps
+// every compute unit busy. About two waves per SIMD is where HBM efficiency peaks;
+// more resident rows lower it. With fewer rows than the chip has compute units, and a
+// workspace to hold the segment pairs, rows are cut into segments (two passes).
 struct Tuning {
     unsigned waves, blocks_per_cu, depth;
+    int32_t nseg;       // segments per row (1 = the row is scanned in one piece)
+    int64_t seg_tiles;  // tiles per segment
 };
-Tuning choose(const Problem& pb) {
+constexpr int64_t kSplitBelowRows = 256;    // rows below which cutting rows is considered
+constexpr int64_t kSplitTargetSlots = 2048;  // segments in flight the cut aims for
+constexpr int64_t kSplitMinTiles = 4;       // a segment is at least this many tiles
+constexpr int64_t kMaxSegments = 255;
+
+void plan_segments(const Problem& pb, Tuning& t, bool may_split) {
+    const int64_t tile1 = (16 / pb.esize) * 64;
+    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;
+    t.nseg = 1;
+    t.seg_tiles = tiles1;
+    if (!may_split) return;
+    int64_t want = pb.segments;
+    if (!want) {
+        if (pb.rows >= kSplitBelowRows || pb.waves) return;
+        want = (kSplitTargetSlots + pb.rows - 1) / pb.rows;
+        const int64_t most = tiles1 / kSplitMinTiles;
+        if (want > most) want = most;
+    }
+    if (want > tiles1) want = tiles1;
+    if (want > kMaxSegments) want = kMaxSegments;
+    if (want < 2) return;
+    const int64_t seg_tiles = (tiles1 + want - 1) / want;
+    const int64_t nseg = (tiles1 + seg_tiles - 1) / seg_tiles;
+    if (nseg < 2) return;
+    // a cut row is scanned by single waves: enough slots exist without sharing a row
+    t.waves = 1;
+    t.seg_tiles = seg_tiles;
+    t.nseg = (int32_t)nseg;
+}
+
+Tuning choose(const Problem& pb, bool may_split) {
     Tuning t;
-    const int64_t tile1 = (16 / pb.esize) * 64;               // elements one wave covers per tile
-    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;        // tiles per row for one wave
+    const int64_t tile1 = (16 / pb.esize) * 64;          // elements one wave covers per tile
+    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;   // tiles per row for one wave
     unsigned w = pb.waves;
     if (!w) {
         if (tiles1 >= 64) w = 4;
         else if (pb.rows < 16384 && tiles1 >= 8) w = 8;
         else w = 1;
-        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                                     // row shorter than a tile
-        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;           // very few rows
+        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
+        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
     }
     t.waves = w;
+    plan_segments(pb, t, may_split);
+    w = t.waves;
+    const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
     if (pb.blocks_per_cu) t.blocks_per_cu = pb.blocks_per_cu;
-    else if (w == 1) t.blocks_per_cu = tiles1 >= 16 ? 2 : 4;
+    else if (w == 1) t.blocks_per_cu = tiles_per_slot >= 16 ? 2 : 4;
     else if (w == 4) t.blocks_per_cu = 2;
     else t.blocks_per_cu = 4;
     if (pb.depth) t.depth = pb.depth;
-    else if (w == 1) t.depth = tiles1 >= 16 ? 3 : 4;
+    else if (w == 1) t.depth = tiles_per_slot >= 16 ? 3 : 4;
     else if (w == 4) t.depth = 4;
     else t.depth = 3;
     return t;
 }
 
-template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
-void launch_fwd(const Problem& pb, unsigned bpc, const void* g, const void* x, const void* h0, void* out,
-                hipStream_t s) {
-    auto kern = fmscan::scan_forward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
-    const Grid grid = throttled_grid((const void*)kern, pb.rows, R, bpc);
-    kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>(
-        (const T*)g, (const T*)x, (const T*)h0, (T*)out, pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L);
+size_t pairs_bytes(const Problem& pb, const Tuning& t) {
+    return t.nseg > 1 ? (size_t)pb.rows * (size_t)t.nseg * sizeof(float2) : 0;
+}
+
+// Settles the plan for one call: rows are cut only when the workspace can hold the pairs.
+// Returns 0, or FMSCAN_E_WORKSPACE when the caller asked for a cut that does not fit.
+int settle(const Problem& pb, const void* workspace, size_t workspace_bytes, const char* who, Tuning* t) {
+    *t = choose(pb, workspace != nullptr);
+    if (t->nseg > 1 && (pairs_bytes(pb, *t) > workspace_bytes || ((uintptr_t)workspace & 7u))) {
+        if (pb.segments > 1)
+            return fail(FMSCAN_E_WORKSPACE, "%s: %u segments per row need an 8-byte aligned workspace of "
+                        "%zu bytes (got %zu)", who, pb.segments, pairs_bytes(pb, *t), workspace_bytes);
+        *t = choose(pb, false);
+    } else if (pb.segments > 1 && !workspace) {
+        return fail(FMSCAN_E_WORKSPACE, "%s: %u segments per row need a workspace", who, pb.segments);
+    }
+    return 0;
 }
 
 template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
-void launch_bwd(const Problem& pb, unsigned bpc, const void* g, const void* G, const void* fpg, void* dx,
-                const void* h, const void* x, void* dg, const void* h0, hipStream_t s) {
+void launch_fwd(const Problem& pb, const Tuning& t, const void* g, const void* x, const void* h0,
+                void* out, const float2* pairs, hipStream_t s) {
+    auto kern = fmscan::scan_forward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
+    const Grid grid = throttled_grid((const void*)kern, pb.rows * t.nseg, R, t.blocks_per_cu);
+    kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>((const T*)g, (const T*)x, (const T*)h0, (T*)out,
+                                                   pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L,
+                                                   t.nseg, t.seg_tiles, pairs);
+}
+
+template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
+void launch_bwd(const Problem& pb, const Tuning& t, const void* g, const void* G, const void* fpg,
+                void* dx, const void* h, const void* x, void* dg, const void* h0, void* dh0,
+                const float2* pairs, hipStream_t s) {
     auto kern = fmscan::scan_backward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
-    const Grid grid = throttled_grid((const void*)kern, pb.rows, R, bpc);
+    const Grid grid = throttled_grid((const void*)kern, pb.rows * t.nseg, R, t.blocks_per_cu);
     kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>(
         (const T*)g, (const T*)G, (const T*)fpg, (T*)dx, (const T*)h, (const T*)x, (T*)dg,
-        (const T*)h0, pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L);
+        (const T*)h0, (T*)dh0, pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L, t.nseg, t.seg_tiles, pairs);
 }
 
 // Expands the run-time choices (dtype, waves per row, prefetch depth, plain, vector
-// access) into the kernel template arguments. F is a generic lambda called with tags.
+// access, fold) into the kernel template arguments. F is a generic lambda called with tags.
 template <typename T> struct TypeTag { using type = T; };
 template <int V> struct IntTag { static constexpr int value = V; };
 template <bool V> struct BoolTag { static constexpr bool value = V; };
 
 template <typename F>
+void with_dtype(int dtype, F&& f) {
+    if (dtype == FMSCAN_DTYPE_F32) f(TypeTag<float>{});
+    else if (dtype == FMSCAN_DTYPE_F16) f(TypeTag<_Float16>{});
+    else f(TypeTag<__bf16>{});
+}
+
+template <typename F>
 void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f) {
-    auto with_type = [&](auto tt) {
+    with_dtype(dtype, [&](auto tt) {
         auto with_waves = [&](auto wt, auto rt) {
             auto with_depth = [&](auto dt, auto vt, auto ft) {
                 if (plain) f(tt, wt, rt, dt, BoolTag<true>{}, vt, ft);
@@ -194,10 +265,32 @@ void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f
             case 4: with_waves(IntTag<4>{}, IntTag<1>{}); break;
             default: with_waves(IntTag<8>{}, IntTag<1>{}); break;
         }
-    };
-    if (dtype == FMSCAN_DTYPE_F32) with_type(TypeTag<float>{});
-    else if (dtype == FMSCAN_DTYPE_F16) with_type(TypeTag<_Float16>{});
-    else with_type(TypeTag<__bf16>{});
+    });
+}
+
+// Pass one of a segmented scan: one wave per segment, four segments per block.
+template <bool BACKWARD>
+void launch_aggregate(int dtype, const Problem& pb, const Tuning& t, bool vec, const void* g,
+                      const void* other, float2* pairs, hipStream_t s) {
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        auto go = [&](auto pt, auto vt) {
+            constexpr int R = 4, P = 3;
+            auto kern =
+                fmscan::scan_aggregate_kernel<T, R, P, decltype(pt)::value, decltype(vt)::value, BACKWARD>;
+            const unsigned blocks = (unsigned)((pb.rows * t.nseg + R - 1) / R);
+            kern<<<blocks, 64 * R, 0, s>>>((const T*)g, (const T*)other, pairs, pb.rows, (int32_t)pb.M,
+                                          (int32_t)pb.D, pb.L, t.nseg, t.seg_tiles);
+        };
+        const bool plain = pb.plain && !BACKWARD;  // the backward pairs are the same in both forms
+        if (plain) {
+            if (vec) go(BoolTag<true>{}, BoolTag<true>{});
+            else go(BoolTag<true>{}, BoolTag<false>{});
+        } else {
+            if (vec) go(BoolTag<false>{}, BoolTag<true>{});
+            else go(BoolTag<false>{}, BoolTag<false>{});
+        }
+    });
 }
 
 }  // namespace
@@ -208,9 +301,15 @@ int fmscan_abi_version(void) { return FMSCAN_ABI_VERSION; }
 
 const char* fmscan_last_error(void) { return g_err; }
 
+size_t fmscan_workspace_bytes(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags) {
+    Problem pb;
+    if (parse(B, M, D, L, dtype, flags, &pb)) return 0;
+    return pairs_bytes(pb, choose(pb, true));
+}
+
 int fmscan_forward(const void* gates, const void* tokens, const void* initial_state, void* out,
                    int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
-                   void* stream) {
+                   void* workspace, size_t workspace_bytes, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags, &pb)) return rc;
     if (!gates || !tokens || !out)
@@ -218,27 +317,35 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
     const Range o{"out", out, pb.rows * L * pb.esize};
     const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
                          {"tokens", tokens, B * D * L * pb.esize},
-                         {"initial_state", initial_state, pb.rows * pb.esize}};
+                         {"initial_state", initial_state, pb.rows * pb.esize},
+                         {"workspace", workspace, (int64_t)workspace_bytes}};
     for (const Range& in : ins)
         if (overlap(o, in))
             return fail(FMSCAN_E_ALIAS, "fmscan_forward: out overlaps %s", in.name);
 
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(tokens) && aligned16(out);
-    const Tuning tune = choose(pb);
+    Tuning tune;
+    if (int rc = settle(pb, workspace, workspace_bytes, "fmscan_forward", &tune)) return rc;
+    float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
+    if (pairs) {
+        launch_aggregate<false>(dtype, pb, tune, vec, gates, tokens, pairs, (hipStream_t)stream);
+        if (int rc = launched("forward (segment pass)")) return rc;
+    }
     const bool fold = M == 1 && D == 1;
     dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;
         launch_fwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
-                   decltype(vt)::value, decltype(ft)::value>(pb, tune.blocks_per_cu, gates, tokens,
-                                                             initial_state, out, (hipStream_t)stream);
+                   decltype(vt)::value, decltype(ft)::value>(pb, tune, gates, tokens, initial_state, out,
+                                                             pairs, (hipStream_t)stream);
     });
     return launched("forward");
 }
 
 int fmscan_backward(const void* gates, const void* out_grad, const void* first_prop_grad,
                     void* token_grad_out, const void* cached_output, const void* input_tokens,
-                    void* gate_grad_out, const void* initial_state, int64_t B, int64_t M, int64_t D,
-                    int64_t L, int dtype, unsigned flags, void* stream) {
+                    void* gate_grad_out, const void* initial_state, void* initial_state_grad,
+                    int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                    void* workspace, size_t workspace_bytes, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags, &pb)) return rc;
     if (!gates || !out_grad || !token_grad_out || !cached_output || !gate_grad_out)
@@ -248,7 +355,10 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
     if (!pb.plain && !input_tokens)
         return fail(FMSCAN_E_NULL, "fmscan_backward: input_tokens must not be NULL without FMSCAN_FLAG_PLAIN");
     const int64_t full = pb.rows * L * pb.esize;
-    const Range outs[] = {{"token_grad_out", token_grad_out, full}, {"gate_grad_out", gate_grad_out, full}};
+    const Range outs[] = {{"token_grad_out", token_grad_out, full},
+                          {"gate_grad_out", gate_grad_out, full},
+                          {"initial_state_grad", initial_state_grad, pb.rows * pb.esize},
+                          {"workspace", workspace, (int64_t)workspace_bytes}};
     const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
                          {"out_grad", out_grad, full},
                          {"first_prop_grad", first_prop_grad, pb.rows * pb.esize},
@@ -259,8 +369,10 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
         for (const Range& in : ins)
             if (overlap(o, in))
                 return fail(FMSCAN_E_ALIAS, "fmscan_backward: %s overlaps %s", o.name, in.name);
-    if (overlap(outs[0], outs[1]))
-        return fail(FMSCAN_E_ALIAS, "fmscan_backward: token_grad_out overlaps gate_grad_out");
+    for (int i = 0; i < 4; ++i)
+        for (int j = i + 1; j < 4; ++j)
+            if (overlap(outs[i], outs[j]))
+                return fail(FMSCAN_E_ALIAS, "fmscan_backward: %s overlaps %s", outs[i].name, outs[j].name);
 
     // NULL initial_state reproduces the reference kernel: h[-1] := first_prop_grad.
     const void* h_init = initial_state ? initial_state : first_prop_grad;
@@ -268,15 +380,21 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
                      aligned16(token_grad_out) && aligned16(cached_output) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_out);
-    const Tuning tune = choose(pb);
+    Tuning tune;
+    if (int rc = settle(pb, workspace, workspace_bytes, "fmscan_backward", &tune)) return rc;
+    float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
+    if (pairs) {
+        launch_aggregate<true>(dtype, pb, tune, vec, gates, out_grad, pairs, (hipStream_t)stream);
+        if (int rc = launched("backward (segment pass)")) return rc;
+    }
     const bool fold = M == 1 && D == 1;
     dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;
         launch_bwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
-                   decltype(vt)::value, decltype(ft)::value>(pb, tune.blocks_per_cu, gates, out_grad,
-                                                             first_prop_grad, token_grad_out, cached_output,
-                                                             input_tokens, gate_grad_out, h_init,
-                                                             (hipStream_t)stream);
+                   decltype(vt)::value, decltype(ft)::value>(pb, tune, gates, out_grad, first_prop_grad,
+                                                             token_grad_out, cached_output, input_tokens,
+                                                             gate_grad_out, h_init, initial_state_grad,
+                                                             pairs, (hipStream_t)stream);
     });
     return launched("backward");
 }

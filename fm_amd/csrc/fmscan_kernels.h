@@ -14,6 +14,12 @@
 // current one. The grid has one block per row (W > 1) or per R rows (W == 1); the
 // host bounds how many blocks a compute unit holds at a time, because the HBM
 // efficiency of this access pattern depends on how many rows stream concurrently.
+//
+// Few rows, long sequences: a row can be cut into `nseg` segments of `seg_tiles` tiles
+// that are scanned as if they were rows of their own (two passes). Pass one
+// (scan_aggregate_kernel) reduces every segment to its step pair (A, B); pass two is
+// the ordinary scan kernel, whose block first folds the pairs of the segments that
+// precede its own into the state that enters it.
 #pragma once
 
 #include "fmscan_device.h"
@@ -35,6 +41,22 @@ __device__ __forceinline__ RowMap map_row(int64_t row, int32_t M, int32_t D) {
     m.gate_row = gate_row;
     m.token_row = (int64_t)b * D + (r - gate_row * (uint32_t)D);
     return m;
+}
+
+// Which part of which row a slot of the grid works on. With nseg == 1 a slot is a row.
+struct Segment {
+    int64_t row;
+    int32_t index;        // segment inside the row
+    int64_t k_lo, k_hi;   // its tiles: [k_lo, k_hi)
+};
+__device__ __forceinline__ Segment locate_segment(int64_t slot, int32_t nseg, int64_t seg_tiles,
+                                                  int64_t ntiles) {
+    Segment s;
+    s.row = nseg > 1 ? slot / nseg : slot;
+    s.index = nseg > 1 ? (int32_t)(slot - s.row * nseg) : 0;
+    s.k_lo = (int64_t)s.index * seg_tiles;
+    s.k_hi = s.k_lo + seg_tiles < ntiles ? s.k_lo + seg_tiles : ntiles;
+    return s;
 }
 
 // Meets the W wave totals of one tile in LDS. `cin` leaves as the state that
@@ -65,15 +87,19 @@ __device__ __forceinline__ void combine_waves(float2 (*slots)[W], int parity, in
 template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
 __global__ __launch_bounds__(64 * W * R) void scan_forward_kernel(
     const T* __restrict__ gates, const T* __restrict__ tokens, const T* __restrict__ h0,
-    T* __restrict__ out, int64_t rows, int32_t M, int32_t D, int64_t L) {
+    T* __restrict__ out, int64_t rows, int32_t M, int32_t D, int64_t L, int32_t nseg,
+    int64_t seg_tiles, const float2* __restrict__ seg_pairs) {
     static_assert(W == 1 || R == 1, "waves that share a barrier must share a row");
     constexpr int E = Elem<T>::E;
     constexpr int64_t TILE = (int64_t)E * 64 * W;
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int w = wave % W;
-    const int64_t r = (int64_t)blockIdx.x * R + wave / W;
-    if (r >= rows) return;  // whole waves only, and only in barrier-free (W == 1) blocks
+    const int64_t slot = (int64_t)blockIdx.x * R + wave / W;
+    if (slot >= rows * nseg) return;  // whole waves only, and only in barrier-free (W == 1) blocks
+    const int64_t ntiles = (L + TILE - 1) / TILE;
+    const Segment seg = locate_segment(slot, nseg, seg_tiles, ntiles);
+    const int64_t r = seg.row;
 
     __shared__ float2 slots[2][W];
 
@@ -82,28 +108,32 @@ __global__ __launch_bounds__(64 * W * R) void scan_forward_kernel(
     const T* __restrict__ xrow = tokens + rm.token_row * L;
     T* __restrict__ orow = out + r * L;
     float carry = h0 ? Elem<T>::widen(h0[r]) : 0.0f;
+    for (int32_t j = 0; j < seg.index; ++j) {  // the segments before this one, oldest first
+        const float2 p = seg_pairs[r * nseg + j];
+        carry = __builtin_fmaf(p.x, carry, p.y);
+    }
 
     const int64_t lane_off = (int64_t)(w * 64 + lane) * E;
-    const int64_t ntiles = (L + TILE - 1) / TILE;
 
     struct Entry {
         u32x4 g, x;
     };
-    auto fetch = [&](Entry& q, int64_t k) {  // k >= ntiles loads nothing
-        const int64_t t0 = k * TILE + lane_off;
+    auto fetch = [&](Entry& q, int64_t k) {
+        // k >= k_hi (past the segment): t0 = L, which every bound check rejects
+        const int64_t t0 = k < seg.k_hi ? k * TILE + lane_off : L;
         q.g = load_chunk<T, VEC, FOLD>(grow, t0, L, Elem<T>::kOnes);
         q.x = load_chunk<T, VEC, FOLD>(xrow, t0, L, 0u);
     };
 
     Entry q[P];
 #pragma unroll
-    for (int s = 0; s < P; ++s) fetch(q[s], s);
+    for (int s = 0; s < P; ++s) fetch(q[s], seg.k_lo + s);
 
-    for (int64_t k0 = 0; k0 < ntiles; k0 += P) {
+    for (int64_t k0 = seg.k_lo; k0 < seg.k_hi; k0 += P) {
 #pragma unroll
         for (int s = 0; s < P; ++s) {
             const int64_t k = k0 + s;
-            if (k >= ntiles) break;
+            if (k >= seg.k_hi) break;
             const Entry cur = q[s];
             fetch(q[s], k + P);
             const int64_t t0 = k * TILE + lane_off;
@@ -160,16 +190,20 @@ template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
 __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad, const T* __restrict__ h_saved, const T* __restrict__ tokens,
-    T* __restrict__ gate_grad, const T* __restrict__ h0, int64_t rows, int32_t M, int32_t D,
-    int64_t L) {
+    T* __restrict__ gate_grad, const T* __restrict__ h0, T* __restrict__ h0_grad, int64_t rows,
+    int32_t M, int32_t D, int64_t L, int32_t nseg, int64_t seg_tiles,
+    const float2* __restrict__ seg_pairs) {
     static_assert(W == 1 || R == 1, "waves that share a barrier must share a row");
     constexpr int E = Elem<T>::E;
     constexpr int64_t TILE = (int64_t)E * 64 * W;
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int w = wave % W;
-    const int64_t r = (int64_t)blockIdx.x * R + wave / W;
-    if (r >= rows) return;
+    const int64_t slot = (int64_t)blockIdx.x * R + wave / W;
+    if (slot >= rows * nseg) return;
+    const int64_t ntiles = (L + TILE - 1) / TILE;
+    const Segment seg = locate_segment(slot, nseg, seg_tiles, ntiles);
+    const int64_t r = seg.row;
 
     __shared__ float2 slots[2][W];
 
@@ -181,18 +215,21 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
     T* __restrict__ dxrow = token_grad + r * L;
     T* __restrict__ dgrow = gate_grad + r * L;
     float carry = first_prop_grad ? Elem<T>::widen(first_prop_grad[r]) : 0.0f;
+    for (int32_t j = nseg - 1; j > seg.index; --j) {  // the segments after this one, last first
+        const float2 p = seg_pairs[r * nseg + j];
+        carry = __builtin_fmaf(p.x, carry, p.y);
+    }
     const float hinit = h0 ? Elem<T>::widen(h0[r]) : 0.0f;
 
     const int64_t lane_off = (int64_t)(64 * W - 1 - (w * 64 + lane)) * E;
-    const int64_t ntiles = (L + TILE - 1) / TILE;
 
     struct Entry {
         u32x4 g, G, h, x;
         float hb;  // lane 63 only: h just before this wave's part of the tile (h[-1] at t = 0)
     };
     auto fetch = [&](Entry& q, int64_t k) {
-        // k < 0 (before the row): t0 = L, which every bound check below rejects
-        const int64_t t0 = k >= 0 ? k * TILE + lane_off : L;
+        // k < k_lo (before the segment): t0 = L, which every bound check below rejects
+        const int64_t t0 = k >= seg.k_lo ? k * TILE + lane_off : L;
         q.g = load_chunk<T, VEC, FOLD>(grow, t0, L, Elem<T>::kOnes);
         q.G = load_chunk<T, VEC, true>(Grow, t0, L, 0u);
         q.h = load_chunk<T, VEC, true>(hrow, t0, L, 0u);
@@ -203,13 +240,13 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
 
     Entry q[P];
 #pragma unroll
-    for (int s = 0; s < P; ++s) fetch(q[s], ntiles - 1 - s);
+    for (int s = 0; s < P; ++s) fetch(q[s], seg.k_hi - 1 - s);
 
-    for (int64_t k0 = ntiles - 1; k0 >= 0; k0 -= P) {
+    for (int64_t k0 = seg.k_hi - 1; k0 >= seg.k_lo; k0 -= P) {
 #pragma unroll
         for (int s = 0; s < P; ++s) {
             const int64_t k = k0 - s;
-            if (k < 0) break;
+            if (k < seg.k_lo) break;
             const Entry cur = q[s];
             fetch(q[s], k - P);
             const int64_t t0 = k * TILE + lane_off;
@@ -263,6 +300,99 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
             store_chunk<T, VEC>(dgrow, t0, L, Elem<T>::pack(dg));
         }
     }
+    // what is left after the first step is g_0 * delta_0: the gradient of the state before the row
+    if (h0_grad && seg.index == 0 && w == 0 && lane == 0) {
+        float v[E] = {carry};
+        const u32x4 packed = Elem<T>::pack(v);
+        if constexpr (sizeof(T) == 4) reinterpret_cast<uint32_t*>(h0_grad)[r] = packed.x;
+        else reinterpret_cast<uint16_t*>(h0_grad)[r] = (uint16_t)(packed.x & 0xffffu);
+    }
+}
+
+// ---- pass one of a segmented scan ------------------------------------------------------
+// Reduces every segment to its step pair. Forward: pairs (g_t, u_t) composed left to
+// right, so that state_after = A * state_before + B. Backward: pairs (g_t, g_t G_t)
+// composed right to left (the carried quantity is c_t, see scan_backward_kernel).
+// One wave per segment, no LDS. The last segment of a row (forward) / the first
+// (backward) is never needed and is skipped.
+template <typename T, int R, int P, bool PLAIN, bool VEC, bool BACKWARD>
+__global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
+    const T* __restrict__ gates, const T* __restrict__ other /* tokens | out_grad */,
+    float2* __restrict__ seg_pairs, int64_t rows, int32_t M, int32_t D, int64_t L, int32_t nseg,
+    int64_t seg_tiles) {
+    constexpr int E = Elem<T>::E;
+    constexpr int64_t TILE = (int64_t)E * 64;
+    const int lane = threadIdx.x & 63;
+    const int wave = uniform(threadIdx.x >> 6);
+    const int64_t slot = (int64_t)blockIdx.x * R + wave;
+    if (slot >= rows * nseg) return;
+    const int64_t ntiles = (L + TILE - 1) / TILE;
+    const Segment seg = locate_segment(slot, nseg, seg_tiles, ntiles);
+    if (seg.index == (BACKWARD ? 0 : nseg - 1)) return;
+    const int64_t r = seg.row;
+
+    const RowMap rm = map_row(r, M, D);
+    const T* __restrict__ grow = gates + rm.gate_row * L;
+    const T* __restrict__ orow = other + (BACKWARD ? r : rm.token_row) * L;
+    const int64_t lane_off = (int64_t)(BACKWARD ? 63 - lane : lane) * E;
+
+    struct Entry {
+        u32x4 g, o;
+    };
+    auto fetch = [&](Entry& q, int64_t k) {
+        const int64_t t0 = (k >= seg.k_lo && k < seg.k_hi) ? k * TILE + lane_off : L;
+        q.g = load_chunk<T, VEC, false>(grow, t0, L, Elem<T>::kOnes);
+        q.o = load_chunk<T, VEC, false>(orow, t0, L, 0u);
+    };
+    const int64_t first = BACKWARD ? seg.k_hi - 1 : seg.k_lo;
+    constexpr int64_t step = BACKWARD ? -1 : 1;
+
+    Entry q[P];
+#pragma unroll
+    for (int s = 0; s < P; ++s) fetch(q[s], first + step * s);
+
+    float A = 1.0f, B = 0.0f;
+    const int64_t count = seg.k_hi - seg.k_lo;
+    for (int64_t n0 = 0; n0 < count; n0 += P) {
+#pragma unroll
+        for (int s = 0; s < P; ++s) {
+            const int64_t n = n0 + s;
+            if (n >= count) break;
+            const Entry cur = q[s];
+            fetch(q[s], first + step * (n + P));
+            float g[E], v[E];
+            Elem<T>::unpack(cur.g, g);
+            Elem<T>::unpack(cur.o, v);
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+                if constexpr (BACKWARD) v[i] = g[i] * v[i];
+                else if constexpr (!PLAIN) v[i] = __builtin_fmaf(-g[i], v[i], v[i]);
+            }
+            float a, b;
+            if constexpr (BACKWARD) {
+                a = g[E - 1];
+                b = v[E - 1];
+#pragma unroll
+                for (int i = E - 2; i >= 0; --i) {
+                    b = __builtin_fmaf(g[i], b, v[i]);
+                    a *= g[i];
+                }
+            } else {
+                a = g[0];
+                b = v[0];
+#pragma unroll
+                for (int i = 1; i < E; ++i) {
+                    b = __builtin_fmaf(g[i], b, v[i]);
+                    a *= g[i];
+                }
+            }
+            wave_scan_inclusive(a, b);
+            const float ta = lane63(a), tb = lane63(b);
+            B = __builtin_fmaf(ta, B, tb);  // segment so far, then this tile
+            A *= ta;
+        }
+    }
+    if (lane == 0) seg_pairs[r * nseg + seg.index] = make_float2(A, B);
 }
 
 }  // namespace fmscan

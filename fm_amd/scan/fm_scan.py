@@ -47,13 +47,23 @@ def _on_gpu(name: str, t: torch.Tensor, dev: torch.device) -> None:
     _require(t.device == dev, f"{name} is on {t.device}, expected {dev}")
 
 
-def _flags(plain: bool, waves_per_row: int, blocks_per_cu: int = 0, depth: int = 0) -> int:
+def _flags(plain: bool, waves_per_row: int, blocks_per_cu: int, depth: int, segments: int) -> int:
     return ((_lib.FLAG_PLAIN if plain else 0) | (int(waves_per_row) << _lib.FLAG_WAVES_SHIFT)
-            | (int(blocks_per_cu) << _lib.FLAG_BLOCKS_SHIFT) | (int(depth) << _lib.FLAG_DEPTH_SHIFT))
+            | (int(blocks_per_cu) << _lib.FLAG_BLOCKS_SHIFT) | (int(depth) << _lib.FLAG_DEPTH_SHIFT)
+            | (int(segments) << _lib.FLAG_SEGMENTS_SHIFT))
+
+
+def _workspace(B, M, D, L, code, flags, device):
+    """Scratch for the carries between the segments of a cut row (few rows, long L);
+    None when the library scans every row in one piece."""
+    need = module.fmscan_workspace_bytes(B, M, D, L, code, flags)
+    if not need:
+        return None, 0
+    return torch.empty(need, dtype=torch.uint8, device=device), need
 
 
 def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per_row=0, blocks_per_cu=0,
-                    depth=0):
+                    depth=0, segments=0):
     """Writes the scan states into `out` (B, M, D, L) and returns `out`.
 
     gates (B, M, L), tokens (B, D, L), initial_state (B, M, D); everything
@@ -75,24 +85,27 @@ def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per
     code = _dtype_code(gates)
     if out.numel() == 0:
         return out
+    flags = _flags(plain, waves_per_row, blocks_per_cu, depth, segments)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
+        ws, ws_bytes = _workspace(B, M, D, L, code, flags, dev)
         _lib.check(module.fmscan_forward(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
-                                         out.data_ptr(), B, M, D, L, code,
-                                         _flags(plain, waves_per_row, blocks_per_cu, depth), stream))
+                                         out.data_ptr(), B, M, D, L, code, flags,
+                                         None if ws is None else ws.data_ptr(), ws_bytes, stream))
     return out
 
 
 def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output, input_tokens,
-                     gateGradOut, *, initial_state=None, plain=False, waves_per_row=0, blocks_per_cu=0,
-                     depth=0):
+                     gateGradOut, *, initial_state=None, initial_state_grad=None, plain=False,
+                     waves_per_row=0, blocks_per_cu=0, depth=0, segments=0):
     """Reverse scan of `outGrad` (B, M, D, L); fills `tokenGradOut` and `gateGradOut`
     (both (B, M, D, L), one contribution per (m, d) pair) and returns None.
 
     With the seven positional arguments alone this computes what the reference
     extension computes, including its use of `firstPropGrad` as the state before
     the first step in the gate gradient (fm_scan.cuh:196,380). `initial_state`
-    (B, M, D), when given, is used there instead.
+    (B, M, D), when given, is used there instead; `initial_state_grad` (B, M, D), when
+    given, receives the gradient with respect to the initial state.
     """
     dev = gates.device
     named = [("gates", gates), ("outGrad", outGrad), ("firstPropGrad", firstPropGrad),
@@ -100,6 +113,8 @@ def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output,
              ("input_tokens", input_tokens), ("gateGradOut", gateGradOut)]
     if initial_state is not None:
         named.append(("initial_state", initial_state))
+    if initial_state_grad is not None:
+        named.append(("initial_state_grad", initial_state_grad))
     for name, t in named:
         _on_gpu(name, t, dev)
         _require(t.is_contiguous(), f"{name} must be contiguous")
@@ -113,18 +128,22 @@ def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output,
     for name, t in (("outGrad", outGrad), ("tokenGradOut", tokenGradOut), ("gateGradOut", gateGradOut)):
         _require(tuple(t.shape) == full, f"{name} must be {full}, got {tuple(t.shape)}")
     _require(firstPropGrad.numel() == B * M * D, f"firstPropGrad must hold {B * M * D} elements")
-    if initial_state is not None:
-        _require(initial_state.numel() == B * M * D, f"initial_state must hold {B * M * D} elements")
+    for name, t in (("initial_state", initial_state), ("initial_state_grad", initial_state_grad)):
+        if t is not None:
+            _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
     code = _dtype_code(gates)
     if cached_output.numel() == 0:
         return None
+    flags = _flags(plain, waves_per_row, blocks_per_cu, depth, segments)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
+        ws, ws_bytes = _workspace(B, M, D, L, code, flags, dev)
         _lib.check(module.fmscan_backward(
             gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), tokenGradOut.data_ptr(),
             cached_output.data_ptr(), input_tokens.data_ptr(), gateGradOut.data_ptr(),
             None if initial_state is None else initial_state.data_ptr(),
-            B, M, D, L, code, _flags(plain, waves_per_row, blocks_per_cu, depth), stream))
+            None if initial_state_grad is None else initial_state_grad.data_ptr(),
+            B, M, D, L, code, flags, None if ws is None else ws.data_ptr(), ws_bytes, stream))
     return None
 
 
@@ -132,8 +151,8 @@ class FM_Scan(torch.autograd.Function):
     """states = FM_Scan.apply(gates, tokens, initial_state=None)
 
     gates (B, M, L), tokens (B, D, L) -> states (B, M, D, L) in gates.dtype;
-    backward returns (d_gates (B, M, L), d_tokens (B, D, L), None)
-    (reference fm_scan.py:37-81).
+    backward returns (d_gates (B, M, L), d_tokens (B, D, L), d_initial_state or None)
+    (reference fm_scan.py:37-81, which always returns None in third place).
     """
 
     @staticmethod
@@ -172,14 +191,18 @@ class FM_Scan(torch.autograd.Function):
         grad_output = grad_output.contiguous()
         per_pair_gates = torch.empty_like(states)   # (B, M, D, L)
         per_pair_tokens = torch.empty_like(states)  # (B, M, D, L)
+        # The reference leaves the initial state's gradient unconnected (fm_scan.py:80-81); it
+        # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
+        d_initial_state = torch.empty_like(first_prop_grad) if ctx.needs_input_grad[2] else None
         fm_scan_backward(gates, grad_output, first_prop_grad, per_pair_tokens, states, tokens,
-                         per_pair_gates, initial_state=initial_state)
+                         per_pair_gates, initial_state=initial_state,
+                         initial_state_grad=d_initial_state)
 
         # (B, M, D, L) -> (B, M, L) and (B, D, L); a sum over an axis of length one
         # is the same tensor, so it is returned as a view without another pass
         d_gates = per_pair_gates.view(B, M, L) if D == 1 else per_pair_gates.sum(dim=2)
         d_tokens = per_pair_tokens.view(B, D, L) if M == 1 else per_pair_tokens.sum(dim=1)
-        return d_gates, d_tokens, None
+        return d_gates, d_tokens, d_initial_state
 
 
 def fm_scan(gates, tokens, initial_state=None):

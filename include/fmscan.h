@@ -11,8 +11,17 @@
  * Every pointer is a device pointer on the GPU that is current when the call
  * is made; all tensors are dense, row-major, sequence (L) innermost. The
  * library owns no memory and keeps no state between calls: the caller
- * allocates inputs and outputs, the calls enqueue kernels on `stream`
- * (a hipStream_t, NULL = the default stream) and return without waiting.
+ * allocates inputs, outputs and the optional workspace, the calls enqueue
+ * kernels on `stream` (a hipStream_t, NULL = the default stream) and return
+ * without waiting.
+ *
+ * Workspace. With fewer rows (B*M*D) than the GPU has compute units a row is
+ * cut into segments that are scanned side by side; the carry between segments
+ * goes through `workspace` (two floats per segment, written by a first pass).
+ * fmscan_workspace_bytes() tells how much a call can use; a NULL or smaller
+ * workspace makes the call scan every row in one piece (same results up to
+ * rounding, fewer compute units busy). Calls that run concurrently need
+ * separate workspaces.
  *
  * These entry points stand where the reference's two extension functions
  * stand (reference fm/scan/fm_scan.cuh:344-358 `fm_scan_forward`, :361-381
@@ -34,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FMSCAN_ABI_VERSION 1
+#define FMSCAN_ABI_VERSION 2
 
 /* element type of every tensor in one call (reference fm_scan.cuh:333-342) */
 #define FMSCAN_DTYPE_F32  0
@@ -54,6 +63,9 @@ extern "C" {
 #define FMSCAN_FLAG_DEPTH_SHIFT  16   /* bits 16..19: tiles whose loads a wave keeps in flight
                                          ahead of the one it scans (2, 3 or 4); 0 = library's choice */
 #define FMSCAN_FLAG_DEPTH_MASK   0xF0000u
+#define FMSCAN_FLAG_SEGMENTS_SHIFT 20 /* bits 20..27: segments a row is cut into (2..255, needs the
+                                         workspace); 1 = never cut; 0 = library's choice */
+#define FMSCAN_FLAG_SEGMENTS_MASK 0xFF00000u
 
 /* error codes (negative returns) */
 #define FMSCAN_E_NULL      (-1) /* a required pointer is NULL */
@@ -61,6 +73,7 @@ extern "C" {
 #define FMSCAN_E_DTYPE     (-3) /* dtype is not one of FMSCAN_DTYPE_* */
 #define FMSCAN_E_FLAGS     (-4) /* unknown flag bit or unsupported waves-per-row value */
 #define FMSCAN_E_ALIAS     (-5) /* an output overlaps an input it must not overlap */
+#define FMSCAN_E_WORKSPACE (-6) /* segments were requested and the workspace is missing or small */
 
 /* Version of this interface; equals FMSCAN_ABI_VERSION of the header the
  * library was built from. No counterpart in the reference (its extension is
@@ -71,6 +84,11 @@ int fmscan_abi_version(void);
  * Replaces the c10::Error text of the reference's TORCH_CHECKs
  * (fm/scan/fm_scan.cuh:329,341,346-354,367-378). */
 const char* fmscan_last_error(void);
+
+/* Bytes of workspace fmscan_forward / fmscan_backward can use for this problem (0 when
+ * rows are never cut). No counterpart in the reference, whose kernel gives one block a
+ * whole row (fm/scan/fm_scan.cuh:62-64,84). */
+size_t fmscan_workspace_bytes(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags);
 
 /*
  * Forward scan. Replaces fm_scan_forward (reference fm/scan/fm_scan.cuh:344-358)
@@ -87,7 +105,8 @@ const char* fmscan_last_error(void);
 int fmscan_forward(const void* gates, const void* tokens, const void* initial_state,
                    void* out,
                    int64_t B, int64_t M, int64_t D, int64_t L,
-                   int dtype, unsigned flags, void* stream);
+                   int dtype, unsigned flags,
+                   void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Backward scan. Replaces fm_scan_backward (reference fm/scan/fm_scan.cuh:361-381)
@@ -107,15 +126,20 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
  *                    (:196 with :380), i.e. h[-1] := first_prop_grad (zeros if that
  *                    is NULL too). Pass the forward call's initial_state to get the
  *                    mathematically exact gate gradient at t = 0.
- * The two outputs must not overlap any input or each other.
+ *   initial_state_grad (B, M, D)   out, may be NULL: dL/d initial_state = g[0] * delta[0].
+ *                    The reference leaves this gradient unconnected
+ *                    (fm/scan/fm_scan.py:80-81); its per-timestep PyTorch path
+ *                    (fm/scan/fm_pytorch.py) yields it through autograd.
+ * Outputs must not overlap any input or each other.
  */
 int fmscan_backward(const void* gates, const void* out_grad, const void* first_prop_grad,
                     void* token_grad_out,
                     const void* cached_output, const void* input_tokens,
                     void* gate_grad_out,
-                    const void* initial_state,
+                    const void* initial_state, void* initial_state_grad,
                     int64_t B, int64_t M, int64_t D, int64_t L,
-                    int dtype, unsigned flags, void* stream);
+                    int dtype, unsigned flags,
+                    void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

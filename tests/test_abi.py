@@ -24,7 +24,7 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_forward",
-                                    "fmscan_last_error"]
+                                    "fmscan_last_error", "fmscan_workspace_bytes"]
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -48,24 +48,28 @@ def test_python_constants_match_header():
     assert _lib.DTYPE_F16 == _const("FMSCAN_DTYPE_F16")
     assert _lib.DTYPE_BF16 == _const("FMSCAN_DTYPE_BF16")
     assert _lib.FLAG_WAVES_SHIFT == _const("FMSCAN_FLAG_WAVES_SHIFT")
+    assert _lib.FLAG_BLOCKS_SHIFT == _const("FMSCAN_FLAG_BLOCKS_SHIFT")
+    assert _lib.FLAG_DEPTH_SHIFT == _const("FMSCAN_FLAG_DEPTH_SHIFT")
+    assert _lib.FLAG_SEGMENTS_SHIFT == _const("FMSCAN_FLAG_SEGMENTS_SHIFT")
+    assert _lib.ABI_VERSION == _const("FMSCAN_ABI_VERSION")
     assert _lib.FLAG_PLAIN == int(re.search(r"FMSCAN_FLAG_PLAIN\s+(0x[0-9a-f]+)u", HEADER).group(1), 16)
 
 
-P = 0x10000  # never dereferenced: every call below is rejected by the argument checks
+P = 1 << 32  # never dereferenced: every call below is rejected by the argument checks
 
 
-def fwd(lib, g=P, x=2 * P, h0=None, out=3 * P, B=1, M=1, D=1, L=8, dtype=0, flags=0):
-    return lib.fmscan_forward(g, x, h0, out, B, M, D, L, dtype, flags, None)
+def fwd(lib, g=P, x=2 * P, h0=None, out=3 * P, B=1, M=1, D=1, L=8, dtype=0, flags=0, ws=None, ws_bytes=0):
+    return lib.fmscan_forward(g, x, h0, out, B, M, D, L, dtype, flags, ws, ws_bytes, None)
 
 
-def bwd(lib, g=P, G=2 * P, fpg=None, dx=3 * P, h=4 * P, x=5 * P, dg=6 * P, h0=None, B=1, M=1, D=1, L=8,
-        dtype=0, flags=0):
-    return lib.fmscan_backward(g, G, fpg, dx, h, x, dg, h0, B, M, D, L, dtype, flags, None)
+def bwd(lib, g=P, G=2 * P, fpg=None, dx=3 * P, h=4 * P, x=5 * P, dg=6 * P, h0=None, dh0=None, B=1, M=1,
+        D=1, L=8, dtype=0, flags=0, ws=None, ws_bytes=0):
+    return lib.fmscan_backward(g, G, fpg, dx, h, x, dg, h0, dh0, B, M, D, L, dtype, flags, ws, ws_bytes, None)
 
 
 def test_rejected_arguments(lib):
-    E_NULL, E_SHAPE, E_DTYPE, E_FLAGS, E_ALIAS = (_const("FMSCAN_E_" + n) for n in
-                                                  ("NULL", "SHAPE", "DTYPE", "FLAGS", "ALIAS"))
+    E_NULL, E_SHAPE, E_DTYPE, E_FLAGS, E_ALIAS, E_WORKSPACE = (
+        _const("FMSCAN_E_" + n) for n in ("NULL", "SHAPE", "DTYPE", "FLAGS", "ALIAS", "WORKSPACE"))
     assert fwd(lib, g=None) == E_NULL
     assert b"NULL" in lib.fmscan_last_error()
     assert fwd(lib, out=None) == E_NULL
@@ -76,6 +80,13 @@ def test_rejected_arguments(lib):
     assert b"dtype" in lib.fmscan_last_error()
     assert fwd(lib, flags=0x2) == E_FLAGS
     assert fwd(lib, flags=3 << 8) == E_FLAGS          # 3 waves per row is not offered
+    assert fwd(lib, flags=5 << 16) == E_FLAGS         # prefetch depth 5 is not offered
+    assert fwd(lib, flags=1 << 28) == E_FLAGS         # unknown bit
+    assert fwd(lib, L=1 << 16, flags=4 << 20) == E_WORKSPACE   # 4 segments asked for, no workspace
+    assert b"workspace" in lib.fmscan_last_error()
+    assert fwd(lib, L=1 << 16, flags=4 << 20, ws=7 * P, ws_bytes=8) == E_WORKSPACE  # too small
+    assert bwd(lib, L=1 << 16, flags=4 << 20) == E_WORKSPACE
+    assert bwd(lib, dh0=4 * P) == E_ALIAS             # initial_state_grad on top of cached_output
     assert fwd(lib, out=P) == E_ALIAS                 # out on top of gates
     assert fwd(lib, out=2 * P + 16) == E_ALIAS        # out inside tokens
     assert bwd(lib, h=None) == E_NULL
@@ -85,3 +96,16 @@ def test_rejected_arguments(lib):
     assert bwd(lib, dx=4 * P) == E_ALIAS              # token_grad_out on top of cached_output
     assert bwd(lib, dg=3 * P) == E_ALIAS              # the two outputs on top of each other
     assert b"overlaps" in lib.fmscan_last_error()
+
+
+def test_workspace_bytes(lib):
+    """Two floats per segment, only for problems with fewer rows than compute units (or on request)."""
+    wb = lib.fmscan_workspace_bytes
+    assert wb(16 * 2048, 1, 1, 16384, 2, 0) == 0          # many rows: never cut
+    assert wb(4, 1, 1, 65536, 2, 0) == 4 * 32 * 8           # 4 rows of 128 tiles -> 32 segments of 4 tiles
+    assert wb(4, 1, 1, 65536, 2, 1 << 20) == 0              # segments = 1: never cut
+    assert wb(4, 1, 1, 65536, 2, 8 << 20) == 4 * 8 * 8      # 8 segments on request
+    assert wb(1000, 1, 1, 65536, 2, 2 << 20) == 1000 * 2 * 8
+    assert wb(4, 1, 1, 512, 2, 0) == 0                      # one tile per row: nothing to cut
+    assert wb(4, 1, 1, 65536, 2, 4 << 8) == 0               # caller fixed the waves per row
+    assert wb(0, 1, 1, 8, 0, 0) == 0                        # invalid problem

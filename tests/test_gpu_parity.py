@@ -299,6 +299,59 @@ def test_segment_chaining(scan):
     check("chained gate grad", torch.cat([dg1, dg2], dim=3), dg.double().cpu().numpy(), 1e-4)
 
 
+# ----------------------------------------------------------------------------- few rows: cut rows
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("plain", [False, True])
+def test_few_long_rows_are_cut_into_segments(scan, dtype, plain):
+    """Fewer rows than compute units: rows are cut into segments (two passes, carries
+    through a workspace). Automatic and requested cuts, aligned and ragged lengths,
+    non-zero initial state and first_prop_grad, initial-state gradient."""
+    cases = [((3, 1, 1, 131072), 0), ((1, 2, 2, 65536), 0), ((2, 1, 1, 40000), 0), ((2, 1, 1, 40001), 0),
+             ((5, 1, 1, 8192), 7), ((300, 1, 1, 4096), 2), ((1, 1, 1, 131072), 255), ((2, 1, 3, 2051), 3)]
+    for (B, M, D, L), segments in cases:
+        gen = torch.Generator().manual_seed(L + segments)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 3).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+        need = scan.module.fmscan_workspace_bytes(B, M, D, L, code, segments << 20)
+        assert need > 0, "this case is meant to take the segmented path"
+        out = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        dx, dg, dh0 = torch.empty_like(out), torch.empty_like(out), torch.empty_like(h0)
+        scan.fm_scan_forward(g, x, h0, out, plain=plain, segments=segments)
+        scan.fm_scan_backward(g, G, fpg, dx, out, x, dg, initial_state=h0, initial_state_grad=dh0,
+                              plain=plain, segments=segments)
+        tag = f"{(B, M, D, L)} {dtype} segments={segments} plain={plain}"
+        check(tag + " states", out, C.forward_f64(g, x, h0, plain), TOL[dtype])
+        tg, gg, delta = O.backward_per_row(g, G, out, x, fpg, h0, plain)
+        check(tag + " token grad", dx, tg, TOL[dtype])
+        check(tag + " gate grad", dg, gg, TOL[dtype])
+        check(tag + " initial state grad", dh0, O.to_f64(g)[:, :, 0][:, :, None] * delta[..., 0], TOL[dtype])
+        # the same problem scanned in one piece agrees to rounding
+        out1 = torch.empty_like(out)
+        scan.fm_scan_forward(g, x, h0, out1, plain=plain, segments=1)
+        check(tag + " cut vs uncut", out, out1.double().cpu().numpy(), TOL[dtype])
+
+
+def test_segment_requests_without_room_fail_loudly(scan):
+    g = torch.rand(2, 1, 65536, device=DEV)
+    x = torch.rand(2, 1, 65536, device=DEV)
+    z = torch.zeros(2, 1, 1, device=DEV)
+    out = torch.empty(2, 1, 1, 65536, device=DEV)
+    lib = scan.module
+    rc = lib.fmscan_forward(g.data_ptr(), x.data_ptr(), z.data_ptr(), out.data_ptr(), 2, 1, 1, 65536, 0,
+                            8 << 20, None, 0, None)
+    assert rc == -6 and b"workspace" in lib.fmscan_last_error()
+    # an automatic cut silently falls back to whole rows when no workspace is offered
+    rc = lib.fmscan_forward(g.data_ptr(), x.data_ptr(), z.data_ptr(), out.data_ptr(), 2, 1, 1, 65536, 0,
+                            0, None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    check("states", out, C.forward_f64(g, x), 1e-5)
+
+
 # ----------------------------------------------------------------------------- autograd level
 
 def test_notebook_design(scan):
@@ -331,8 +384,8 @@ def test_notebook_design(scan):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_autograd_with_initial_state(scan, dtype):
     """FM_Scan with a non-zero initial state: gradients equal the derivative of the
-    recurrence (what autograd gives through the per-timestep form), third gradient
-    is None as in the reference."""
+    recurrence (what autograd gives through the per-timestep form), the one for the
+    initial state included (the reference's CUDA path leaves that one unconnected)."""
     B, M, D, L = 2, 3, 4, 256
     gen = torch.Generator().manual_seed(11)
     g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 1).to(dtype).to(DEV).requires_grad_()
@@ -342,11 +395,16 @@ def test_autograd_with_initial_state(scan, dtype):
     states = scan.fm_scan(g, x, h0)
     assert states.shape == (B, M, D, L) and states.dtype == dtype
     states.backward(G)
-    assert h0.grad is None
     tg, gg = C.backward_f64(g, G, states, x, None, h0)
     check("states", states, C.forward_f64(g, x, h0), TOL[dtype])
     check("d_gates", g.grad, gg.sum(axis=2), TOL[dtype])
     check("d_tokens", x.grad, tg.sum(axis=1), TOL[dtype])
+    _, _, d_h0 = O.backward(g, x, G, h0, states=states)
+    check("d_initial_state", h0.grad, d_h0, TOL[dtype])
+    # without a gradient request for the initial state the third gradient stays None
+    g2, x2 = g.detach().clone().requires_grad_(), x.detach().clone().requires_grad_()
+    scan.fm_scan(g2, x2, h0.detach()).backward(G)
+    assert torch.equal(g2.grad, g.grad) and torch.equal(x2.grad, x.grad)
 
 
 def test_seven_argument_backward_reproduces_reference_kernel(scan):
