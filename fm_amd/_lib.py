@@ -46,6 +46,10 @@ def load() -> ctypes.CDLL:
                                     c_void_p, c_void_p, c_void_p,
                                     c_int64, c_int64, c_int64, c_int64, c_int, c_uint,
                                     c_void_p, c_size_t, c_void_p]
+    lib.fmscan_reduced_groups.restype = c_int64
+    lib.fmscan_reduced_groups.argtypes = [c_int64]
+    lib.fmscan_backward_reduced.restype = c_int
+    lib.fmscan_backward_reduced.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     got = lib.fmscan_abi_version()
     if got != ABI_VERSION:
         raise RuntimeError(f"libfmscan_hip.so has ABI version {got}, this package needs {ABI_VERSION}; "

@@ -120,14 +120,15 @@ Grid throttled_grid(const void* kern, int64_t slots, int R, unsigned blocks_per_
 // best when there are many rows of moderate length; long rows want several waves side
 // by side so that fewer rows are open at a time; with few rows a block per row keeps
 // every compute unit busy. About two waves per SIMD is where HBM efficiency peaks;
-// more resident rows lower it. With fewer rows than the chip has compute units, and a
-// workspace to hold the segment pairs, rows are cut into segments (two passes).
+// more resident rows lower it. With so few rows that even eight waves per row leave
+// compute units idle (fewer than 32 rows), and a workspace to hold the segment pairs,
+// rows are cut into segments (two passes).
 struct Tuning {
     unsigned waves, blocks_per_cu, depth;
     int32_t nseg;       // segments per row (1 = the row is scanned in one piece)
     int64_t seg_tiles;  // tiles per segment
 };
-constexpr int64_t kSplitBelowRows = 256;    // rows below which cutting rows is considered
+constexpr int64_t kSplitBelowRows = 32;     // rows below which cutting rows pays (measured)
 constexpr int64_t kSplitTargetSlots = 2048;  // segments in flight the cut aims for
 constexpr int64_t kSplitMinTiles = 4;       // a segment is at least this many tiles
 constexpr int64_t kMaxSegments = 255;
@@ -293,6 +294,8 @@ void launch_aggregate(int dtype, const Problem& pb, const Tuning& t, bool vec, c
     });
 }
 
+constexpr int kReducedGroup = 8;  // consecutive d one block of the reduced backward kernel sums over
+
 }  // namespace
 
 extern "C" {
@@ -397,6 +400,74 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
                                                              pairs, (hipStream_t)stream);
     });
     return launched("backward");
+}
+
+int64_t fmscan_reduced_groups(int64_t D) { return D < 1 ? 0 : (D + kReducedGroup - 1) / kReducedGroup; }
+
+int fmscan_backward_reduced(const void* gates, const void* out_grad, const void* first_prop_grad,
+                            void* token_grad, const void* cached_output, const void* input_tokens,
+                            float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                            int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                            void* stream) {
+    Problem pb;
+    if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
+    if (flags & ~FMSCAN_FLAG_PLAIN)
+        return fail(FMSCAN_E_FLAGS, "fmscan_backward_reduced: only FMSCAN_FLAG_PLAIN is understood here");
+    if (!gates || !out_grad || !token_grad || !cached_output || !gate_grad_partial)
+        return fail(FMSCAN_E_NULL, "fmscan_backward_reduced: gates, out_grad, token_grad, cached_output and "
+                    "gate_grad_partial must not be NULL");
+    if (!pb.plain && !input_tokens)
+        return fail(FMSCAN_E_NULL, "fmscan_backward_reduced: input_tokens must not be NULL without "
+                    "FMSCAN_FLAG_PLAIN");
+    if (B > INT32_MAX / fmscan_reduced_groups(D))
+        return fail(FMSCAN_E_SHAPE, "fmscan_backward_reduced: B * ceil(D/%d) must be < 2^31", kReducedGroup);
+    const int64_t full = pb.rows * L * pb.esize;
+    const int64_t groups = fmscan_reduced_groups(D);
+    const Range outs[] = {{"token_grad", token_grad, B * D * L * pb.esize},
+                          {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
+                          {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
+    const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
+                         {"out_grad", out_grad, full},
+                         {"first_prop_grad", first_prop_grad, pb.rows * pb.esize},
+                         {"cached_output", cached_output, full},
+                         {"input_tokens", pb.plain ? nullptr : input_tokens, B * D * L * pb.esize},
+                         {"initial_state", initial_state, pb.rows * pb.esize}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in))
+                return fail(FMSCAN_E_ALIAS, "fmscan_backward_reduced: %s overlaps %s", o.name, in.name);
+    for (int i = 0; i < 3; ++i)
+        for (int j = i + 1; j < 3; ++j)
+            if (overlap(outs[i], outs[j]))
+                return fail(FMSCAN_E_ALIAS, "fmscan_backward_reduced: %s overlaps %s", outs[i].name, outs[j].name);
+    const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
+                     aligned16(token_grad) && aligned16(cached_output) &&
+                     (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial);
+    if (!vec)
+        return fail(FMSCAN_E_UNALIGNED, "fmscan_backward_reduced: pointers and L * sizeof(element) must be "
+                    "multiples of 16 bytes; use fmscan_backward");
+    const size_t tile = (size_t)(16 / pb.esize) * 64;
+    const size_t lds = (2 * kReducedGroup * tile + (size_t)kReducedGroup * (size_t)M) * sizeof(float);
+    if (lds > 160u * 1024u)
+        return fail(FMSCAN_E_SHAPE, "fmscan_backward_reduced: M = %lld needs %zu bytes of LDS (limit 163840); "
+                    "use fmscan_backward", (long long)M, lds);
+    const void* h_init = initial_state ? initial_state : first_prop_grad;
+    const unsigned grid = (unsigned)(B * groups);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        auto go = [&](auto pt) {
+            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, 3, decltype(pt)::value>;
+            if (lds > 48u * 1024u)
+                (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            kern<<<grid, 64 * kReducedGroup, lds, (hipStream_t)stream>>>(
+                (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
+                (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
+                (T*)initial_state_grad, (int32_t)M, (int32_t)D, L);
+        };
+        if (pb.plain) go(BoolTag<true>{});
+        else go(BoolTag<false>{});
+    });
+    return launched("backward (reduced)");
 }
 
 }  // extern "C"

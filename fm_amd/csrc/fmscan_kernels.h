@@ -395,4 +395,181 @@ __global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
     if (lane == 0) seg_pairs[r * nseg + seg.index] = make_float2(A, B);
 }
 
+// ---- backward with the D and M sums inside -------------------------------------------
+// For M > 1 and D > 1 the per-pair gradients are only ever summed: d_gates = sum over d,
+// d_tokens = sum over m (reference fm/scan/fm_scan.py:76-78; its kernel writes both
+// (B, M, D, L) tensors "to avoid atomicAdd", fm_scan.cuh:200-207, and torch.sum reads them
+// back). This kernel never writes them. A block is one batch element b and DG
+// consecutive d (one wave each); its waves walk the tiles of their rows from the end,
+// and at every tile visit the M rows (b, m, d) one after the other, all waves on the same
+// (tile, m) step:
+//   * token gradient: summed over m in registers, stored once per tile as d_tokens[b, d, :]
+//   * gate gradient: the DG waves add their tiles up in LDS (one barrier per step) and
+//     store the sum for this group of d, gate_partial[b, m, group, :] in float32; the
+//     caller adds the ceil(D / DG) groups.
+// Each wave keeps the running state of its M rows in LDS (one float per row).
+// HBM traffic: G and h once (2s per element) plus 4/DG bytes per element of partials,
+// against 6s for the unfused kernel plus the two torch.sum passes.
+template <typename T, int DG, int P, bool PLAIN>
+__global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
+    const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
+    T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved,
+    const T* __restrict__ tokens, float* __restrict__ gate_partial /* (B, M, NG, L) */,
+    const T* __restrict__ h0, T* __restrict__ h0_grad, int32_t M, int32_t D, int64_t L) {
+    constexpr int E = Elem<T>::E;
+    constexpr int TILE = E * 64;
+    constexpr int SLICE = TILE / DG;  // elements of a summed tile each wave adds up and stores
+    static_assert(TILE % DG == 0, "a tile must split evenly over the waves");
+    extern __shared__ float lds[];
+    float* red = lds;                            // [2][DG][TILE]
+    float* carries = lds + 2 * DG * TILE;        // [DG][M]
+
+    const int lane = threadIdx.x & 63;
+    const int w = uniform(threadIdx.x >> 6);
+    const int32_t NG = (D + DG - 1) / DG;
+    const int64_t b = blockIdx.x / NG;
+    const int32_t grp = (int32_t)(blockIdx.x - b * NG);
+    const bool active = grp * DG + w < D;        // a wave past the last d still joins every barrier
+    const int64_t d = active ? grp * DG + w : D - 1;
+    const int64_t ntiles = (L + TILE - 1) / TILE;
+    const int64_t lane_off = (int64_t)(63 - lane) * E;
+    float* mycarry = carries + w * M;
+
+    for (int32_t m = lane; m < M; m += 64)
+        mycarry[m] = first_prop_grad ? Elem<T>::widen(first_prop_grad[(b * M + m) * D + d]) : 0.0f;
+
+    const T* __restrict__ xrow = tokens + (b * D + d) * L;  // never read when PLAIN
+    T* __restrict__ dxrow = token_grad + (b * D + d) * L;
+
+    struct Entry {
+        u32x4 g, G, h;
+        float hb;
+    };
+    // steps are numbered q = (ntiles - 1 - k) * M + m; `q >= nsteps` loads nothing
+    const int64_t nsteps = ntiles * M;
+    auto fetch = [&](Entry& e, int64_t k, int32_t m, bool live) {
+        const int64_t row = (b * M + m) * D + d;
+        const int64_t t0 = live ? k * TILE + lane_off : L;
+        const T* __restrict__ hrow = h_saved + row * L;
+        e.g = load_chunk<T, true, false>(gates + (b * M + m) * L, t0, L, Elem<T>::kOnes);
+        e.G = load_chunk<T, true, true>(out_grad + row * L, t0, L, 0u);
+        e.h = load_chunk<T, true, true>(hrow, t0, L, 0u);
+        e.hb = 0.0f;
+        if (lane == 63 && t0 < L) {
+            if (t0 > 0) e.hb = Elem<T>::widen(hrow[t0 - 1]);
+            else if (h0) e.hb = Elem<T>::widen(h0[row]);
+        }
+    };
+
+    // head: the next step to fetch
+    int64_t hk = ntiles - 1;
+    int32_t hm = 0;
+    int64_t hq = 0;
+    auto fetch_next = [&](Entry& e) {
+        fetch(e, hk, hm, hq < nsteps);
+        ++hq;
+        if (++hm == M) { hm = 0; --hk; }
+    };
+
+    Entry q[P];
+#pragma unroll
+    for (int s = 0; s < P; ++s) fetch_next(q[s]);
+    // the token tile is shared by the M steps of a tile; the one for the next tile is
+    // fetched while the current tile is worked on
+    u32x4 x_raw = {0u, 0u, 0u, 0u}, x_next = {0u, 0u, 0u, 0u};
+    if constexpr (!PLAIN) x_next = load_chunk<T, true, false>(xrow, (ntiles - 1) * TILE + lane_off, L, 0u);
+
+    __syncthreads();  // carries are in place
+
+    float dtok[E];
+    int64_t k = ntiles - 1;
+    int32_t m = 0;
+    for (int64_t q0 = 0; q0 < nsteps; q0 += P) {
+#pragma unroll
+        for (int s = 0; s < P; ++s) {
+            const int64_t step = q0 + s;
+            if (step >= nsteps) break;
+            const Entry cur = q[s];
+            fetch_next(q[s]);
+            const int64_t t0 = k * TILE + lane_off;
+            if (m == 0) {
+                if constexpr (!PLAIN) {
+                    x_raw = x_next;
+                    x_next = load_chunk<T, true, false>(xrow, k > 0 ? t0 - TILE : L, L, 0u);
+                }
+#pragma unroll
+                for (int i = 0; i < E; ++i) dtok[i] = 0.0f;
+            }
+            const float carry = mycarry[m];
+
+            float g[E], G[E], h[E], p[E];
+            Elem<T>::unpack(cur.g, g);
+            Elem<T>::unpack(cur.G, G);
+            Elem<T>::unpack(cur.h, h);
+#pragma unroll
+            for (int i = 0; i < E; ++i) p[i] = g[i] * G[i];
+            float a = g[E - 1], bb = p[E - 1];
+#pragma unroll
+            for (int i = E - 2; i >= 0; --i) {
+                bb = __builtin_fmaf(g[i], bb, p[i]);
+                a *= g[i];
+            }
+            wave_scan_inclusive(a, bb);
+            const float ea = dpp<kWaveShr1>(1.0f, a);
+            const float eb = dpp<kWaveShr1>(0.0f, bb);
+            const float ta = lane63(a), tb = lane63(bb);
+            const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
+            if (lane == 0) mycarry[m] = __builtin_fmaf(ta, carry, tb);
+
+            float c = __builtin_fmaf(ea, carry, eb);
+            float dg[E];
+            if constexpr (!PLAIN) Elem<T>::unpack(x_raw, dg);  // dg[] starts as x_t
+#pragma unroll
+            for (int i = E - 1; i >= 0; --i) {
+                const float delta = G[i] + c;
+                c = __builtin_fmaf(g[i], c, p[i]);
+                const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
+                if constexpr (PLAIN) {
+                    dtok[i] += delta;
+                    dg[i] = hp * delta;
+                } else {
+                    dtok[i] += __builtin_fmaf(-g[i], delta, delta);
+                    dg[i] = (hp - dg[i]) * delta;
+                }
+                if (!active) dg[i] = 0.0f;
+            }
+
+            // add the gate gradient tiles of the DG waves: each wave lays its tile out in
+            // memory order, then sums one slice of the tile over all waves and stores it
+            float* mine = red + ((step & 1) * DG + w) * TILE + lane_off;
+#pragma unroll
+            for (int i = 0; i < E; i += 4)
+                *reinterpret_cast<float4*>(mine + i) = make_float4(dg[i], dg[i + 1], dg[i + 2], dg[i + 3]);
+            __syncthreads();
+            const float* all = red + (step & 1) * DG * TILE + w * SLICE;
+            float* __restrict__ prow = gate_partial + ((b * M + m) * NG + grp) * L + k * TILE + w * SLICE;
+            for (int e = lane; e < SLICE; e += 64) {
+                float sum = 0.0f;
+#pragma unroll
+                for (int v = 0; v < DG; ++v) sum += all[v * TILE + e];
+                if (k * TILE + w * SLICE + e < L) __builtin_nontemporal_store(sum, prow + e);
+            }
+
+            if (m == M - 1 && active) store_chunk<T, true>(dxrow, t0, L, Elem<T>::pack(dtok));
+            if (++m == M) { m = 0; --k; }
+        }
+    }
+
+    if (h0_grad && active) {
+        __builtin_amdgcn_wave_barrier();  // lane 0's last carry writes are visible to the wave
+        for (int32_t mm = lane; mm < M; mm += 64) {
+            float v[E] = {mycarry[mm]};
+            const u32x4 packed = Elem<T>::pack(v);
+            const int64_t row = (b * M + mm) * D + d;
+            if constexpr (sizeof(T) == 4) reinterpret_cast<uint32_t*>(h0_grad)[row] = packed.x;
+            else reinterpret_cast<uint16_t*>(h0_grad)[row] = (uint16_t)(packed.x & 0xffffu);
+        }
+    }
+}
+
 }  // namespace fmscan

@@ -19,7 +19,8 @@ import torch
 
 from .. import _lib
 
-__all__ = ["fm_scan_forward", "fm_scan_backward", "FM_Scan", "fm_scan", "fm_memory", "module"]
+__all__ = ["fm_scan_forward", "fm_scan_backward", "fm_scan_backward_reduced", "FM_Scan", "fm_scan",
+           "fm_memory", "module"]
 
 _DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16,
            torch.bfloat16: _lib.DTYPE_BF16}
@@ -147,6 +148,58 @@ def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output,
     return None
 
 
+def _reduced_ok(gates, tokens, states, grad_output) -> bool:
+    """The fused-sum backward needs both sums to be real (M > 1 and D > 1), 16-byte aligned
+    rows and pointers, and one float of LDS per memory row and wave."""
+    B, M, D, L = states.shape
+    if M < 2 or D < 2 or M > 2048 or (L * states.element_size()) % 16:
+        return False
+    return all(t.data_ptr() % 16 == 0 for t in (gates, tokens, states, grad_output))
+
+
+def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input_tokens, *,
+                             initial_state=None, initial_state_grad=None, plain=False):
+    """Backward scan that returns the summed gradients (d_gates (B, M, L), d_tokens (B, D, L))
+    without materialising the two (B, M, D, L) per-pair tensors the reference writes and
+    sums afterwards (fm_scan.py:70-78). Same mathematics as `fm_scan_backward` followed by
+    `.sum(dim=2)` / `.sum(dim=1)`, with the sums accumulated in float32."""
+    dev = gates.device
+    named = [("gates", gates), ("outGrad", outGrad), ("firstPropGrad", firstPropGrad),
+             ("cached_output", cached_output), ("input_tokens", input_tokens)]
+    for name, t in (("initial_state", initial_state), ("initial_state_grad", initial_state_grad)):
+        if t is not None:
+            named.append((name, t))
+    for name, t in named:
+        _on_gpu(name, t, dev)
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        _require(t.dtype == gates.dtype, f"{name} has dtype {t.dtype}, gates has {gates.dtype}")
+    _require(cached_output.dim() == 4, "cached_output must be (B, M, D, L)")
+    B, M, D, L = cached_output.shape
+    _require(tuple(gates.shape) == (B, M, L), f"gates must be {(B, M, L)}, got {tuple(gates.shape)}")
+    _require(tuple(input_tokens.shape) == (B, D, L),
+             f"input_tokens must be {(B, D, L)}, got {tuple(input_tokens.shape)}")
+    _require(tuple(outGrad.shape) == (B, M, D, L), f"outGrad must be {(B, M, D, L)}")
+    for name, t in (("firstPropGrad", firstPropGrad), ("initial_state", initial_state),
+                    ("initial_state_grad", initial_state_grad)):
+        if t is not None:
+            _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
+    code = _dtype_code(gates)
+    groups = module.fmscan_reduced_groups(D)
+    d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
+    partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
+    if cached_output.numel():
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            _lib.check(module.fmscan_backward_reduced(
+                gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), d_tokens.data_ptr(),
+                cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(),
+                None if initial_state is None else initial_state.data_ptr(),
+                None if initial_state_grad is None else initial_state_grad.data_ptr(),
+                B, M, D, L, code, _lib.FLAG_PLAIN if plain else 0, stream))
+    d_gates = partial.sum(dim=2).to(gates.dtype)  # the few groups of d, still in float32
+    return d_gates, d_tokens
+
+
 class FM_Scan(torch.autograd.Function):
     """states = FM_Scan.apply(gates, tokens, initial_state=None)
 
@@ -189,11 +242,19 @@ class FM_Scan(torch.autograd.Function):
 
         first_prop_grad = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
         grad_output = grad_output.contiguous()
-        per_pair_gates = torch.empty_like(states)   # (B, M, D, L)
-        per_pair_tokens = torch.empty_like(states)  # (B, M, D, L)
         # The reference leaves the initial state's gradient unconnected (fm_scan.py:80-81); it
         # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
         d_initial_state = torch.empty_like(first_prop_grad) if ctx.needs_input_grad[2] else None
+
+        if _reduced_ok(gates, tokens, states, grad_output):
+            # both sums are real: one kernel produces d_gates and d_tokens directly
+            d_gates, d_tokens = fm_scan_backward_reduced(
+                gates, grad_output, first_prop_grad, states, tokens,
+                initial_state=initial_state, initial_state_grad=d_initial_state)
+            return d_gates, d_tokens, d_initial_state
+
+        per_pair_gates = torch.empty_like(states)   # (B, M, D, L)
+        per_pair_tokens = torch.empty_like(states)  # (B, M, D, L)
         fm_scan_backward(gates, grad_output, first_prop_grad, per_pair_tokens, states, tokens,
                          per_pair_gates, initial_state=initial_state,
                          initial_state_grad=d_initial_state)

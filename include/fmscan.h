@@ -15,7 +15,7 @@
  * kernels on `stream` (a hipStream_t, NULL = the default stream) and return
  * without waiting.
  *
- * Workspace. With fewer rows (B*M*D) than the GPU has compute units a row is
+ * Workspace. With very few rows (B*M*D < 32) and long sequences a row is
  * cut into segments that are scanned side by side; the carry between segments
  * goes through `workspace` (two floats per segment, written by a first pass).
  * fmscan_workspace_bytes() tells how much a call can use; a NULL or smaller
@@ -74,6 +74,7 @@ extern "C" {
 #define FMSCAN_E_FLAGS     (-4) /* unknown flag bit or unsupported waves-per-row value */
 #define FMSCAN_E_ALIAS     (-5) /* an output overlaps an input it must not overlap */
 #define FMSCAN_E_WORKSPACE (-6) /* segments were requested and the workspace is missing or small */
+#define FMSCAN_E_UNALIGNED (-7) /* this entry point needs 16-byte aligned pointers and rows */
 
 /* Version of this interface; equals FMSCAN_ABI_VERSION of the header the
  * library was built from. No counterpart in the reference (its extension is
@@ -140,6 +141,30 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
                     int64_t B, int64_t M, int64_t D, int64_t L,
                     int dtype, unsigned flags,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Backward scan with the two sums of FM_Scan.backward inside (reference
+ * fm/scan/fm_scan.py:70-78: d_gates = gateGradOut.sum(dim=2), d_tokens =
+ * tokenGradOut.sum(dim=1); the reference's kernel writes both (B, M, D, L) tensors in
+ * full, fm/scan/fm_scan.cuh:200-207, and names the fused form as a TODO). Meant for
+ * M > 1 and D > 1; the per-pair tensors are never written.
+ *   token_grad         (B, D, L)     out, element dtype: sum over m of (1 - g) * delta
+ *   gate_grad_partial  (B, M, G, L)  out, float32, G = fmscan_reduced_groups(D): the sum of
+ *                      (h[t-1] - x[t]) * delta over each group of 8 consecutive d;
+ *                      d_gates[b,m,t] is the sum of the G partials (one more small pass
+ *                      for the caller; sums are accumulated in float32 throughout)
+ * Other arguments as fmscan_backward. Needs 16-byte aligned pointers and
+ * L * sizeof(element) % 16 == 0 (FMSCAN_E_UNALIGNED otherwise: use fmscan_backward);
+ * flags: only FMSCAN_FLAG_PLAIN.
+ */
+int64_t fmscan_reduced_groups(int64_t D);
+int fmscan_backward_reduced(const void* gates, const void* out_grad, const void* first_prop_grad,
+                            void* token_grad,
+                            const void* cached_output, const void* input_tokens,
+                            float* gate_grad_partial,
+                            const void* initial_state, void* initial_state_grad,
+                            int64_t B, int64_t M, int64_t D, int64_t L,
+                            int dtype, unsigned flags, void* stream);
 
 #ifdef __cplusplus
 }

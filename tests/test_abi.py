@@ -23,8 +23,9 @@ def declared_functions():
 
 
 def test_header_declares_the_expected_entry_points():
-    assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_forward",
-                                    "fmscan_last_error", "fmscan_workspace_bytes"]
+    assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_reduced",
+                                    "fmscan_forward", "fmscan_last_error", "fmscan_reduced_groups",
+                                    "fmscan_workspace_bytes"]
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -87,6 +88,15 @@ def test_rejected_arguments(lib):
     assert fwd(lib, L=1 << 16, flags=4 << 20, ws=7 * P, ws_bytes=8) == E_WORKSPACE  # too small
     assert bwd(lib, L=1 << 16, flags=4 << 20) == E_WORKSPACE
     assert bwd(lib, dh0=4 * P) == E_ALIAS             # initial_state_grad on top of cached_output
+    red = lambda **k: lib.fmscan_backward_reduced(
+        k.get("g", P), 2 * P, None, k.get("dx", 3 * P), 4 * P, 5 * P, k.get("part", 6 * P), None, None,
+        2, 2, k.get("D", 2), k.get("L", 8), k.get("dtype", 0), k.get("flags", 0), None)
+    assert red(part=None) == E_NULL
+    assert red(flags=1 << 8) == E_FLAGS               # tuning flags do not apply here
+    assert red(dx=4 * P) == E_ALIAS
+    assert red(L=7) == _const("FMSCAN_E_UNALIGNED")
+    assert red(g=P + 4) == _const("FMSCAN_E_UNALIGNED")
+    assert lib.fmscan_reduced_groups(128) == 16 and lib.fmscan_reduced_groups(9) == 2
     assert fwd(lib, out=P) == E_ALIAS                 # out on top of gates
     assert fwd(lib, out=2 * P + 16) == E_ALIAS        # out inside tokens
     assert bwd(lib, h=None) == E_NULL
@@ -99,7 +109,7 @@ def test_rejected_arguments(lib):
 
 
 def test_workspace_bytes(lib):
-    """Two floats per segment, only for problems with fewer rows than compute units (or on request)."""
+    """Two floats per segment, only for problems with very few rows (or on request)."""
     wb = lib.fmscan_workspace_bytes
     assert wb(16 * 2048, 1, 1, 16384, 2, 0) == 0          # many rows: never cut
     assert wb(4, 1, 1, 65536, 2, 0) == 4 * 32 * 8           # 4 rows of 128 tiles -> 32 segments of 4 tiles

@@ -352,6 +352,53 @@ def test_segment_requests_without_room_fail_loudly(scan):
     check("states", out, C.forward_f64(g, x), 1e-5)
 
 
+# ----------------------------------------------------------------------------- sums inside the kernel
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("plain", [False, True])
+def test_backward_with_sums_inside(scan, dtype, plain):
+    """fm_scan_backward_reduced (d_gates, d_tokens straight from one kernel) against the
+    float64 oracle's summed gradients, and against the two-tensor path plus torch.sum."""
+    for (B, M, D, L) in [(2, 3, 5, 512), (1, 2, 2, 8), (2, 4, 8, 4096), (1, 33, 17, 1000 // 8 * 8),
+                         (3, 2, 9, 2048), (1, 70, 3, 640)]:
+        gen = torch.Generator().manual_seed(M * 100 + D)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        out = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        scan.fm_scan_forward(g, x, h0, out, plain=plain)
+        dh0 = torch.empty_like(h0)
+        d_g, d_x = scan.fm_scan_backward_reduced(g, G, fpg, out, x, initial_state=h0,
+                                                 initial_state_grad=dh0, plain=plain)
+        assert d_g.shape == (B, M, L) and d_x.shape == (B, D, L) and d_g.dtype == dtype
+        tg, gg, delta = O.backward_per_row(g, G, out, x, fpg, h0, plain)
+        tag = f"{(B, M, D, L)} {dtype} plain={plain}"
+        check(tag + " d_gates", d_g, gg.sum(axis=2), TOL[dtype])
+        check(tag + " d_tokens", d_x, tg.sum(axis=1), TOL[dtype])
+        check(tag + " d_initial_state", dh0, O.to_f64(g)[:, :, 0][:, :, None] * delta[..., 0], TOL[dtype])
+        # the reference's route: two full tensors, then torch.sum
+        dx, dg = torch.empty_like(out), torch.empty_like(out)
+        scan.fm_scan_backward(g, G, fpg, dx, out, x, dg, initial_state=h0, plain=plain)
+        check(tag + " vs two-tensor route (gates)", d_g, dg.sum(dim=2).double().cpu().numpy(), 2 * TOL[dtype])
+        check(tag + " vs two-tensor route (tokens)", d_x, dx.sum(dim=1).double().cpu().numpy(), 2 * TOL[dtype])
+
+
+def test_backward_with_sums_inside_is_deterministic(scan):
+    B, M, D, L, dt = 2, 8, 24, 2048, torch.bfloat16
+    gen = gpu_gen(21)
+    g = torch.rand(B, M, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(B, D, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    z = torch.zeros(B, M, D, dtype=dt, device=DEV)
+    out = torch.empty(B, M, D, L, dtype=dt, device=DEV)
+    scan.fm_scan_forward(g, x, z, out)
+    a = scan.fm_scan_backward_reduced(g, G, z, out, x)
+    b = scan.fm_scan_backward_reduced(g, G, z, out, x)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
 # ----------------------------------------------------------------------------- autograd level
 
 def test_notebook_design(scan):
