@@ -295,6 +295,7 @@ void launch_aggregate(int dtype, const Problem& pb, const Tuning& t, bool vec, c
 }
 
 constexpr int kReducedGroup = 8;  // consecutive d one block of the reduced backward kernel sums over
+constexpr int kReducedChunk = 1;  // tiles of a row visited before moving to the next m (1 measured best)
 
 }  // namespace
 
@@ -456,7 +457,7 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
         auto go = [&](auto pt) {
-            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, 3, decltype(pt)::value>;
+            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, kReducedChunk, decltype(pt)::value>;
             if (lds > 48u * 1024u)
                 (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             kern<<<grid, 64 * kReducedGroup, lds, (hipStream_t)stream>>>(

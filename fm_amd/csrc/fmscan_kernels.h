@@ -400,17 +400,22 @@ __global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
 // d_tokens = sum over m (reference fm/scan/fm_scan.py:76-78; its kernel writes both
 // (B, M, D, L) tensors "to avoid atomicAdd", fm_scan.cuh:200-207, and torch.sum reads them
 // back). This kernel never writes them. A block is one batch element b and DG
-// consecutive d (one wave each); its waves walk the tiles of their rows from the end,
-// and at every tile visit the M rows (b, m, d) one after the other, all waves on the same
-// (tile, m) step:
-//   * token gradient: summed over m in registers, stored once per tile as d_tokens[b, d, :]
+// consecutive d (one wave each). Its waves walk their rows from the end in chunks of C
+// tiles; inside a chunk they visit the M rows (b, m, d) one after the other and, for each,
+// the C tiles of the chunk, all waves on the same (chunk, m, tile) step:
+//   * token gradient: summed over m in registers (C tiles of accumulators), stored once
+//     per chunk as d_tokens[b, d, :]
 //   * gate gradient: the DG waves add their tiles up in LDS (one barrier per step) and
 //     store the sum for this group of d, gate_partial[b, m, group, :] in float32; the
 //     caller adds the ceil(D / DG) groups.
-// Each wave keeps the running state of its M rows in LDS (one float per row).
+// Each wave keeps the running state of its M rows in LDS (one float per row); the loads
+// of the same tile position of the next row are in flight while a tile is worked on.
 // HBM traffic: G and h once (2s per element) plus 4/DG bytes per element of partials,
-// against 6s for the unfused kernel plus the two torch.sum passes.
-template <typename T, int DG, int P, bool PLAIN>
+// against 6s for the unfused kernel plus the two torch.sum passes. With a third of the
+// bytes per element the arithmetic (about 20 VALU operations per element) weighs as
+// much as the memory here: measured 2.5-4.3 TB/s of G + h, 1.2-2.3x faster end to end
+// than the two-tensor route; C = 1 measured best.
+template <typename T, int DG, int C, bool PLAIN>
 __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved,
@@ -432,6 +437,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const bool active = grp * DG + w < D;        // a wave past the last d still joins every barrier
     const int64_t d = active ? grp * DG + w : D - 1;
     const int64_t ntiles = (L + TILE - 1) / TILE;
+    const int64_t nchunks = (ntiles + C - 1) / C;
     const int64_t lane_off = (int64_t)(63 - lane) * E;
     float* mycarry = carries + w * M;
 
@@ -445,11 +451,10 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
         u32x4 g, G, h;
         float hb;
     };
-    // steps are numbered q = (ntiles - 1 - k) * M + m; `q >= nsteps` loads nothing
-    const int64_t nsteps = ntiles * M;
-    auto fetch = [&](Entry& e, int64_t k, int32_t m, bool live) {
+    // tile k of row (b, m, d); k outside [0, ntiles) loads nothing
+    auto fetch = [&](Entry& e, int64_t k, int32_t m) {
         const int64_t row = (b * M + m) * D + d;
-        const int64_t t0 = live ? k * TILE + lane_off : L;
+        const int64_t t0 = (k >= 0 && k < ntiles) ? k * TILE + lane_off : L;
         const T* __restrict__ hrow = h_saved + row * L;
         e.g = load_chunk<T, true, false>(gates + (b * M + m) * L, t0, L, Elem<T>::kOnes);
         e.G = load_chunk<T, true, true>(out_grad + row * L, t0, L, 0u);
@@ -461,107 +466,111 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
         }
     };
 
-    // head: the next step to fetch
-    int64_t hk = ntiles - 1;
-    int32_t hm = 0;
-    int64_t hq = 0;
-    auto fetch_next = [&](Entry& e) {
-        fetch(e, hk, hm, hq < nsteps);
-        ++hq;
-        if (++hm == M) { hm = 0; --hk; }
-    };
-
-    Entry q[P];
+    // ring slot i holds tile (chunk * C + i) of the row that is worked on next at that
+    // position: slot i is refilled, right after use, with the same position of row m + 1
+    // (or of row 0 of the chunk before)
+    Entry q[C];
+    u32x4 x_raw[C], x_next[C];
 #pragma unroll
-    for (int s = 0; s < P; ++s) fetch_next(q[s]);
-    // the token tile is shared by the M steps of a tile; the one for the next tile is
-    // fetched while the current tile is worked on
-    u32x4 x_raw = {0u, 0u, 0u, 0u}, x_next = {0u, 0u, 0u, 0u};
-    if constexpr (!PLAIN) x_next = load_chunk<T, true, false>(xrow, (ntiles - 1) * TILE + lane_off, L, 0u);
+    for (int i = 0; i < C; ++i) {
+        const int64_t k = (nchunks - 1) * C + i;
+        fetch(q[i], k, 0);
+        x_raw[i] = u32x4{0u, 0u, 0u, 0u};
+        x_next[i] = u32x4{0u, 0u, 0u, 0u};
+        if constexpr (!PLAIN) x_next[i] = load_chunk<T, true, false>(xrow, k < ntiles ? k * TILE + lane_off : L, L, 0u);
+    }
 
     __syncthreads();  // carries are in place
 
-    float dtok[E];
-    int64_t k = ntiles - 1;
-    int32_t m = 0;
-    for (int64_t q0 = 0; q0 < nsteps; q0 += P) {
+    int parity = 0;
+    for (int64_t chunk = nchunks - 1; chunk >= 0; --chunk) {
+        float dtok[C][E];
 #pragma unroll
-        for (int s = 0; s < P; ++s) {
-            const int64_t step = q0 + s;
-            if (step >= nsteps) break;
-            const Entry cur = q[s];
-            fetch_next(q[s]);
-            const int64_t t0 = k * TILE + lane_off;
-            if (m == 0) {
-                if constexpr (!PLAIN) {
-                    x_raw = x_next;
-                    x_next = load_chunk<T, true, false>(xrow, k > 0 ? t0 - TILE : L, L, 0u);
+        for (int i = 0; i < C; ++i) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) dtok[i][j] = 0.0f;
+            if constexpr (!PLAIN) {  // this chunk's token tiles; fetch the ones of the chunk before
+                x_raw[i] = x_next[i];
+                const int64_t kp = (chunk - 1) * C + i;
+                x_next[i] = load_chunk<T, true, false>(xrow, chunk > 0 ? kp * TILE + lane_off : L, L, 0u);
+            }
+        }
+        for (int32_t m = 0; m < M; ++m) {
+            float carry = mycarry[m];
+#pragma unroll
+            for (int i = C - 1; i >= 0; --i) {
+                const int64_t k = chunk * C + i;
+                const Entry cur = q[i];
+                if (m + 1 < M) fetch(q[i], k, m + 1);
+                else fetch(q[i], k - C, 0);
+                if (k >= ntiles) continue;  // the last chunk of a row may be short (same for every wave)
+                const int64_t t0 = k * TILE + lane_off;
+
+                float g[E], G[E], h[E], p[E];
+                Elem<T>::unpack(cur.g, g);
+                Elem<T>::unpack(cur.G, G);
+                Elem<T>::unpack(cur.h, h);
+#pragma unroll
+                for (int j = 0; j < E; ++j) p[j] = g[j] * G[j];
+                float a = g[E - 1], bb = p[E - 1];
+#pragma unroll
+                for (int j = E - 2; j >= 0; --j) {
+                    bb = __builtin_fmaf(g[j], bb, p[j]);
+                    a *= g[j];
                 }
-#pragma unroll
-                for (int i = 0; i < E; ++i) dtok[i] = 0.0f;
-            }
-            const float carry = mycarry[m];
+                wave_scan_inclusive(a, bb);
+                const float ea = dpp<kWaveShr1>(1.0f, a);
+                const float eb = dpp<kWaveShr1>(0.0f, bb);
+                const float ta = lane63(a), tb = lane63(bb);
+                const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
 
-            float g[E], G[E], h[E], p[E];
-            Elem<T>::unpack(cur.g, g);
-            Elem<T>::unpack(cur.G, G);
-            Elem<T>::unpack(cur.h, h);
+                float c = __builtin_fmaf(ea, carry, eb);
+                carry = __builtin_fmaf(ta, carry, tb);
+                float dg[E];
+                if constexpr (!PLAIN) Elem<T>::unpack(x_raw[i], dg);  // dg[] starts as x_t
 #pragma unroll
-            for (int i = 0; i < E; ++i) p[i] = g[i] * G[i];
-            float a = g[E - 1], bb = p[E - 1];
-#pragma unroll
-            for (int i = E - 2; i >= 0; --i) {
-                bb = __builtin_fmaf(g[i], bb, p[i]);
-                a *= g[i];
-            }
-            wave_scan_inclusive(a, bb);
-            const float ea = dpp<kWaveShr1>(1.0f, a);
-            const float eb = dpp<kWaveShr1>(0.0f, bb);
-            const float ta = lane63(a), tb = lane63(bb);
-            const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
-            if (lane == 0) mycarry[m] = __builtin_fmaf(ta, carry, tb);
-
-            float c = __builtin_fmaf(ea, carry, eb);
-            float dg[E];
-            if constexpr (!PLAIN) Elem<T>::unpack(x_raw, dg);  // dg[] starts as x_t
-#pragma unroll
-            for (int i = E - 1; i >= 0; --i) {
-                const float delta = G[i] + c;
-                c = __builtin_fmaf(g[i], c, p[i]);
-                const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
-                if constexpr (PLAIN) {
-                    dtok[i] += delta;
-                    dg[i] = hp * delta;
-                } else {
-                    dtok[i] += __builtin_fmaf(-g[i], delta, delta);
-                    dg[i] = (hp - dg[i]) * delta;
+                for (int j = E - 1; j >= 0; --j) {
+                    const float delta = G[j] + c;
+                    c = __builtin_fmaf(g[j], c, p[j]);
+                    const float hp = (j > 0) ? h[j > 0 ? j - 1 : 0] : hprev0;
+                    if constexpr (PLAIN) {
+                        dtok[i][j] += delta;
+                        dg[j] = hp * delta;
+                    } else {
+                        dtok[i][j] += __builtin_fmaf(-g[j], delta, delta);
+                        dg[j] = (hp - dg[j]) * delta;
+                    }
+                    if (!active) dg[j] = 0.0f;
                 }
-                if (!active) dg[i] = 0.0f;
-            }
 
-            // add the gate gradient tiles of the DG waves: each wave lays its tile out in
-            // memory order, then sums one slice of the tile over all waves and stores it
-            float* mine = red + ((step & 1) * DG + w) * TILE + lane_off;
+                // add the gate gradient tiles of the DG waves: each wave lays its tile out in
+                // memory order, then sums one slice of the tile over all waves and stores it
+                float* mine = red + (parity * DG + w) * TILE + lane_off;
 #pragma unroll
-            for (int i = 0; i < E; i += 4)
-                *reinterpret_cast<float4*>(mine + i) = make_float4(dg[i], dg[i + 1], dg[i + 2], dg[i + 3]);
-            __syncthreads();
-            const float* all = red + (step & 1) * DG * TILE + w * SLICE;
-            float* __restrict__ prow = gate_partial + ((b * M + m) * NG + grp) * L + k * TILE + w * SLICE;
-            for (int e = lane; e < SLICE; e += 64) {
-                float sum = 0.0f;
+                for (int j = 0; j < E; j += 4)
+                    *reinterpret_cast<float4*>(mine + j) = make_float4(dg[j], dg[j + 1], dg[j + 2], dg[j + 3]);
+                __syncthreads();
+                const float* all = red + parity * DG * TILE + w * SLICE;
+                float* __restrict__ prow = gate_partial + ((b * M + m) * NG + grp) * L + k * TILE + w * SLICE;
+                for (int e = lane; e < SLICE; e += 64) {
+                    float sum = 0.0f;
 #pragma unroll
-                for (int v = 0; v < DG; ++v) sum += all[v * TILE + e];
-                if (k * TILE + w * SLICE + e < L) __builtin_nontemporal_store(sum, prow + e);
+                    for (int v = 0; v < DG; ++v) sum += all[v * TILE + e];
+                    if (k * TILE + w * SLICE + e < L) __builtin_nontemporal_store(sum, prow + e);
+                }
+                parity ^= 1;
             }
-
-            if (m == M - 1 && active) store_chunk<T, true>(dxrow, t0, L, Elem<T>::pack(dtok));
-            if (++m == M) { m = 0; --k; }
+            if (lane == 0) mycarry[m] = carry;
+        }
+        if (active) {
+#pragma unroll
+            for (int i = 0; i < C; ++i)
+                store_chunk<T, true>(dxrow, (chunk * C + i) * TILE + lane_off, L, Elem<T>::pack(dtok[i]));
         }
     }
 
     if (h0_grad && active) {
-        __builtin_amdgcn_wave_barrier();  // lane 0's last carry writes are visible to the wave
+        __builtin_amdgcn_wave_barrier();  // lane 0's carry writes precede the reads below
         for (int32_t mm = lane; mm < M; mm += 64) {
             float v[E] = {mycarry[mm]};
             const u32x4 packed = Elem<T>::pack(v);
