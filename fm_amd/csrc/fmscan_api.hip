@@ -170,15 +170,22 @@ Tuning choose(const Problem& pb, bool may_split) {
         while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
         while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
     }
+    // Gates shared by D rows and tokens shared by M rows come from the caches: the kernel
+    // then mostly writes (forward) and the limit on concurrent rows no longer applies.
+    // Measured on (B, M, D, L) = (32,32,128,2048), (1,32,2048,8192), (2,32,512,16384).
+    const bool shared_inputs = pb.M > 1 || pb.D > 1;
+    if (shared_inputs && !pb.waves && pb.rows >= 16384) w = 1;
     t.waves = w;
     plan_segments(pb, t, may_split);
     w = t.waves;
     const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
     if (pb.blocks_per_cu) t.blocks_per_cu = pb.blocks_per_cu;
+    else if (shared_inputs) t.blocks_per_cu = 8;
     else if (w == 1) t.blocks_per_cu = tiles_per_slot >= 16 ? 2 : 4;
     else if (w == 4) t.blocks_per_cu = 2;
     else t.blocks_per_cu = 4;
     if (pb.depth) t.depth = pb.depth;
+    else if (shared_inputs) t.depth = 2;
     else if (w == 1) t.depth = tiles_per_slot >= 16 ? 3 : 4;
     else if (w == 4) t.depth = 4;
     else t.depth = 3;
