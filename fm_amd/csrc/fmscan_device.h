@@ -92,16 +92,26 @@ template <> struct Elem<_Float16> {
 // no other row reads again: it is loaded with the non-temporal hint so that it does
 // not displace anything from the caches on its way through (measured: worth about a
 // tenth of the bandwidth on 1 GiB tensors). Stores always carry the hint.
+template <typename T, bool ONCE>
+__device__ __forceinline__ u32x4 load16(const T* __restrict__ p) {
+    if constexpr (ONCE) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    else return *reinterpret_cast<const u32x4*>(p);
+}
+
+// The VEC form never branches around its load: a chunk outside [0, L) reads the last
+// chunk of the row instead and is replaced by `fill` afterwards. A load that is only
+// sometimes issued would make the compiler wait for every outstanding load before each
+// use (it can no longer count how many newer ones are in flight), which throws the
+// prefetch distance away.
 template <typename T, bool VEC, bool ONCE>
 __device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t0, int64_t L,
                                             uint32_t fill) {
     constexpr int E = Elem<T>::E;
     u32x4 r = {fill, fill, fill, fill};
     if constexpr (VEC) {
-        if (t0 < L) {
-            if constexpr (ONCE) r = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + t0));
-            else r = *reinterpret_cast<const u32x4*>(row + t0);
-        }
+        const bool inside = t0 < L;
+        const u32x4 v = load16<T, ONCE>(row + (inside ? t0 : L - E));
+        r = inside ? v : r;
     } else {
         if (t0 < L) {
             if constexpr (sizeof(T) == 4) {
@@ -122,6 +132,11 @@ __device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t
         }
     }
     return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void store16(T* __restrict__ p, u32x4 r) {
+    __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(p));
 }
 
 template <typename T, bool VEC>

@@ -22,11 +22,21 @@
 // precede its own into the state that enters it.
 #pragma once
 
+#include <type_traits>
+
 #include "fmscan_device.h"
 
 namespace fmscan {
 
+// Values that are the same in every lane of a wave but come out of vector instructions
+// (integer division has no scalar form) are moved to scalar registers, so that the row
+// pointers derived from them do not occupy two vector registers each.
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
 
 // Output row r = (b*M + m)*D + d  ->  gate row b*M + m, token row b*D + d
 // (reference fm/scan/fm_scan.cuh:76-82).
@@ -38,8 +48,8 @@ __device__ __forceinline__ RowMap map_row(int64_t row, int32_t M, int32_t D) {
     const uint32_t gate_row = r / (uint32_t)D;
     const uint32_t b = gate_row / (uint32_t)M;
     RowMap m;
-    m.gate_row = gate_row;
-    m.token_row = (int64_t)b * D + (r - gate_row * (uint32_t)D);
+    m.gate_row = (int64_t)(uint32_t)uniform((int)gate_row);
+    m.token_row = uniform64((int64_t)b * D + (r - gate_row * (uint32_t)D));
     return m;
 }
 
@@ -52,7 +62,7 @@ struct Segment {
 __device__ __forceinline__ Segment locate_segment(int64_t slot, int32_t nseg, int64_t seg_tiles,
                                                   int64_t ntiles) {
     Segment s;
-    s.row = nseg > 1 ? slot / nseg : slot;
+    s.row = nseg > 1 ? uniform64(slot / nseg) : slot;
     s.index = nseg > 1 ? (int32_t)(slot - s.row * nseg) : 0;
     s.k_lo = (int64_t)s.index * seg_tiles;
     s.k_hi = s.k_lo + seg_tiles < ntiles ? s.k_lo + seg_tiles : ntiles;
@@ -93,7 +103,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_forward_kernel(
     constexpr int E = Elem<T>::E;
     constexpr int64_t TILE = (int64_t)E * 64 * W;
     const int lane = threadIdx.x & 63;
-    const int wave = uniform(threadIdx.x >> 6);
+    const int wave = uniform((int)(threadIdx.x >> 6));
     const int w = wave % W;
     const int64_t slot = (int64_t)blockIdx.x * R + wave / W;
     if (slot >= rows * nseg) return;  // whole waves only, and only in barrier-free (W == 1) blocks
@@ -118,61 +128,95 @@ __global__ __launch_bounds__(64 * W * R) void scan_forward_kernel(
     struct Entry {
         u32x4 g, x;
     };
+    // loads stop at the end of the segment (the end of the row when rows are not cut);
+    // tiles below k_whole lie wholly inside
+    const int64_t t_end = seg.k_hi * TILE < L ? seg.k_hi * TILE : L;
+    const int64_t k_whole = VEC ? t_end / TILE : 0;
+    auto fetch_whole = [&](Entry& q, int64_t k) {  // no check of any kind
+        const int64_t t0 = k * TILE + lane_off;
+        q.g = load16<T, FOLD>(grow + t0);
+        q.x = load16<T, FOLD>(xrow + t0);
+    };
     auto fetch = [&](Entry& q, int64_t k) {
-        // k >= k_hi (past the segment): t0 = L, which every bound check rejects
-        const int64_t t0 = k < seg.k_hi ? k * TILE + lane_off : L;
-        q.g = load_chunk<T, VEC, FOLD>(grow, t0, L, Elem<T>::kOnes);
-        q.x = load_chunk<T, VEC, FOLD>(xrow, t0, L, 0u);
+        const int64_t t0 = k * TILE + lane_off;
+        q.g = load_chunk<T, VEC, FOLD>(grow, t0, t_end, Elem<T>::kOnes);
+        q.x = load_chunk<T, VEC, FOLD>(xrow, t0, t_end, 0u);
     };
 
-    Entry q[P];
+    // One tile: fold, wave scan, meet the other waves, replay, store. `whole` tiles store
+    // without a bound check.
+    auto scan_tile = [&](const Entry& cur, int64_t k, auto whole) {
+        const int64_t t0 = k * TILE + lane_off;
+        float g[E], u[E];
+        Elem<T>::unpack(cur.g, g);
+        Elem<T>::unpack(cur.x, u);
+        if constexpr (!PLAIN) {
 #pragma unroll
-    for (int s = 0; s < P; ++s) fetch(q[s], seg.k_lo + s);
+            for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], u[i], u[i]);  // (1-g)x, one rounding
+        }
 
-    for (int64_t k0 = seg.k_lo; k0 < seg.k_hi; k0 += P) {
+        // the chunk as one step: h_out = a*h_in + b
+        float a = g[0], b = u[0];
+#pragma unroll
+        for (int i = 1; i < E; ++i) {
+            b = __builtin_fmaf(g[i], b, u[i]);
+            a *= g[i];
+        }
+        wave_scan_inclusive(a, b);
+        const float ea = dpp<kWaveShr1>(1.0f, a);  // composition of the chunks before this lane
+        const float eb = dpp<kWaveShr1>(0.0f, b);
+        const float ta = lane63(a), tb = lane63(b);
+
+        float cin = carry;
+        if constexpr (W > 1) {
+            combine_waves<W>(slots, (int)(k & 1), w, lane, ta, tb, cin, carry);
+        } else {
+            carry = __builtin_fmaf(ta, carry, tb);
+        }
+
+        float h = __builtin_fmaf(ea, cin, eb);
+        float o[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+            h = __builtin_fmaf(g[i], h, u[i]);
+            o[i] = h;
+        }
+        if constexpr (decltype(whole)::value) store16<T>(orow + t0, Elem<T>::pack(o));
+        else store_chunk<T, VEC>(orow, t0, L, Elem<T>::pack(o));
+    };
+
+    // The steady part of the row runs without a single conditional memory operation:
+    // only then can the hardware counter tell how many newer loads are in flight when
+    // a tile is needed, and the wave really runs P tiles ahead. It covers the tiles whose
+    // prefetch target is still a whole tile; the rest of the row takes the checked path.
+    Entry q[P];
+    const int64_t count = seg.k_hi - seg.k_lo;
+    const int64_t nwhole = k_whole - seg.k_lo;  // whole tiles at the start of the segment
+    int64_t n = 0;
+    if (nwhole >= 2 * P) {
+#pragma unroll
+        for (int s = 0; s < P; ++s) fetch_whole(q[s], seg.k_lo + s);
+        for (; n + 2 * P <= nwhole; n += P) {
+#pragma unroll
+            for (int s = 0; s < P; ++s) {
+                const int64_t k = seg.k_lo + n + s;
+                const Entry cur = q[s];
+                fetch_whole(q[s], k + P);
+                scan_tile(cur, k, std::true_type{});
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < P; ++s) fetch(q[s], seg.k_lo + s);
+    }
+    for (; n < count; n += P) {
 #pragma unroll
         for (int s = 0; s < P; ++s) {
-            const int64_t k = k0 + s;
-            if (k >= seg.k_hi) break;
+            if (n + s >= count) break;
+            const int64_t k = seg.k_lo + n + s;
             const Entry cur = q[s];
             fetch(q[s], k + P);
-            const int64_t t0 = k * TILE + lane_off;
-
-            float g[E], u[E];
-            Elem<T>::unpack(cur.g, g);
-            Elem<T>::unpack(cur.x, u);
-            if constexpr (!PLAIN) {
-#pragma unroll
-                for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], u[i], u[i]);  // (1-g)x, one rounding
-            }
-
-            // the chunk as one step: h_out = a*h_in + b
-            float a = g[0], b = u[0];
-#pragma unroll
-            for (int i = 1; i < E; ++i) {
-                b = __builtin_fmaf(g[i], b, u[i]);
-                a *= g[i];
-            }
-            wave_scan_inclusive(a, b);
-            const float ea = dpp<kWaveShr1>(1.0f, a);  // composition of the chunks before this lane
-            const float eb = dpp<kWaveShr1>(0.0f, b);
-            const float ta = lane63(a), tb = lane63(b);
-
-            float cin = carry;
-            if constexpr (W > 1) {
-                combine_waves<W>(slots, (int)(k & 1), w, lane, ta, tb, cin, carry);
-            } else {
-                carry = __builtin_fmaf(ta, carry, tb);
-            }
-
-            float h = __builtin_fmaf(ea, cin, eb);
-            float o[E];
-#pragma unroll
-            for (int i = 0; i < E; ++i) {
-                h = __builtin_fmaf(g[i], h, u[i]);
-                o[i] = h;
-            }
-            store_chunk<T, VEC>(orow, t0, L, Elem<T>::pack(o));
+            scan_tile(cur, k, std::false_type{});
         }
     }
 }
@@ -197,7 +241,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
     constexpr int E = Elem<T>::E;
     constexpr int64_t TILE = (int64_t)E * 64 * W;
     const int lane = threadIdx.x & 63;
-    const int wave = uniform(threadIdx.x >> 6);
+    const int wave = uniform((int)(threadIdx.x >> 6));
     const int w = wave % W;
     const int64_t slot = (int64_t)blockIdx.x * R + wave / W;
     if (slot >= rows * nseg) return;
@@ -227,79 +271,146 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
         u32x4 g, G, h, x;
         float hb;  // lane 63 only: h just before this wave's part of the tile (h[-1] at t = 0)
     };
+    // tiles in [k_lo, k_whole) lie wholly inside the row
+    const int64_t k_whole = VEC ? L / TILE : 0;
+    // first position of this wave's part of a tile, relative to the tile: what lane 63 owns
+    const int64_t wave_off = (int64_t)(64 * W - 64 - w * 64) * E;
+    // a whole tile that is not the first of the row: no check of any kind
+    auto fetch_whole = [&](Entry& q, int64_t k) {
+        const int64_t t0 = k * TILE + lane_off;
+        q.g = load16<T, FOLD>(grow + t0);
+        q.G = load16<T, true>(Grow + t0);
+        q.h = load16<T, true>(hrow + t0);
+        if constexpr (!PLAIN) q.x = load16<T, FOLD>(xrow + t0);
+        q.hb = Elem<T>::widen(hrow[k * TILE + wave_off - 1]);
+    };
     auto fetch = [&](Entry& q, int64_t k) {
-        // k < k_lo (before the segment): t0 = L, which every bound check below rejects
+        // k < k_lo (before the segment): t0 = L, which every bound check rejects
         const int64_t t0 = k >= seg.k_lo ? k * TILE + lane_off : L;
         q.g = load_chunk<T, VEC, FOLD>(grow, t0, L, Elem<T>::kOnes);
         q.G = load_chunk<T, VEC, true>(Grow, t0, L, 0u);
         q.h = load_chunk<T, VEC, true>(hrow, t0, L, 0u);
         if constexpr (!PLAIN) q.x = load_chunk<T, VEC, FOLD>(xrow, t0, L, 0u);
-        q.hb = hinit;
-        if (lane == 63 && t0 > 0 && t0 < L) q.hb = Elem<T>::widen(hrow[t0 - 1]);
+        // h just before this wave's part of the tile: one address for the whole wave,
+        // always loaded (position 0 stands in where there is nothing before) and replaced by
+        // h[-1] at the start of the row
+        const int64_t tw = k * TILE + wave_off;
+        const bool before = k >= seg.k_lo && tw > 0 && tw < L;
+        const float loaded = Elem<T>::widen(hrow[before ? tw - 1 : 0]);
+        q.hb = before ? loaded : hinit;
     };
 
-    Entry q[P];
+    // One tile: fold, wave scan, meet the other waves, replay with both epilogues, store.
+    // `whole` tiles store without a bound check.
+    auto scan_tile = [&](const Entry& cur, int64_t k, auto whole) {
+        const int64_t t0 = k * TILE + lane_off;
+        float g[E], G[E], h[E], p[E];
+        Elem<T>::unpack(cur.g, g);
+        Elem<T>::unpack(cur.G, G);
+        Elem<T>::unpack(cur.h, h);
 #pragma unroll
-    for (int s = 0; s < P; ++s) fetch(q[s], seg.k_hi - 1 - s);
+        for (int i = 0; i < E; ++i) p[i] = g[i] * G[i];
 
-    for (int64_t k0 = seg.k_hi - 1; k0 >= seg.k_lo; k0 -= P) {
+        // the chunk as one step on the incoming part: c_out = a*c_in + b
+        float a = g[E - 1], b = p[E - 1];
 #pragma unroll
-        for (int s = 0; s < P; ++s) {
-            const int64_t k = k0 - s;
-            if (k < seg.k_lo) break;
-            const Entry cur = q[s];
-            fetch(q[s], k - P);
-            const int64_t t0 = k * TILE + lane_off;
+        for (int i = E - 2; i >= 0; --i) {
+            b = __builtin_fmaf(g[i], b, p[i]);
+            a *= g[i];
+        }
+        wave_scan_inclusive(a, b);
+        const float ea = dpp<kWaveShr1>(1.0f, a);
+        const float eb = dpp<kWaveShr1>(0.0f, b);
+        const float ta = lane63(a), tb = lane63(b);
+        // h at the position before this chunk: last element of the chunk before it
+        // in memory, which the next lane holds; lane 63 takes the look-behind value.
+        const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
 
-            float g[E], G[E], h[E], p[E];
-            Elem<T>::unpack(cur.g, g);
-            Elem<T>::unpack(cur.G, G);
-            Elem<T>::unpack(cur.h, h);
+        float cin = carry;
+        if constexpr (W > 1) {
+            combine_waves<W>(slots, (int)(k & 1), w, lane, ta, tb, cin, carry);
+        } else {
+            carry = __builtin_fmaf(ta, carry, tb);
+        }
+
+        float c = __builtin_fmaf(ea, cin, eb);
+        float dx[E], dg[E];
+        if constexpr (!PLAIN) Elem<T>::unpack(cur.x, dg);  // dg[] starts as x_t
 #pragma unroll
-            for (int i = 0; i < E; ++i) p[i] = g[i] * G[i];
-
-            // the chunk as one step on the incoming part: c_out = a*c_in + b
-            float a = g[E - 1], b = p[E - 1];
-#pragma unroll
-            for (int i = E - 2; i >= 0; --i) {
-                b = __builtin_fmaf(g[i], b, p[i]);
-                a *= g[i];
-            }
-            wave_scan_inclusive(a, b);
-            const float ea = dpp<kWaveShr1>(1.0f, a);
-            const float eb = dpp<kWaveShr1>(0.0f, b);
-            const float ta = lane63(a), tb = lane63(b);
-            // h at the position before this chunk: last element of the chunk before it
-            // in memory, which the next lane holds; lane 63 fetched it (or h[-1]) itself.
-            const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
-
-            float cin = carry;
-            if constexpr (W > 1) {
-                combine_waves<W>(slots, (int)(k & 1), w, lane, ta, tb, cin, carry);
+        for (int i = E - 1; i >= 0; --i) {
+            const float delta = G[i] + c;
+            c = __builtin_fmaf(g[i], c, p[i]);
+            const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
+            if constexpr (PLAIN) {
+                dx[i] = delta;
+                dg[i] = hp * delta;
             } else {
-                carry = __builtin_fmaf(ta, carry, tb);
+                dx[i] = __builtin_fmaf(-g[i], delta, delta);
+                dg[i] = (hp - dg[i]) * delta;
             }
-
-            float c = __builtin_fmaf(ea, cin, eb);
-            float dx[E], dg[E];
-            if constexpr (!PLAIN) Elem<T>::unpack(cur.x, dg);  // dg[] starts as x_t
-#pragma unroll
-            for (int i = E - 1; i >= 0; --i) {
-                const float delta = G[i] + c;
-                c = __builtin_fmaf(g[i], c, p[i]);
-                const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
-                if constexpr (PLAIN) {
-                    dx[i] = delta;
-                    dg[i] = hp * delta;
-                } else {
-                    dx[i] = __builtin_fmaf(-g[i], delta, delta);
-                    dg[i] = (hp - dg[i]) * delta;
-                }
-            }
+        }
+        if constexpr (decltype(whole)::value) {
+            store16<T>(dxrow + t0, Elem<T>::pack(dx));
+            store16<T>(dgrow + t0, Elem<T>::pack(dg));
+        } else {
             store_chunk<T, VEC>(dxrow, t0, L, Elem<T>::pack(dx));
             store_chunk<T, VEC>(dgrow, t0, L, Elem<T>::pack(dg));
         }
+    };
+
+    // Tiles are taken from the end of the segment: n = 0 is tile k_hi - 1. As in the
+    // forward kernel the steady part has no conditional memory operation. It starts after
+    // a first checked group when the last tile of the row is ragged, and ends where the
+    // prefetch target would fall before the segment (or on the first tile of the row,
+    // whose look-behind value is h[-1]).
+    Entry q[P];
+    const int64_t count = seg.k_hi - seg.k_lo;
+    const bool ragged_top = seg.k_hi > k_whole;
+    int64_t n = 0;
+    if (VEC && !ragged_top && count >= 2 * P + 1) {
+#pragma unroll
+        for (int s = 0; s < P; ++s) fetch_whole(q[s], seg.k_hi - 1 - s);
+    } else {
+#pragma unroll
+        for (int s = 0; s < P; ++s) fetch(q[s], seg.k_hi - 1 - s);
+        if (VEC && ragged_top && count >= 3 * P + 1) {  // one checked group, then whole tiles follow
+#pragma unroll
+            for (int s = 0; s < P; ++s) {
+                const int64_t k = seg.k_hi - 1 - s;
+                const Entry cur = q[s];
+                fetch(q[s], k - P);
+                scan_tile(cur, k, std::false_type{});
+            }
+            n = P;
+        } else {
+            n = count;  // marks "no steady part": the checked loop below starts from zero
+        }
     }
+    if (n < count) {
+        // prefetch targets n + P .. n + 2P - 1 must stay above the first tile of the segment
+        for (; n + 2 * P + 1 <= count; n += P) {
+#pragma unroll
+            for (int s = 0; s < P; ++s) {
+                const int64_t k = seg.k_hi - 1 - (n + s);
+                const Entry cur = q[s];
+                fetch_whole(q[s], k - P);
+                scan_tile(cur, k, std::true_type{});
+            }
+        }
+    } else {
+        n = 0;
+    }
+    for (; n < count; n += P) {
+#pragma unroll
+        for (int s = 0; s < P; ++s) {
+            if (n + s >= count) break;
+            const int64_t k = seg.k_hi - 1 - (n + s);
+            const Entry cur = q[s];
+            fetch(q[s], k - P);
+            scan_tile(cur, k, std::false_type{});
+        }
+    }
+
     // what is left after the first step is g_0 * delta_0: the gradient of the state before the row
     if (h0_grad && seg.index == 0 && w == 0 && lane == 0) {
         float v[E] = {carry};
@@ -323,7 +434,7 @@ __global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
     constexpr int E = Elem<T>::E;
     constexpr int64_t TILE = (int64_t)E * 64;
     const int lane = threadIdx.x & 63;
-    const int wave = uniform(threadIdx.x >> 6);
+    const int wave = uniform((int)(threadIdx.x >> 6));
     const int64_t slot = (int64_t)blockIdx.x * R + wave;
     if (slot >= rows * nseg) return;
     const int64_t ntiles = (L + TILE - 1) / TILE;
@@ -430,7 +541,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     float* carries = lds + 2 * DG * TILE;        // [DG][M]
 
     const int lane = threadIdx.x & 63;
-    const int w = uniform(threadIdx.x >> 6);
+    const int w = uniform((int)(threadIdx.x >> 6));
     const int32_t NG = (D + DG - 1) / DG;
     const int64_t b = blockIdx.x / NG;
     const int32_t grp = (int32_t)(blockIdx.x - b * NG);
@@ -459,11 +570,15 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
         e.g = load_chunk<T, true, false>(gates + (b * M + m) * L, t0, L, Elem<T>::kOnes);
         e.G = load_chunk<T, true, true>(out_grad + row * L, t0, L, 0u);
         e.h = load_chunk<T, true, true>(hrow, t0, L, 0u);
-        e.hb = 0.0f;
-        if (lane == 63 && t0 < L) {
-            if (t0 > 0) e.hb = Elem<T>::widen(hrow[t0 - 1]);
-            else if (h0) e.hb = Elem<T>::widen(h0[row]);
-        }
+        // h just before the tile (h[-1] at the start of the row): one address for the whole
+        // wave, always loaded, so that the number of loads in flight is known at compile time
+        const int64_t tw = k * TILE;
+        const bool live = k >= 0 && k < ntiles;
+        const bool before = live && tw > 0;
+        const bool initial = live && tw == 0 && h0 != nullptr;
+        const T* src = before ? hrow + (tw - 1) : (initial ? h0 + row : hrow);
+        const float loaded = Elem<T>::widen(*src);
+        e.hb = (before || initial) ? loaded : 0.0f;
     };
 
     // ring slot i holds tile (chunk * C + i) of the row that is worked on next at that
