@@ -116,11 +116,11 @@ Grid throttled_grid(const void* kern, int64_t slots, int R, unsigned blocks_per_
 // Waves per row, resident blocks per compute unit, prefetch depth and segments per row
 // when the caller leaves the choice to the library. The table comes from sweeps on an
 // MI355X over the benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536
-// in 16-bit types and 8192 x 4096 in float32. What it encodes: a wave per row streams
-// best when there are many rows of moderate length; long rows want several waves side
-// by side so that fewer rows are open at a time; with few rows a block per row keeps
-// every compute unit busy. About two waves per SIMD is where HBM efficiency peaks;
-// more resident rows lower it. With so few rows that even eight waves per row leave
+// in 16-bit types and 8192 x 4096 in float32, forward and backward separately. What it
+// encodes: one or two waves per row stream best when there are many rows of moderate
+// length; long rows want eight waves side by side so that fewer rows are open at a
+// time; with few rows a block per row keeps every compute unit busy. One to two waves
+// per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few rows that even eight waves per row leave
 // compute units idle (fewer than 32 rows), and a workspace to hold the segment pairs,
 // rows are cut into segments (two passes).
 struct Tuning {
@@ -158,37 +158,38 @@ void plan_segments(const Problem& pb, Tuning& t, bool may_split) {
     t.nseg = (int32_t)nseg;
 }
 
-Tuning choose(const Problem& pb, bool may_split) {
+Tuning choose(const Problem& pb, bool backward, bool may_split) {
     Tuning t;
     const int64_t tile1 = (16 / pb.esize) * 64;          // elements one wave covers per tile
     const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;   // tiles per row for one wave
-    unsigned w = pb.waves;
-    if (!w) {
-        if (tiles1 >= 64) w = 4;
-        else if (pb.rows < 16384 && tiles1 >= 8) w = 8;
-        else w = 1;
-        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
-        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
-    }
     // Gates shared by D rows and tokens shared by M rows come from the caches: the kernel
     // then mostly writes (forward) and the limit on concurrent rows no longer applies.
     // Measured on (B, M, D, L) = (32,32,128,2048), (1,32,2048,8192), (2,32,512,16384).
     const bool shared_inputs = pb.M > 1 || pb.D > 1;
-    if (shared_inputs && !pb.waves && pb.rows >= 16384) w = 1;
+    const bool long_rows = tiles1 >= 64, few_rows = pb.rows < 16384 && tiles1 >= 8;
+    unsigned w = pb.waves;
+    if (!w) {
+        if (shared_inputs && pb.rows >= 16384) w = 1;
+        else if (long_rows) w = 8;
+        else if (few_rows) w = 4;
+        else if (tiles1 >= 16) w = backward ? 1 : 2;
+        else w = 1;
+        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
+        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
+    }
     t.waves = w;
     plan_segments(pb, t, may_split);
     w = t.waves;
     const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
-    if (pb.blocks_per_cu) t.blocks_per_cu = pb.blocks_per_cu;
-    else if (shared_inputs) t.blocks_per_cu = 8;
-    else if (w == 1) t.blocks_per_cu = tiles_per_slot >= 16 ? 2 : 4;
-    else if (w == 4) t.blocks_per_cu = 2;
-    else t.blocks_per_cu = 4;
-    if (pb.depth) t.depth = pb.depth;
-    else if (shared_inputs) t.depth = 2;
-    else if (w == 1) t.depth = tiles_per_slot >= 16 ? 3 : 4;
-    else if (w == 4) t.depth = 4;
-    else t.depth = 3;
+    unsigned bpc, depth;
+    if (shared_inputs) { bpc = 8; depth = 2; }
+    else if (w == 8) { bpc = backward ? 2 : 1; depth = 4; }
+    else if (w == 4) { bpc = 4; depth = backward ? 4 : 2; }
+    else if (w == 2) { bpc = 4; depth = 2; }
+    else if (tiles_per_slot >= 16) { bpc = backward ? 1 : 2; depth = 2; }
+    else { bpc = 4; depth = 2; }
+    t.blocks_per_cu = pb.blocks_per_cu ? pb.blocks_per_cu : bpc;
+    t.depth = pb.depth ? pb.depth : depth;
     return t;
 }
 
@@ -198,13 +199,14 @@ size_t pairs_bytes(const Problem& pb, const Tuning& t) {
 
 // Settles the plan for one call: rows are cut only when the workspace can hold the pairs.
 // Returns 0, or FMSCAN_E_WORKSPACE when the caller asked for a cut that does not fit.
-int settle(const Problem& pb, const void* workspace, size_t workspace_bytes, const char* who, Tuning* t) {
-    *t = choose(pb, workspace != nullptr);
+int settle(const Problem& pb, bool backward, const void* workspace, size_t workspace_bytes, const char* who,
+           Tuning* t) {
+    *t = choose(pb, backward, workspace != nullptr);
     if (t->nseg > 1 && (pairs_bytes(pb, *t) > workspace_bytes || ((uintptr_t)workspace & 7u))) {
         if (pb.segments > 1)
             return fail(FMSCAN_E_WORKSPACE, "%s: %u segments per row need an 8-byte aligned workspace of "
                         "%zu bytes (got %zu)", who, pb.segments, pairs_bytes(pb, *t), workspace_bytes);
-        *t = choose(pb, false);
+        *t = choose(pb, backward, false);
     } else if (pb.segments > 1 && !workspace) {
         return fail(FMSCAN_E_WORKSPACE, "%s: %u segments per row need a workspace", who, pb.segments);
     }
@@ -315,7 +317,7 @@ const char* fmscan_last_error(void) { return g_err; }
 size_t fmscan_workspace_bytes(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags) {
     Problem pb;
     if (parse(B, M, D, L, dtype, flags, &pb)) return 0;
-    return pairs_bytes(pb, choose(pb, true));
+    return pairs_bytes(pb, choose(pb, false, true));  // the cut is the same in both directions
 }
 
 int fmscan_forward(const void* gates, const void* tokens, const void* initial_state, void* out,
@@ -336,7 +338,7 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
 
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(tokens) && aligned16(out);
     Tuning tune;
-    if (int rc = settle(pb, workspace, workspace_bytes, "fmscan_forward", &tune)) return rc;
+    if (int rc = settle(pb, false, workspace, workspace_bytes, "fmscan_forward", &tune)) return rc;
     float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
     if (pairs) {
         launch_aggregate<false>(dtype, pb, tune, vec, gates, tokens, pairs, (hipStream_t)stream);
@@ -392,7 +394,7 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
                      aligned16(token_grad_out) && aligned16(cached_output) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_out);
     Tuning tune;
-    if (int rc = settle(pb, workspace, workspace_bytes, "fmscan_backward", &tune)) return rc;
+    if (int rc = settle(pb, true, workspace, workspace_bytes, "fmscan_backward", &tune)) return rc;
     float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
     if (pairs) {
         launch_aggregate<true>(dtype, pb, tune, vec, gates, out_grad, pairs, (hipStream_t)stream);
