@@ -110,6 +110,25 @@ def cpu_baseline(torch, g, x, G, budget_s=12.0):
                       f"{el:.1f} s, C port oracle/fmscan_cpu.c with OpenMP over rows"}
 
 
+def reference_cpu_path(torch, g, x, G):
+    """Config 1 only: the per-timestep PyTorch form (the counterpart of the reference's CPU path,
+    fm/scan/fm_pytorch.py: a Python loop over t, backward by autograd) on the host cores."""
+    from fm.scan.fm_pytorch import fm_scan_pytorch
+
+    gc = g.float().cpu().requires_grad_()
+    xc = x.float().cpu().requires_grad_()
+    Gc = G.float().cpu()
+    t0 = time.perf_counter()
+    states = fm_scan_pytorch(gc, xc)
+    t1 = time.perf_counter()
+    states.backward(Gc)
+    t2 = time.perf_counter()
+    n = states.numel()
+    return {"value": round(36 * n / (t2 - t0) / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "per-timestep torch loop with autograd (fm_amd/scan/fm_pytorch.py)",
+            "elements_per_s": round(n / (t2 - t0), 1), "fwd_s": round(t1 - t0, 3), "bwd_s": round(t2 - t1, 3)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -213,6 +232,8 @@ def main() -> int:
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, g, x, G)
+        if args.workload == "cfg1":
+            result["reference_cpu_path"] = reference_cpu_path(torch, g, x, G)
     print(json.dumps(result), flush=True)
     return 0
 

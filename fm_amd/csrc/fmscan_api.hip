@@ -94,14 +94,16 @@ int launched(const char* what) {
 struct Grid {
     unsigned blocks, lds;
 };
-Grid throttled_grid(const void* kern, int64_t slots, int R, unsigned blocks_per_cu) {
+// `last_set` belongs to one kernel instantiation: (device, bytes) of its last attribute call,
+// so that the attribute is only set again when the cap or the device changes.
+Grid throttled_grid(const void* kern, std::atomic<uint64_t>& last_set, int64_t slots, int R,
+                    unsigned blocks_per_cu) {
     Grid g;
     g.blocks = (unsigned)((slots + R - 1) / R);
     g.lds = ((160u * 1024u - 2048u) / blocks_per_cu) & ~1023u;
-    static std::atomic<uint64_t> last_set{~0ull};  // (kernel, device, bytes) of the last attribute call
     int dev = 0;
     (void)hipGetDevice(&dev);
-    const uint64_t key = ((uint64_t)(uintptr_t)kern << 24) ^ ((uint64_t)dev << 20) ^ g.lds;
+    const uint64_t key = ((uint64_t)dev << 32) | g.lds;
     if (last_set.load(std::memory_order_relaxed) != key) {
         if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds) != hipSuccess) {
             (void)hipGetLastError();
@@ -217,7 +219,8 @@ template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
 void launch_fwd(const Problem& pb, const Tuning& t, const void* g, const void* x, const void* h0,
                 void* out, const float2* pairs, hipStream_t s) {
     auto kern = fmscan::scan_forward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
-    const Grid grid = throttled_grid((const void*)kern, pb.rows * t.nseg, R, t.blocks_per_cu);
+    static std::atomic<uint64_t> last_set{~0ull};
+    const Grid grid = throttled_grid((const void*)kern, last_set, pb.rows * t.nseg, R, t.blocks_per_cu);
     kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>((const T*)g, (const T*)x, (const T*)h0, (T*)out,
                                                    pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L,
                                                    t.nseg, t.seg_tiles, pairs);
@@ -228,7 +231,8 @@ void launch_bwd(const Problem& pb, const Tuning& t, const void* g, const void* G
                 void* dx, const void* h, const void* x, void* dg, const void* h0, void* dh0,
                 const float2* pairs, hipStream_t s) {
     auto kern = fmscan::scan_backward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
-    const Grid grid = throttled_grid((const void*)kern, pb.rows * t.nseg, R, t.blocks_per_cu);
+    static std::atomic<uint64_t> last_set{~0ull};
+    const Grid grid = throttled_grid((const void*)kern, last_set, pb.rows * t.nseg, R, t.blocks_per_cu);
     kern<<<grid.blocks, 64 * W * R, grid.lds, s>>>(
         (const T*)g, (const T*)G, (const T*)fpg, (T*)dx, (const T*)h, (const T*)x, (T*)dg,
         (const T*)h0, (T*)dh0, pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L, t.nseg, t.seg_tiles, pairs);

@@ -48,6 +48,24 @@ def _on_gpu(name: str, t: torch.Tensor, dev: torch.device) -> None:
     _require(t.device == dev, f"{name} is on {t.device}, expected {dev}")
 
 
+class _on_device:
+    """`with torch.cuda.device(dev)` without its cost when `dev` is already current."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev):
+        self.ctx = None if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
 def _flags(plain: bool, waves_per_row: int, blocks_per_cu: int, depth: int, segments: int) -> int:
     return ((_lib.FLAG_PLAIN if plain else 0) | (int(waves_per_row) << _lib.FLAG_WAVES_SHIFT)
             | (int(blocks_per_cu) << _lib.FLAG_BLOCKS_SHIFT) | (int(depth) << _lib.FLAG_DEPTH_SHIFT)
@@ -57,6 +75,8 @@ def _flags(plain: bool, waves_per_row: int, blocks_per_cu: int, depth: int, segm
 def _workspace(B, M, D, L, code, flags, device):
     """Scratch for the carries between the segments of a cut row (few rows, long L);
     None when the library scans every row in one piece."""
+    if B * M * D >= 32 and not (flags >> _lib.FLAG_SEGMENTS_SHIFT):
+        return None, 0  # rows are only cut on request or when there are very few of them
     need = module.fmscan_workspace_bytes(B, M, D, L, code, flags)
     if not need:
         return None, 0
@@ -87,7 +107,7 @@ def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per
     if out.numel() == 0:
         return out
     flags = _flags(plain, waves_per_row, blocks_per_cu, depth, segments)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         ws, ws_bytes = _workspace(B, M, D, L, code, flags, dev)
         _lib.check(module.fmscan_forward(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
@@ -136,7 +156,7 @@ def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output,
     if cached_output.numel() == 0:
         return None
     flags = _flags(plain, waves_per_row, blocks_per_cu, depth, segments)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         ws, ws_bytes = _workspace(B, M, D, L, code, flags, dev)
         _lib.check(module.fmscan_backward(
@@ -188,7 +208,7 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
     d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
     partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
     if cached_output.numel():
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(module.fmscan_backward_reduced(
                 gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), d_tokens.data_ptr(),
