@@ -175,6 +175,7 @@ Tuning choose(const Problem& pb, bool backward, bool may_split) {
         else if (long_rows) w = 8;
         else if (few_rows) w = 4;
         else if (tiles1 >= 16) w = backward ? 1 : 2;
+        else if (tiles1 >= 8) w = backward ? 2 : 1;
         else w = 1;
         while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
         while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
@@ -189,6 +190,7 @@ Tuning choose(const Problem& pb, bool backward, bool may_split) {
     else if (w == 4) { bpc = 4; depth = backward ? 4 : 2; }
     else if (w == 2) { bpc = 4; depth = 2; }
     else if (tiles_per_slot >= 16) { bpc = backward ? 1 : 2; depth = 2; }
+    else if (tiles_per_slot >= 8) { bpc = 2; depth = 2; }
     else { bpc = 4; depth = 2; }
     t.blocks_per_cu = pb.blocks_per_cu ? pb.blocks_per_cu : bpc;
     t.depth = pb.depth ? pb.depth : depth;

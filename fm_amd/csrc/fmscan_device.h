@@ -166,8 +166,6 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ row, int64_t t0, int
 // DPP lane permutes (data-parallel primitives: the permute happens in the VALU
 // operand path, no LDS traffic). A lane whose source lane does not exist, or
 // that the row mask switches off, receives `old`.
-constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
-constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
 constexpr int kWaveShl1 = 0x130;  // lane i <- lane i+1
 constexpr int kWaveShr1 = 0x138;  // lane i <- lane i-1
 
@@ -182,21 +180,36 @@ __device__ __forceinline__ float dpp(float old, float v) {
 // On entry lane l holds the pair of its own chunk; on exit it holds the
 // composition of chunks 0..l: four shifted steps inside each 16-lane row, then
 // the row totals are broadcast into rows 1,3 and finally into rows 2,3.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ void scan_step(float& a, float& b) {
-    const float pa = dpp<CTRL, ROW_MASK>(1.0f, a);
-    const float pb = dpp<CTRL, ROW_MASK>(0.0f, b);
-    b = __builtin_fmaf(pb, a, b);
-    a = pa * a;
-}
-
+// One wave scan = six steps; each is two VALU instructions that take their first source
+// through DPP: b += b[src] * a, then a *= a[src]. A lane whose source lane does not
+// exist or whose row is masked off is left untouched, which is exactly "combine only if
+// there is something to the left" (the `laneId >= delta` test at reference
+// fm/scan/fm_scan.cuh:138). Written as one asm block because the compiler keeps the
+// permute as a separate move with an explicit identity (three times the instructions).
+// s_nop: a VGPR written by a VALU instruction may be read through DPP two wait states
+// later at the earliest; inside the block the instruction in between provides one.
 __device__ __forceinline__ void wave_scan_inclusive(float& a, float& b) {
-    scan_step<kRowShr1, 0xf>(a, b);
-    scan_step<kRowShr2, 0xf>(a, b);
-    scan_step<kRowShr4, 0xf>(a, b);
-    scan_step<kRowShr8, 0xf>(a, b);
-    scan_step<kRowBcast15, 0xa>(a, b);
-    scan_step<kRowBcast31, 0xc>(a, b);
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "+v"(b));
 }
 
 __device__ __forceinline__ float lane63(float v) {
