@@ -310,7 +310,8 @@ void launch_aggregate(int dtype, const Problem& pb, const Tuning& t, bool vec, c
 }
 
 constexpr int kReducedGroup = 8;  // consecutive d one block of the reduced backward kernel sums over
-constexpr int kReducedChunk = 1;  // tiles of a row visited before moving to the next m (1 measured best)
+constexpr int kReducedChunk = 4;  // tiles of a row visited before moving to the next m
+constexpr int kReducedDepth = 1;  // visits whose loads are in flight ahead of the one worked on
 
 }  // namespace
 
@@ -467,12 +468,14 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
     if (lds > 160u * 1024u)
         return fail(FMSCAN_E_SHAPE, "fmscan_backward_reduced: M = %lld needs %zu bytes of LDS (limit 163840); "
                     "use fmscan_backward", (long long)M, lds);
+    if ((L + (int64_t)tile - 1) / (int64_t)tile + kReducedChunk > INT32_MAX / M)
+        return fail(FMSCAN_E_SHAPE, "fmscan_backward_reduced: M * ceil(L / %zu) must be < 2^31", tile);
     const void* h_init = initial_state ? initial_state : first_prop_grad;
     const unsigned grid = (unsigned)(B * groups);
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
         auto go = [&](auto pt) {
-            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, kReducedChunk, decltype(pt)::value>;
+            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, kReducedChunk, kReducedDepth, decltype(pt)::value>;
             if (lds > 48u * 1024u)
                 (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             kern<<<grid, 64 * kReducedGroup, lds, (hipStream_t)stream>>>(

@@ -512,21 +512,22 @@ __global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
 // (B, M, D, L) tensors "to avoid atomicAdd", fm_scan.cuh:200-207, and torch.sum reads them
 // back). This kernel never writes them. A block is one batch element b and DG
 // consecutive d (one wave each). Its waves walk their rows from the end in chunks of C
-// tiles; inside a chunk they visit the M rows (b, m, d) one after the other and, for each,
-// the C tiles of the chunk, all waves on the same (chunk, m, tile) step:
+// tiles; for a chunk they visit the M rows (b, m, d) one after the other and, in each, the
+// C tiles of the chunk from the last to the first, all waves on the same step:
 //   * token gradient: summed over m in registers (C tiles of accumulators), stored once
 //     per chunk as d_tokens[b, d, :]
 //   * gate gradient: the DG waves add their tiles up in LDS (one barrier per step) and
 //     store the sum for this group of d, gate_partial[b, m, group, :] in float32; the
 //     caller adds the ceil(D / DG) groups.
-// Each wave keeps the running state of its M rows in LDS (one float per row); the loads
-// of the same tile position of the next row are in flight while a tile is worked on.
+// Each wave keeps the running state of its M rows in LDS (one float per row). The visits
+// (chunk, m) form one linear sequence; a ring holds the loads of the next R visits, and
+// every step issues the same loads whatever its position (addresses are clamped into
+// the row), so the number of loads in flight is known at compile time and a step waits
+// for its own entry only. A larger C makes the pieces a wave reads from one row longer
+// (C KiB at a time), which the memory likes, at C tiles of accumulators.
 // HBM traffic: G and h once (2s per element) plus 4/DG bytes per element of partials,
-// against 6s for the unfused kernel plus the two torch.sum passes. With a third of the
-// bytes per element the arithmetic (about 20 VALU operations per element) weighs as
-// much as the memory here: measured 2.5-4.3 TB/s of G + h, 1.2-2.3x faster end to end
-// than the two-tensor route; C = 1 measured best.
-template <typename T, int DG, int C, bool PLAIN>
+// against 6s for the unfused kernel plus the two torch.sum passes.
+template <typename T, int DG, int C, int R, bool PLAIN>
 __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved,
@@ -535,6 +536,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     constexpr int SLICE = TILE / DG;  // elements of a summed tile each wave adds up and stores
+    constexpr bool HOIST = C <= 2;    // keep the chunk's tokens widened across its M rows
     static_assert(TILE % DG == 0, "a tile must split evenly over the waves");
     extern __shared__ float lds[];
     float* red = lds;                            // [2][DG][TILE]
@@ -543,12 +545,15 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const int lane = threadIdx.x & 63;
     const int w = uniform((int)(threadIdx.x >> 6));
     const int32_t NG = (D + DG - 1) / DG;
-    const int64_t b = blockIdx.x / NG;
-    const int32_t grp = (int32_t)(blockIdx.x - b * NG);
+    // (the division runs on the vector unit; everything derived from b is an address, so
+    // bring it back to a scalar register)
+    const int32_t b32 = uniform((int)(blockIdx.x / (uint32_t)NG));
+    const int64_t b = b32;
+    const int32_t grp = (int32_t)blockIdx.x - b32 * NG;
     const bool active = grp * DG + w < D;        // a wave past the last d still joins every barrier
     const int64_t d = active ? grp * DG + w : D - 1;
-    const int64_t ntiles = (L + TILE - 1) / TILE;
-    const int64_t nchunks = (ntiles + C - 1) / C;
+    const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
+    const int32_t nchunks = (ntiles + C - 1) / C;
     const int64_t lane_off = (int64_t)(63 - lane) * E;
     float* mycarry = carries + w * M;
 
@@ -558,73 +563,114 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const T* __restrict__ xrow = tokens + (b * D + d) * L;  // never read when PLAIN
     T* __restrict__ dxrow = token_grad + (b * D + d) * L;
 
+    // What a step loads, exactly as it arrives: anything computed from a loaded value at
+    // the time of the load would have to be finished before the loop comes round, which
+    // means waiting for every load in flight. Fill values for chunks beyond L and the
+    // choice of h[-1] are therefore applied when the entry is used.
     struct Entry {
-        u32x4 g, G, h;
-        float hb;
+        u32x4 g, G, h, x;
+        T hb;
     };
-    // tile k of row (b, m, d); k outside [0, ntiles) loads nothing
-    auto fetch = [&](Entry& e, int64_t k, int32_t m) {
-        const int64_t row = (b * M + m) * D + d;
-        const int64_t t0 = (k >= 0 && k < ntiles) ? k * TILE + lane_off : L;
-        const T* __restrict__ hrow = h_saved + row * L;
-        e.g = load_chunk<T, true, false>(gates + (b * M + m) * L, t0, L, Elem<T>::kOnes);
-        e.G = load_chunk<T, true, true>(out_grad + row * L, t0, L, 0u);
-        e.h = load_chunk<T, true, true>(hrow, t0, L, 0u);
-        // h just before the tile (h[-1] at the start of the row): one address for the whole
-        // wave, always loaded, so that the number of loads in flight is known at compile time
-        const int64_t tw = k * TILE;
-        const bool live = k >= 0 && k < ntiles;
-        const bool before = live && tw > 0;
-        const bool initial = live && tw == 0 && h0 != nullptr;
-        const T* src = before ? hrow + (tw - 1) : (initial ? h0 + row : hrow);
-        const float loaded = Elem<T>::widen(*src);
-        e.hb = (before || initial) ? loaded : 0.0f;
+    // Where a visit is: chunk `chunk` of row (b, m, d), with the offsets that go with it
+    // kept as running sums in scalar registers (a 64-bit product per step would run on the
+    // vector unit, at a quarter of the rate).
+    struct Cursor {
+        int32_t chunk, m;
+        int64_t row;   // (b * M + m) * D + d
+        int64_t hoff;  // row * L: where the row starts in out_grad and h
+        int64_t goff;  // (b * M + m) * L: in gates
+        int64_t poff;  // ((b * M + m) * NG + grp) * L: in gate_partial
+    };
+    const int64_t row_step = D, hoff_step = (int64_t)D * L, goff_step = L, poff_step = (int64_t)NG * L;
+    // the visit after: the next row at the same chunk, then row 0 of the chunk before
+    auto advance = [&](Cursor& c) {
+        const bool wrap = c.m + 1 == M;
+        c.chunk = wrap ? c.chunk - 1 : c.chunk;
+        c.m = wrap ? 0 : c.m + 1;
+        c.row = uniform64(wrap ? c.row - (M - 1) * row_step : c.row + row_step);
+        c.hoff = uniform64(wrap ? c.hoff - (M - 1) * hoff_step : c.hoff + hoff_step);
+        c.goff = uniform64(wrap ? c.goff - (M - 1) * goff_step : c.goff + goff_step);
+        c.poff = uniform64(wrap ? c.poff - (M - 1) * poff_step : c.poff + poff_step);
+    };
+    const int32_t lane_off32 = (63 - lane) * E;
+    // tile i of the chunk; addresses are clamped into the row (a chunk before the first, or
+    // a tile past the last, reads the nearest tile of the row)
+    auto fetch = [&](Entry& e, const Cursor& c, int i) {
+        int32_t k = c.chunk * C + i;
+        k = k < 0 ? 0 : (k > ntiles - 1 ? ntiles - 1 : k);
+        const int64_t tw = (int64_t)k * TILE;
+        const int64_t left = L - tw;
+        const int32_t rem = left < TILE ? (int32_t)left : TILE;
+        const uint32_t loff = (uint32_t)(lane_off32 < rem ? lane_off32 : rem - E) * (uint32_t)sizeof(T);
+        auto at = [&](const T* base) {  // scalar base + 32-bit lane offset
+            return reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + loff);
+        };
+        const T* __restrict__ hrow = h_saved + c.hoff;
+        e.g = load16<T, false>(at(gates + c.goff + tw));
+        e.G = load16<T, true>(at(out_grad + c.hoff + tw));
+        e.h = load16<T, true>(at(hrow + tw));
+        e.x = u32x4{0u, 0u, 0u, 0u};
+        if constexpr (!PLAIN) e.x = load16<T, false>(at(xrow + tw));
+        // h just before the tile (h[-1] at the start of the row): one address for the whole wave
+        const T* src = tw > 0 ? hrow + (tw - 1) : (h0 != nullptr ? h0 + c.row : hrow);
+        e.hb = *src;
     };
 
-    // ring slot i holds tile (chunk * C + i) of the row that is worked on next at that
-    // position: slot i is refilled, right after use, with the same position of row m + 1
-    // (or of row 0 of the chunk before)
-    Entry q[C];
-    u32x4 x_raw[C], x_next[C];
+    Entry q[R][C];
+    Cursor ahead = {nchunks - 1, 0, uniform64(b * M * D + d), uniform64((b * M * D + d) * L),
+                    uniform64(b * M * L), uniform64((b * M * NG + grp) * L)};
+    Cursor at = ahead;
 #pragma unroll
-    for (int i = 0; i < C; ++i) {
-        const int64_t k = (nchunks - 1) * C + i;
-        fetch(q[i], k, 0);
-        x_raw[i] = u32x4{0u, 0u, 0u, 0u};
-        x_next[i] = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (!PLAIN) x_next[i] = load_chunk<T, true, false>(xrow, k < ntiles ? k * TILE + lane_off : L, L, 0u);
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int i = C - 1; i >= 0; --i) fetch(q[r][i], ahead, i);
+        advance(ahead);
     }
 
     __syncthreads();  // carries are in place
 
+    float dtok[C][E], xf[HOIST ? C : 1][E];
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) dtok[i][j] = 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < (HOIST ? C : 1); ++i) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) xf[i][j] = 0.0f;
+    }
     int parity = 0;
-    for (int64_t chunk = nchunks - 1; chunk >= 0; --chunk) {
-        float dtok[C][E];
+    const int32_t visits = nchunks * M;  // the host checks that this fits
+    for (int32_t n = 0; n < visits; n += R) {
 #pragma unroll
-        for (int i = 0; i < C; ++i) {
-#pragma unroll
-            for (int j = 0; j < E; ++j) dtok[i][j] = 0.0f;
-            if constexpr (!PLAIN) {  // this chunk's token tiles; fetch the ones of the chunk before
-                x_raw[i] = x_next[i];
-                const int64_t kp = (chunk - 1) * C + i;
-                x_next[i] = load_chunk<T, true, false>(xrow, chunk > 0 ? kp * TILE + lane_off : L, L, 0u);
-            }
-        }
-        for (int32_t m = 0; m < M; ++m) {
+        for (int r = 0; r < R; ++r) {
+            if (n + r >= visits) break;  // same for every wave of the block
+            const int32_t m = at.m;
             float carry = mycarry[m];
 #pragma unroll
             for (int i = C - 1; i >= 0; --i) {
-                const int64_t k = chunk * C + i;
-                const Entry cur = q[i];
-                if (m + 1 < M) fetch(q[i], k, m + 1);
-                else fetch(q[i], k - C, 0);
-                if (k >= ntiles) continue;  // the last chunk of a row may be short (same for every wave)
-                const int64_t t0 = k * TILE + lane_off;
+                Entry cur = q[r][i];
+                fetch(q[r][i], ahead, i);
 
-                float g[E], G[E], h[E], p[E];
+                const int32_t k = at.chunk * C + i;  // may be past the last tile in the last chunk
+                const int64_t tw = (int64_t)k * TILE;
+                if (tw + TILE > L && tw + lane_off >= L) {  // short or absent tile: nothing there
+                    cur.g = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
+                    cur.G = cur.h = cur.x = u32x4{0u, 0u, 0u, 0u};
+                }
+                const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(cur.hb) : 0.0f;
+                float g[E], G[E], h[E], p[E], xs[E];
                 Elem<T>::unpack(cur.g, g);
                 Elem<T>::unpack(cur.G, G);
                 Elem<T>::unpack(cur.h, h);
+                if constexpr (!PLAIN) {
+                    if constexpr (HOIST) {
+                        if (m == 0) Elem<T>::unpack(cur.x, xf[i]);  // the M rows share their tokens
+                    } else {
+                        Elem<T>::unpack(cur.x, xs);
+                    }
+                }
 #pragma unroll
                 for (int j = 0; j < E; ++j) p[j] = g[j] * G[j];
                 float a = g[E - 1], bb = p[E - 1];
@@ -637,12 +683,11 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                 const float ea = dpp<kWaveShr1>(1.0f, a);
                 const float eb = dpp<kWaveShr1>(0.0f, bb);
                 const float ta = lane63(a), tb = lane63(bb);
-                const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
+                const float hprev0 = dpp<kWaveShl1>(hb, h[E - 1]);
 
                 float c = __builtin_fmaf(ea, carry, eb);
                 carry = __builtin_fmaf(ta, carry, tb);
                 float dg[E];
-                if constexpr (!PLAIN) Elem<T>::unpack(x_raw[i], dg);  // dg[] starts as x_t
 #pragma unroll
                 for (int j = E - 1; j >= 0; --j) {
                     const float delta = G[j] + c;
@@ -653,9 +698,13 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                         dg[j] = hp * delta;
                     } else {
                         dtok[i][j] += __builtin_fmaf(-g[j], delta, delta);
-                        dg[j] = (hp - dg[j]) * delta;
+                        const float x = HOIST ? xf[HOIST ? i : 0][j] : xs[j];
+                        dg[j] = (hp - x) * delta;
                     }
-                    if (!active) dg[j] = 0.0f;
+                }
+                if (!active) {  // whole wave: a wave past the last d adds nothing
+#pragma unroll
+                    for (int j = 0; j < E; ++j) dg[j] = 0.0f;
                 }
 
                 // add the gate gradient tiles of the DG waves: each wave lays its tile out in
@@ -666,21 +715,28 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                     *reinterpret_cast<float4*>(mine + j) = make_float4(dg[j], dg[j + 1], dg[j + 2], dg[j + 3]);
                 __syncthreads();
                 const float* all = red + parity * DG * TILE + w * SLICE;
-                float* __restrict__ prow = gate_partial + ((b * M + m) * NG + grp) * L + k * TILE + w * SLICE;
+                float* __restrict__ prow = gate_partial + at.poff + tw + w * SLICE;
                 for (int e = lane; e < SLICE; e += 64) {
                     float sum = 0.0f;
 #pragma unroll
                     for (int v = 0; v < DG; ++v) sum += all[v * TILE + e];
-                    if (k * TILE + w * SLICE + e < L) __builtin_nontemporal_store(sum, prow + e);
+                    if (tw + w * SLICE + e < L) __builtin_nontemporal_store(sum, prow + e);
                 }
                 parity ^= 1;
             }
             if (lane == 0) mycarry[m] = carry;
-        }
-        if (active) {
+
+            if (m + 1 == M) {  // the chunk's token gradient is complete
 #pragma unroll
-            for (int i = 0; i < C; ++i)
-                store_chunk<T, true>(dxrow, (chunk * C + i) * TILE + lane_off, L, Elem<T>::pack(dtok[i]));
+                for (int i = 0; i < C; ++i) {
+                    const int64_t t0 = (int64_t)(at.chunk * C + i) * TILE + lane_off;
+                    if (active) store_chunk<T, true>(dxrow, t0, L, Elem<T>::pack(dtok[i]));
+#pragma unroll
+                    for (int j = 0; j < E; ++j) dtok[i][j] = 0.0f;
+                }
+            }
+            advance(at);
+            advance(ahead);
         }
     }
 

@@ -360,7 +360,7 @@ def test_backward_with_sums_inside(scan, dtype, plain):
     """fm_scan_backward_reduced (d_gates, d_tokens straight from one kernel) against the
     float64 oracle's summed gradients, and against the two-tensor path plus torch.sum."""
     for (B, M, D, L) in [(2, 3, 5, 512), (1, 2, 2, 8), (2, 4, 8, 4096), (1, 33, 17, 1000 // 8 * 8),
-                         (3, 2, 9, 2048), (1, 70, 3, 640)]:
+                         (3, 2, 9, 2048), (1, 70, 3, 640), (2, 3, 4, 2568)]:
         gen = torch.Generator().manual_seed(M * 100 + D)
         g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
         x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
