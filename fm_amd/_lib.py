@@ -7,11 +7,11 @@ on a GPU are rejected.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_uint, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint, c_void_p
 
 from . import build as _build
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 FLAG_PLAIN = 0x1
@@ -50,6 +50,15 @@ def load() -> ctypes.CDLL:
     lib.fmscan_reduced_groups.argtypes = [c_int64]
     lib.fmscan_backward_reduced.restype = c_int
     lib.fmscan_backward_reduced.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
+    dims = [c_int64] * 4
+    lib.fmscan_readout_inv_rms.restype = c_int
+    lib.fmscan_readout_inv_rms.argtypes = [c_void_p] * 2 + dims + [c_int, c_float, c_void_p]
+    lib.fmscan_readout_forward.restype = c_int
+    lib.fmscan_readout_forward.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
+    lib.fmscan_readout_dot.restype = c_int
+    lib.fmscan_readout_dot.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
+    lib.fmscan_readout_backward.restype = c_int
+    lib.fmscan_readout_backward.argtypes = [c_void_p] * 8 + dims + [c_int, c_void_p]
     got = lib.fmscan_abi_version()
     if got != ABI_VERSION:
         raise RuntimeError(f"libfmscan_hip.so has ABI version {got}, this package needs {ABI_VERSION}; "

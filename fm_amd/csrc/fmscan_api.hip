@@ -9,6 +9,7 @@
 #include <cstdio>
 
 #include "fmscan_kernels.h"
+#include "fmscan_readout.h"
 
 namespace {
 
@@ -487,6 +488,185 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
         else go(BoolTag<false>{});
     });
     return launched("backward (reduced)");
+}
+
+}  // extern "C"
+
+// ---- read-out of the Factorization-Memory layer -----------------------------------------
+
+namespace {
+
+constexpr int kRowDotWaves = 8;  // waves of a block that share the D rows of a slot
+constexpr int kReadoutRows = 4;  // consecutive d per wave in the read-out kernels
+
+struct ReadoutShape {
+    int64_t B, M, D, L;
+    int esize;
+    int32_t tiles;
+};
+
+int parse_readout(const char* who, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, ReadoutShape* rs) {
+    Problem pb;
+    if (int rc = parse(B, M, D, L, dtype, 0, &pb)) return rc;
+    const int64_t tile = (16 / pb.esize) * 64;
+    const int64_t tiles = (L + tile - 1) / tile;
+    if (D >= (1 << 20) || (__int128)B * M * tiles > (__int128)INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: D must be < 2^20 and B * M * ceil(L / %lld) < 2^31", who, (long long)tile);
+    rs->B = B; rs->M = M; rs->D = D; rs->L = L;
+    rs->esize = pb.esize;
+    rs->tiles = (int32_t)tiles;
+    return 0;
+}
+
+bool vector_path(const ReadoutShape& rs, std::initializer_list<const void*> pointers) {
+    if ((rs.L * rs.esize) % 16 != 0) return false;
+    for (const void* p : pointers)
+        if (p && !aligned16(p)) return false;
+    return true;
+}
+
+template <typename F>
+void with_bool(bool v, F&& f) {
+    if (v) f(BoolTag<true>{});
+    else f(BoolTag<false>{});
+}
+
+}  // namespace
+
+extern "C" {
+
+int fmscan_readout_inv_rms(const void* states, float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L,
+                           int dtype, float eps, void* stream) {
+    ReadoutShape rs;
+    if (int rc = parse_readout("fmscan_readout_inv_rms", B, M, D, L, dtype, &rs)) return rc;
+    if (!states || !inv_rms) return fail(FMSCAN_E_NULL, "fmscan_readout_inv_rms: states and inv_rms must not be NULL");
+    if (!(eps >= 0.0f)) return fail(FMSCAN_E_SHAPE, "fmscan_readout_inv_rms: eps must be >= 0");
+    if (overlap({"inv_rms", inv_rms, B * M * L * 4}, {"states", states, B * M * D * L * rs.esize}))
+        return fail(FMSCAN_E_ALIAS, "fmscan_readout_inv_rms: inv_rms overlaps states");
+    const bool vec = vector_path(rs, {states});
+    const unsigned grid = (unsigned)(B * M * rs.tiles);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        with_bool(vec, [&](auto vt) {
+            fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kSumSq, false, decltype(vt)::value>
+                <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>((const T*)states, nullptr, nullptr, inv_rms,
+                                                                      nullptr, (int32_t)M, (int32_t)D, L,
+                                                                      rs.tiles, eps);
+        });
+    });
+    return launched("read-out (inverse rms)");
+}
+
+int fmscan_readout_forward(const void* states, const float* inv_rms, const void* read, void* states_out,
+                           void* output, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
+    ReadoutShape rs;
+    if (int rc = parse_readout("fmscan_readout_forward", B, M, D, L, dtype, &rs)) return rc;
+    if (!states || !read || !output)
+        return fail(FMSCAN_E_NULL, "fmscan_readout_forward: states, read and output must not be NULL");
+    if (inv_rms && !states_out)
+        return fail(FMSCAN_E_NULL, "fmscan_readout_forward: states_out must not be NULL with inv_rms");
+    const int64_t full = B * M * D * L * rs.esize;
+    const Range out_r = {"output", output, B * D * L * rs.esize};
+    const Range sn_r = {"states_out", inv_rms ? states_out : nullptr, full};
+    const Range ins[] = {{"states", states, full}, {"inv_rms", inv_rms, B * M * L * 4},
+                         {"read", read, B * M * L * rs.esize}};
+    for (const Range& in : ins) {
+        if (overlap(out_r, in)) return fail(FMSCAN_E_ALIAS, "fmscan_readout_forward: output overlaps %s", in.name);
+        // states_out == states (in place) is allowed: every element is read before it is written
+        if (overlap(sn_r, in) && !(in.p == states && states_out == states))
+            return fail(FMSCAN_E_ALIAS, "fmscan_readout_forward: states_out overlaps %s", in.name);
+    }
+    if (overlap(out_r, sn_r)) return fail(FMSCAN_E_ALIAS, "fmscan_readout_forward: output overlaps states_out");
+    const bool vec = vector_path(rs, {states, inv_rms, read, inv_rms ? states_out : nullptr, output});
+    const dim3 grid((unsigned)(B * rs.tiles), (unsigned)((D + 4 * kReadoutRows - 1) / (4 * kReadoutRows)));
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        with_bool(inv_rms != nullptr, [&](auto nt) {
+            with_bool(vec, [&](auto vt) {
+                fmscan::readout_forward_kernel<T, kReadoutRows, decltype(nt)::value, decltype(vt)::value>
+                    <<<grid, 256, 0, (hipStream_t)stream>>>((const T*)states, inv_rms, (const T*)read,
+                                                            (T*)states_out, (T*)output, (int32_t)M, (int32_t)D,
+                                                            L, rs.tiles);
+            });
+        });
+    });
+    return launched("read-out (forward)");
+}
+
+int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad, float* q, float* qe,
+                       int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
+    ReadoutShape rs;
+    if (int rc = parse_readout("fmscan_readout_dot", B, M, D, L, dtype, &rs)) return rc;
+    if (!states_n || !out_grad || !q)
+        return fail(FMSCAN_E_NULL, "fmscan_readout_dot: states_n, out_grad and q must not be NULL");
+    if (ext_grad && !qe) return fail(FMSCAN_E_NULL, "fmscan_readout_dot: qe must not be NULL with ext_grad");
+    const int64_t full = B * M * D * L * rs.esize;
+    const Range outs[] = {{"q", q, B * M * L * 4}, {"qe", ext_grad ? qe : nullptr, B * M * L * 4}};
+    const Range ins[] = {{"states_n", states_n, full}, {"out_grad", out_grad, B * D * L * rs.esize},
+                         {"ext_grad", ext_grad, full}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", o.name, in.name);
+    if (overlap(outs[0], outs[1])) return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: q overlaps qe");
+    const bool vec = vector_path(rs, {states_n, out_grad, ext_grad});
+    const unsigned grid = (unsigned)(B * M * rs.tiles);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        with_bool(ext_grad != nullptr, [&](auto et) {
+            with_bool(vec, [&](auto vt) {
+                fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kDot, decltype(et)::value, decltype(vt)::value>
+                    <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>((const T*)states_n, (const T*)out_grad,
+                                                                          (const T*)ext_grad, q, qe, (int32_t)M,
+                                                                          (int32_t)D, L, rs.tiles, 0.0f);
+            });
+        });
+    });
+    return launched("read-out (dot)");
+}
+
+int fmscan_readout_backward(const void* states_n, const float* inv_rms, const void* read, const void* out_grad,
+                            const void* ext_grad, const float* q, const float* qe, void* state_grad, int64_t B,
+                            int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
+    ReadoutShape rs;
+    if (int rc = parse_readout("fmscan_readout_backward", B, M, D, L, dtype, &rs)) return rc;
+    if (!read || !out_grad || !state_grad)
+        return fail(FMSCAN_E_NULL, "fmscan_readout_backward: read, out_grad and state_grad must not be NULL");
+    const bool norm = inv_rms != nullptr;
+    if (norm && (!states_n || !q))
+        return fail(FMSCAN_E_NULL, "fmscan_readout_backward: states_n and q must not be NULL with inv_rms");
+    if (norm && ext_grad && !qe)
+        return fail(FMSCAN_E_NULL, "fmscan_readout_backward: qe must not be NULL with inv_rms and ext_grad");
+    const int64_t full = B * M * D * L * rs.esize;
+    const Range out_r = {"state_grad", state_grad, full};
+    const Range ins[] = {{"states_n", norm ? states_n : nullptr, full}, {"inv_rms", inv_rms, B * M * L * 4},
+                         {"read", read, B * M * L * rs.esize}, {"out_grad", out_grad, B * D * L * rs.esize},
+                         {"ext_grad", ext_grad, full}, {"q", norm ? q : nullptr, B * M * L * 4},
+                         {"qe", norm && ext_grad ? qe : nullptr, B * M * L * 4}};
+    for (const Range& in : ins) {
+        // state_grad == ext_grad (in place) is allowed: every element is read before it is written
+        if (overlap(out_r, in) && !(in.p == ext_grad && state_grad == ext_grad))
+            return fail(FMSCAN_E_ALIAS, "fmscan_readout_backward: state_grad overlaps %s", in.name);
+    }
+    const bool vec = vector_path(rs, {norm ? states_n : nullptr, inv_rms, read, out_grad, ext_grad,
+                                      norm ? (const void*)q : nullptr, norm && ext_grad ? (const void*)qe : nullptr,
+                                      state_grad});
+    const dim3 grid((unsigned)(B * rs.tiles), (unsigned)((D + 4 * kReadoutRows - 1) / (4 * kReadoutRows)));
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        with_bool(norm, [&](auto nt) {
+            with_bool(ext_grad != nullptr, [&](auto et) {
+                with_bool(vec, [&](auto vt) {
+                    fmscan::readout_backward_kernel<T, kReadoutRows, decltype(nt)::value, decltype(et)::value,
+                                                    decltype(vt)::value>
+                        <<<grid, 256, 0, (hipStream_t)stream>>>((const T*)states_n, inv_rms, (const T*)read,
+                                                                (const T*)out_grad, (const T*)ext_grad, q, qe,
+                                                                (T*)state_grad, (int32_t)M, (int32_t)D, L,
+                                                                rs.tiles);
+                });
+            });
+        });
+    });
+    return launched("read-out (backward)");
 }
 
 }  // extern "C"

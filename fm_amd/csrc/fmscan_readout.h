@@ -1,0 +1,228 @@
+// The part of the Factorization-Memory layer that consumes the scanned states
+// (reference fm/scan/fm_scan.py:124-131): RMS norm over the D axis of every memory
+// slot, then the read-out  output[b,t,d] = sum_m read[b,t,m] * states[b,m,d,t].
+// The reference runs it as five PyTorch operations over (B, M, D, L) tensors (square,
+// mean, rsqrt, multiply, einsum), each a full pass through HBM, and autograd doubles
+// that. Here, forward and backward are two kernels each:
+//
+//   rowdot_kernel     one value per (b, m, t) from all D rows of a slot:
+//                       SUMSQ: inv_rms = rsqrt(mean_d h^2 + eps)
+//                       DOT:   q = sum_d out_grad[b,d,t] * hn[b,m,d,t]   (= d read)
+//                              qe = sum_d ext_grad[b,m,d,t] * hn[b,m,d,t] (optional)
+//   readout_forward   hn = h * inv_rms (stored), out[b,d,t] = sum_m read * hn
+//   readout_backward  d h = inv_rms * (dhn - hn * mean_d(dhn * hn)),
+//                       dhn = read * out_grad (+ ext_grad)
+//
+// All of them stream rows the way the scan kernels do: a wave instruction covers 1 KiB
+// of one row (16 bytes per lane), fp32 arithmetic, one rounding on store. Time is the
+// innermost axis of every tensor here, as the scan leaves it: output is (B, D, L).
+#pragma once
+
+#include "fmscan_device.h"
+
+namespace fmscan {
+
+// E consecutive floats of a per-(b, m) vector (inv_rms, q): row + t0 .. t0 + E - 1
+template <int E, bool VEC>
+__device__ __forceinline__ void load_floats(const float* __restrict__ row, int64_t t0, int64_t L,
+                                            float (&v)[E], float fill) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) v[i] = fill;
+    if (t0 >= L) return;
+    if constexpr (VEC) {  // L is a multiple of E and rows start 16-byte aligned
+#pragma unroll
+        for (int i = 0; i < E; i += 4) {
+            const float4 f = *reinterpret_cast<const float4*>(row + t0 + i);
+            v[i] = f.x; v[i + 1] = f.y; v[i + 2] = f.z; v[i + 3] = f.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < E; ++i)
+            if (t0 + i < L) v[i] = row[t0 + i];
+    }
+}
+
+enum class RowDot { kSumSq, kDot };
+
+// One block per (b, m, tile of L), blockIdx.x = (b * M + m) * tiles + tile; WV waves take
+// the D rows of the slot in turn.
+template <typename T, int WV, RowDot MODE, bool EXT, bool VEC>
+__global__ __launch_bounds__(64 * WV) void rowdot_kernel(
+    const T* __restrict__ states /* (B, M, D, L) */, const T* __restrict__ out_grad /* (B, D, L) */,
+    const T* __restrict__ ext_grad /* (B, M, D, L) */, float* __restrict__ result /* (B, M, L) */,
+    float* __restrict__ result_ext /* (B, M, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles,
+    float eps) {
+    constexpr int E = Elem<T>::E;
+    constexpr int TILE = E * 64;
+    __shared__ float part[EXT ? 2 : 1][WV][TILE];
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int64_t bm = blockIdx.x / (uint32_t)tiles;
+    const int64_t tile = blockIdx.x - bm * tiles;
+    const int64_t b = bm / M;
+    const int64_t t0 = tile * TILE + (int64_t)lane * E;
+
+    float acc[E], acc_ext[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) acc[i] = acc_ext[i] = 0.0f;
+#pragma unroll 4
+    for (int32_t d = w; d < D; d += WV) {
+        float h[E];
+        Elem<T>::unpack(load_chunk<T, VEC, MODE == RowDot::kSumSq>(states + (bm * D + d) * L, t0, L, 0u), h);
+        if constexpr (MODE == RowDot::kSumSq) {
+#pragma unroll
+            for (int i = 0; i < E; ++i) acc[i] = __builtin_fmaf(h[i], h[i], acc[i]);
+        } else {
+            float y[E];
+            Elem<T>::unpack(load_chunk<T, VEC, false>(out_grad + (b * D + d) * L, t0, L, 0u), y);
+#pragma unroll
+            for (int i = 0; i < E; ++i) acc[i] = __builtin_fmaf(h[i], y[i], acc[i]);
+            if constexpr (EXT) {
+                Elem<T>::unpack(load_chunk<T, VEC, true>(ext_grad + (bm * D + d) * L, t0, L, 0u), y);
+#pragma unroll
+                for (int i = 0; i < E; ++i) acc_ext[i] = __builtin_fmaf(h[i], y[i], acc_ext[i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+        part[0][w][lane * E + i] = acc[i];
+        if constexpr (EXT) part[1][w][lane * E + i] = acc_ext[i];
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < TILE; e += 64 * WV) {
+        const int64_t t = tile * TILE + e;
+        if (t >= L) break;
+        float s = 0.0f, se = 0.0f;
+#pragma unroll
+        for (int v = 0; v < WV; ++v) {  // fixed order: run-to-run identical
+            s += part[0][v][e];
+            if constexpr (EXT) se += part[1][v][e];
+        }
+        if constexpr (MODE == RowDot::kSumSq) s = 1.0f / __builtin_sqrtf(s / (float)D + eps);
+        result[bm * L + t] = s;
+        if constexpr (EXT) result_ext[bm * L + t] = se;
+    }
+}
+
+// grid (B * tiles of L, groups of 4 * J consecutive d); wave w of a block owns J
+// consecutive d and walks the M slots; the per-slot vectors (inv_rms, read) are loaded
+// once per slot and reused for the J rows.
+template <typename T, int J, bool NORM, bool VEC>
+__global__ __launch_bounds__(256) void readout_forward_kernel(
+    const T* __restrict__ states /* (B, M, D, L) */, const float* __restrict__ inv_rms /* (B, M, L) */,
+    const T* __restrict__ read /* (B, M, L) */, T* __restrict__ states_out /* (B, M, D, L) */,
+    T* __restrict__ output /* (B, D, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles) {
+    constexpr int E = Elem<T>::E;
+    constexpr int TILE = E * 64;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int64_t b = blockIdx.x / (uint32_t)tiles;
+    const int32_t d0 = ((int32_t)blockIdx.y * 4 + w) * J;
+    if (d0 >= D) return;  // whole waves; no barrier in this kernel
+    const int64_t t0 = (blockIdx.x - b * tiles) * TILE + (int64_t)lane * E;
+
+    float acc[J][E];
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) acc[j][i] = 0.0f;
+    }
+    for (int32_t m = 0; m < M; ++m) {
+        const int64_t bm = b * M + m;
+        float r[E], wr[E];
+        if constexpr (NORM) load_floats<E, VEC>(inv_rms + bm * L, t0, L, r, 0.0f);
+        Elem<T>::unpack(load_chunk<T, VEC, false>(read + bm * L, t0, L, 0u), wr);
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            if (d0 + j < D) {
+                const int64_t row = (bm * D + d0 + j) * L;
+                float h[E];
+                Elem<T>::unpack(load_chunk<T, VEC, true>(states + row, t0, L, 0u), h);
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int i = 0; i < E; ++i) h[i] *= r[i];
+                    const u32x4 packed = Elem<T>::pack(h);
+                    store_chunk<T, VEC>(states_out + row, t0, L, packed);
+                    Elem<T>::unpack(packed, h);  // the read-out sees what was stored
+                }
+#pragma unroll
+                for (int i = 0; i < E; ++i) acc[j][i] = __builtin_fmaf(wr[i], h[i], acc[j][i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+        if (d0 + j < D) store_chunk<T, VEC>(output + (b * D + d0 + j) * L, t0, L, Elem<T>::pack(acc[j]));
+}
+
+// Same grid. dhn = read * out_grad (+ ext_grad); with the norm
+// d h = inv_rms * (dhn - hn * s / D), s = sum_d dhn * hn = read * q (+ qe).
+template <typename T, int J, bool NORM, bool EXT, bool VEC>
+__global__ __launch_bounds__(256) void readout_backward_kernel(
+    const T* __restrict__ states_n /* (B, M, D, L), normalised; unused without the norm */,
+    const float* __restrict__ inv_rms, const T* __restrict__ read, const T* __restrict__ out_grad /* (B, D, L) */,
+    const T* __restrict__ ext_grad /* (B, M, D, L) */, const float* __restrict__ q, const float* __restrict__ qe,
+    T* __restrict__ state_grad /* (B, M, D, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles) {
+    constexpr int E = Elem<T>::E;
+    constexpr int TILE = E * 64;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int64_t b = blockIdx.x / (uint32_t)tiles;
+    const int32_t d0 = ((int32_t)blockIdx.y * 4 + w) * J;
+    if (d0 >= D) return;
+    const int64_t t0 = (blockIdx.x - b * tiles) * TILE + (int64_t)lane * E;
+
+    float dout[J][E];
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) dout[j][i] = 0.0f;
+        if (d0 + j < D)
+            Elem<T>::unpack(load_chunk<T, VEC, false>(out_grad + (b * D + d0 + j) * L, t0, L, 0u), dout[j]);
+    }
+    const float inv_d = 1.0f / (float)D;
+    for (int32_t m = 0; m < M; ++m) {
+        const int64_t bm = b * M + m;
+        float wr[E], r[E], s[E];
+        Elem<T>::unpack(load_chunk<T, VEC, false>(read + bm * L, t0, L, 0u), wr);
+        if constexpr (NORM) {
+            load_floats<E, VEC>(inv_rms + bm * L, t0, L, r, 0.0f);
+            load_floats<E, VEC>(q + bm * L, t0, L, s, 0.0f);
+#pragma unroll
+            for (int i = 0; i < E; ++i) s[i] *= wr[i];
+            if constexpr (EXT) {
+                float se[E];
+                load_floats<E, VEC>(qe + bm * L, t0, L, se, 0.0f);
+#pragma unroll
+                for (int i = 0; i < E; ++i) s[i] += se[i];
+            }
+#pragma unroll
+            for (int i = 0; i < E; ++i) s[i] *= inv_d;
+        }
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            if (d0 + j < D) {
+                const int64_t row = (bm * D + d0 + j) * L;
+                float g[E];
+#pragma unroll
+                for (int i = 0; i < E; ++i) g[i] = wr[i] * dout[j][i];
+                if constexpr (EXT) {
+                    float e[E];
+                    Elem<T>::unpack(load_chunk<T, VEC, true>(ext_grad + row, t0, L, 0u), e);
+#pragma unroll
+                    for (int i = 0; i < E; ++i) g[i] += e[i];
+                }
+                if constexpr (NORM) {
+                    float hn[E];
+                    Elem<T>::unpack(load_chunk<T, VEC, true>(states_n + row, t0, L, 0u), hn);
+#pragma unroll
+                    for (int i = 0; i < E; ++i) g[i] = r[i] * __builtin_fmaf(-hn[i], s[i], g[i]);
+                }
+                store_chunk<T, VEC>(state_grad + row, t0, L, Elem<T>::pack(g));
+            }
+        }
+    }
+}
+
+}  // namespace fmscan

@@ -10,6 +10,11 @@ Exports, with the reference's names and positional signatures:
     fm_scan(gates, tokens, initial_state=None)                       fm_scan.py:84-99
     fm_memory(alpha, update_scale, output_scale, inputs, ...)        fm_scan.py:102-133
 
+and, for what fm_memory does with the states after the scan (RMS norm over D and the
+read-out over the M slots, fm_scan.py:124-131), `fm_readout` / `FM_Readout`, which run
+those steps and their gradients as four kernels instead of PyTorch operations over
+(B, M, D, L) tensors.
+
 The two extension functions call libfmscan_hip.so through ctypes with raw device
 pointers and the current HIP stream; there is no CPU implementation behind them.
 """
@@ -20,7 +25,7 @@ import torch
 from .. import _lib
 
 __all__ = ["fm_scan_forward", "fm_scan_backward", "fm_scan_backward_reduced", "FM_Scan", "fm_scan",
-           "fm_memory", "module"]
+           "fm_readout_forward", "fm_readout_backward", "FM_Readout", "fm_readout", "fm_memory", "module"]
 
 _DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16,
            torch.bfloat16: _lib.DTYPE_BF16}
@@ -301,6 +306,117 @@ def fm_scan(gates, tokens, initial_state=None):
     return FM_Scan.apply(gates, tokens, initial_state)
 
 
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6):
+    """RMS norm over D and read-out over M of scanned states (reference fm_scan.py:124-131).
+
+    states (B, M, D, L), read (B, M, L) = (alpha * output_scale) with time last; same dtype,
+    contiguous, on one GPU. Returns (output (B, D, L), normalised states (B, M, D, L) or None
+    without the norm, inv_rms (B, M, L) float32 or None).
+    """
+    dev = states.device
+    for name, t in (("states", states), ("read", read)):
+        _on_gpu(name, t, dev)
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        _require(t.dtype == states.dtype, f"{name} has dtype {t.dtype}, states has {states.dtype}")
+    _require(states.dim() == 4, "states must be (B, M, D, L)")
+    B, M, D, L = states.shape
+    _require(tuple(read.shape) == (B, M, L), f"read must be {(B, M, L)}, got {tuple(read.shape)}")
+    code = _dtype_code(states)
+    output = torch.empty((B, D, L), dtype=states.dtype, device=dev)
+    normed = torch.empty_like(states) if mem_norm else None
+    inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev) if mem_norm else None
+    if states.numel():
+        with _on_device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            if mem_norm:
+                _lib.check(module.fmscan_readout_inv_rms(states.data_ptr(), inv_rms.data_ptr(), B, M, D, L,
+                                                         code, float(norm_eps), stream))
+            _lib.check(module.fmscan_readout_forward(states.data_ptr(), _ptr(inv_rms), read.data_ptr(),
+                                                     _ptr(normed), output.data_ptr(), B, M, D, L, code,
+                                                     stream))
+    return output, normed, inv_rms
+
+
+def fm_readout_backward(out_grad, ext_grad, read, states_n, inv_rms):
+    """Gradients of fm_readout_forward.
+
+    out_grad (B, D, L): gradient of the output; ext_grad (B, M, D, L) or None: gradient that
+    arrives at the returned (normalised) states; states_n: the normalised states (the scanned
+    states themselves without the norm); inv_rms (B, M, L) float32 or None without the norm.
+    Returns (state_grad (B, M, D, L), read_grad (B, M, L)).
+    """
+    dev = states_n.device
+    for name, t in (("out_grad", out_grad), ("ext_grad", ext_grad), ("read", read), ("states_n", states_n),
+                    ("inv_rms", inv_rms)):
+        if t is None:
+            continue
+        _on_gpu(name, t, dev)
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        if name != "inv_rms":
+            _require(t.dtype == states_n.dtype, f"{name} has dtype {t.dtype}, states_n has {states_n.dtype}")
+    B, M, D, L = states_n.shape
+    _require(tuple(out_grad.shape) == (B, D, L), f"out_grad must be {(B, D, L)}")
+    _require(tuple(read.shape) == (B, M, L), f"read must be {(B, M, L)}")
+    _require(ext_grad is None or tuple(ext_grad.shape) == (B, M, D, L), f"ext_grad must be {(B, M, D, L)}")
+    _require(inv_rms is None or (tuple(inv_rms.shape) == (B, M, L) and inv_rms.dtype == torch.float32),
+             f"inv_rms must be float32 {(B, M, L)}")
+    code = _dtype_code(states_n)
+    q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
+    qe = torch.empty_like(q) if (ext_grad is not None and inv_rms is not None) else None
+    state_grad = torch.empty_like(states_n)
+    if states_n.numel():
+        with _on_device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            _lib.check(module.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(),
+                                                 None if qe is None else ext_grad.data_ptr(), q.data_ptr(),
+                                                 _ptr(qe), B, M, D, L, code, stream))
+            _lib.check(module.fmscan_readout_backward(states_n.data_ptr(), _ptr(inv_rms), read.data_ptr(),
+                                                      out_grad.data_ptr(), _ptr(ext_grad), q.data_ptr(),
+                                                      _ptr(qe), state_grad.data_ptr(), B, M, D, L, code,
+                                                      stream))
+    return state_grad, q.to(states_n.dtype)
+
+
+class FM_Readout(torch.autograd.Function):
+    """output, states_n = FM_Readout.apply(states, read, mem_norm, norm_eps)
+
+    states (B, M, D, L), read (B, M, L) -> output (B, D, L) and the normalised states
+    (None when mem_norm is false: the scanned states are then what the layer returns).
+    """
+
+    @staticmethod
+    def forward(ctx, states, read, mem_norm=True, norm_eps=1e-6):
+        output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps)
+        ctx.mem_norm = bool(mem_norm)
+        # the normalised states and inv_rms carry everything the gradient needs
+        ctx.save_for_backward(read, normed if mem_norm else states, inv_rms)
+        ctx.set_materialize_grads(False)
+        return output, (normed if mem_norm else None)
+
+    @staticmethod
+    def backward(ctx, out_grad, ext_grad):
+        read, states_n, inv_rms = ctx.saved_tensors
+        if out_grad is None and ext_grad is None:
+            return None, None, None, None
+        if out_grad is None:
+            B, M, D, L = states_n.shape
+            out_grad = torch.zeros((B, D, L), dtype=states_n.dtype, device=states_n.device)
+        state_grad, read_grad = fm_readout_backward(
+            out_grad.contiguous(), None if ext_grad is None else ext_grad.contiguous(), read, states_n,
+            inv_rms)
+        return state_grad, read_grad, None, None
+
+
+def fm_readout(states, read, mem_norm=True, norm_eps=1e-6):
+    """(output (B, D, L), states as the layer returns them (B, M, D, L))."""
+    output, normed = FM_Readout.apply(states, read, mem_norm, norm_eps)
+    return output, (normed if mem_norm else states)
+
+
 def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True,
               norm_eps=1e-6):
     """The Factorization-Memory layer around the scan (reference fm_scan.py:102-133).
@@ -311,15 +427,14 @@ def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem
         inputs:       (B, L, D)
         initial_state (B, M, D), optional
     Returns (output (B, L, D), memory_states (B, M, D, L)).
+
+    Only the (B, L, *) tensors pass through PyTorch operations here; everything of size
+    (B, M, D, L) is produced and consumed by the library's kernels.
     """
     write = (alpha * update_scale).transpose(1, 2).contiguous()  # (B, M, L)
     tokens = inputs.transpose(1, 2).contiguous()                 # (B, D, L)
     memory_states = fm_scan(1.0 - write, tokens, initial_state)  # decay gate = 1 - write weight
 
-    if mem_norm:  # RMS norm over the D axis of every memory slot
-        inv_rms = torch.rsqrt(memory_states.pow(2).mean(dim=2, keepdim=True) + norm_eps)
-        memory_states = memory_states * inv_rms
-
-    read = alpha * output_scale  # (B, L, M)
-    output = torch.einsum("blm,bmdl->bld", read, memory_states).contiguous()
-    return output, memory_states
+    read = (alpha * output_scale).transpose(1, 2).contiguous()   # (B, M, L)
+    output, memory_states = fm_readout(memory_states, read, mem_norm, norm_eps)  # (B, D, L)
+    return output.transpose(1, 2).contiguous(), memory_states

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FMSCAN_ABI_VERSION 2
+#define FMSCAN_ABI_VERSION 3
 
 /* element type of every tensor in one call (reference fm_scan.cuh:333-342) */
 #define FMSCAN_DTYPE_F32  0
@@ -165,6 +165,52 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
                             const void* initial_state, void* initial_state_grad,
                             int64_t B, int64_t M, int64_t D, int64_t L,
                             int dtype, unsigned flags, void* stream);
+
+/*
+ * The read-out of the Factorization-Memory layer (reference fm/scan/fm_scan.py:124-131,
+ * inside fm_memory): RMS norm of the scanned states over the D axis of every memory slot
+ *   inv_rms[b,m,t] = rsqrt(mean_d states[b,m,d,t]^2 + eps)            (:126)
+ *   normalised     = states * inv_rms                                  (:127)
+ * and the output projection over the M slots
+ *   output[b,d,t]  = sum_m read[b,m,t] * normalised[b,m,d,t]           (:130-131,
+ * einsum 'blm,bmdl->bld' with read = (alpha * output_scale) laid out (B, M, L); the
+ * caller transposes output to the reference's (B, L, D)). The reference leaves these to
+ * five PyTorch operations over (B, M, D, L) tensors and to autograd; the four calls
+ * below are their forward and backward with fp32 arithmetic and one rounding per
+ * stored value. Every tensor is dense with L innermost, of the call's dtype unless
+ * marked float32. Any L; 16-byte aligned pointers with L * sizeof(element) % 16 == 0
+ * take the vector path. B * M * ceil(L / tile) must be < 2^31 (tile = 256 float32 /
+ * 512 16-bit elements) and D < 2^20.
+ *
+ * fmscan_readout_inv_rms:   inv_rms (B, M, L) float32 out.
+ * fmscan_readout_forward:   inv_rms NULL = no norm (mem_norm=False, :125): states_out
+ *                           is then ignored and the read-out sees `states`; otherwise
+ *                           states_out (B, M, D, L) receives the normalised states (it
+ *                           may be the same buffer as `states`), and the read-out uses
+ *                           the stored (rounded) values as the reference does.
+ * fmscan_readout_dot:       q[b,m,t] = sum_d out_grad[b,d,t] * states_n[b,m,d,t]
+ *                           (float32; it is the gradient of `read`) and, when ext_grad
+ *                           (a gradient arriving at the returned memory states,
+ *                           (B, M, D, L)) is not NULL, qe = sum_d ext_grad * states_n.
+ * fmscan_readout_backward:  state_grad (B, M, D, L) = gradient of the scanned states:
+ *                           dn = read * out_grad (+ ext_grad);
+ *                           with the norm  inv_rms * (dn - states_n * (read*q + qe) / D),
+ *                           without it     dn  (states_n, inv_rms, q, qe unused, may be NULL).
+ * Return values as for the scan calls.
+ */
+int fmscan_readout_inv_rms(const void* states, float* inv_rms,
+                           int64_t B, int64_t M, int64_t D, int64_t L, int dtype, float eps,
+                           void* stream);
+int fmscan_readout_forward(const void* states, const float* inv_rms, const void* read,
+                           void* states_out, void* output,
+                           int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
+int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad,
+                       float* q, float* qe,
+                       int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
+int fmscan_readout_backward(const void* states_n, const float* inv_rms, const void* read,
+                            const void* out_grad, const void* ext_grad,
+                            const float* q, const float* qe, void* state_grad,
+                            int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

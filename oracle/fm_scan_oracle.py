@@ -21,6 +21,14 @@ What each function follows in the reference:
                        firstPropGrad, :380).
 * `backward`           fm/scan/fm_scan.py:61-81 (zero firstPropGrad, the sums
                        over D for d_gates and over M for d_tokens).
+* `readout_forward`    fm/scan/fm_scan.py:124-131 (inside fm_memory): RMS norm over D
+                       of every slot, then einsum 'blm,bmdl->bld'; here with time
+                       last: read (B, M, L), output (B, D, L).
+* `readout_backward`   the gradients of those lines, which the reference leaves to
+                       autograd; written out by hand and pinned against finite
+                       differences and against autograd through the same PyTorch
+                       operations the reference lines name (tests/test_oracle.py).
+* `memory_forward`     fm/scan/fm_scan.py:115-133, the whole layer.
 
 How it is pinned (tests/test_oracle.py): exact rational arithmetic on small
 inputs with forward-mode derivatives (tests/golden/), closed forms (constant
@@ -37,7 +45,8 @@ from __future__ import annotations
 
 import numpy as np
 
-__all__ = ["forward", "backward_per_row", "backward", "to_f64"]
+__all__ = ["forward", "backward_per_row", "backward", "to_f64", "readout_forward", "readout_backward",
+           "memory_forward"]
 
 
 def to_f64(a):
@@ -144,3 +153,53 @@ def backward(gates, tokens, out_grad, initial_state=None, plain=False, states=No
     d_tokens = tg.sum(axis=1)
     d_h0 = g[:, :, 0][:, :, None] * delta[:, :, :, 0]
     return d_gates, d_tokens, d_h0
+
+
+def readout_forward(states, read, mem_norm=True, eps=1e-6):
+    """states (B, M, D, L), read (B, M, L) -> (output (B, D, L), states as returned, inv_rms).
+
+    fm_scan.py:125-127: inv_rms = rsqrt(mean(states**2, dim=2) + eps), states * inv_rms;
+    fm_scan.py:130-131: output[b,l,d] = sum_m read[b,l,m] * states[b,m,d,l].
+    """
+    states = to_f64(states)
+    read = to_f64(read)
+    inv_rms = None
+    if mem_norm:
+        inv_rms = 1.0 / np.sqrt(np.mean(states * states, axis=2) + eps)  # (B, M, L)
+        states = states * inv_rms[:, :, None, :]
+    output = np.einsum("bml,bmdl->bdl", read, states)
+    return output, states, inv_rms
+
+
+def readout_backward(out_grad, ext_grad, read, states, mem_norm=True, eps=1e-6):
+    """Gradients of readout_forward with respect to `states` (before the norm) and `read`.
+
+    out_grad (B, D, L) is the gradient of the output, ext_grad (B, M, D, L) or None the
+    one arriving at the returned states. With n = states * r, r = inv_rms:
+        dn = read * out_grad + ext_grad,  d read = sum_d out_grad * n,
+        d states = r * (dn - n * mean_d(dn * n)).
+    """
+    states = to_f64(states)
+    read = to_f64(read)
+    out_grad = to_f64(out_grad)
+    _, normed, inv_rms = readout_forward(states, read, mem_norm, eps)
+    dn = read[:, :, None, :] * out_grad[:, None, :, :]
+    if ext_grad is not None:
+        dn = dn + to_f64(ext_grad)
+    read_grad = np.einsum("bdl,bmdl->bml", out_grad, normed)
+    if not mem_norm:
+        return dn, read_grad
+    inner = np.mean(dn * normed, axis=2, keepdims=True)
+    return inv_rms[:, :, None, :] * (dn - normed * inner), read_grad
+
+
+def memory_forward(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True, eps=1e-6):
+    """fm_memory (fm_scan.py:102-133): alpha (B, L, M), scales (B, L, 1), inputs (B, L, D)
+    -> (output (B, L, D), memory states (B, M, D, L))."""
+    alpha, update_scale, output_scale, inputs = (to_f64(a) for a in (alpha, update_scale, output_scale, inputs))
+    write = np.ascontiguousarray(np.transpose(alpha * update_scale, (0, 2, 1)))  # :116,118
+    tokens = np.ascontiguousarray(np.transpose(inputs, (0, 2, 1)))              # :117
+    states = forward(1.0 - write, tokens, initial_state)                         # :119,121
+    read = np.ascontiguousarray(np.transpose(alpha * output_scale, (0, 2, 1)))   # :130
+    output, states, _ = readout_forward(states, read, mem_norm, eps)
+    return np.ascontiguousarray(np.transpose(output, (0, 2, 1))), states

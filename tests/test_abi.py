@@ -24,8 +24,9 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_reduced",
-                                    "fmscan_forward", "fmscan_last_error", "fmscan_reduced_groups",
-                                    "fmscan_workspace_bytes"]
+                                    "fmscan_forward", "fmscan_last_error", "fmscan_readout_backward",
+                                    "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
+                                    "fmscan_reduced_groups", "fmscan_workspace_bytes"]
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -106,6 +107,34 @@ def test_rejected_arguments(lib):
     assert bwd(lib, dx=4 * P) == E_ALIAS              # token_grad_out on top of cached_output
     assert bwd(lib, dg=3 * P) == E_ALIAS              # the two outputs on top of each other
     assert b"overlaps" in lib.fmscan_last_error()
+
+
+def test_rejected_readout_arguments(lib):
+    E_NULL, E_SHAPE, E_DTYPE, E_ALIAS = (_const("FMSCAN_E_" + n) for n in ("NULL", "SHAPE", "DTYPE", "ALIAS"))
+    dims = (2, 3, 4, 64)
+    rms = lambda s=P, r=2 * P, dims=dims, dtype=2, eps=1e-6: lib.fmscan_readout_inv_rms(s, r, *dims, dtype, eps, None)
+    assert rms(s=None) == E_NULL
+    assert rms(dims=(2, 3, 0, 64)) == E_SHAPE
+    assert rms(dims=(2, 3, 1 << 20, 64)) == E_SHAPE      # D beyond the grid
+    assert rms(dtype=5) == E_DTYPE
+    assert rms(eps=-1.0) == E_SHAPE
+    assert rms(r=P + 64) == E_ALIAS
+    fw = lambda s=P, r=2 * P, w=3 * P, so=4 * P, o=5 * P: lib.fmscan_readout_forward(s, r, w, so, o, *dims, 2, None)
+    assert fw(w=None) == E_NULL
+    assert fw(so=None) == E_NULL                        # the norm needs somewhere to put the states
+    assert fw(o=P) == E_ALIAS
+    assert fw(so=3 * P) == E_ALIAS                       # normalised states on top of read
+    assert b"overlaps" in lib.fmscan_last_error()
+    dot = lambda sn=P, og=2 * P, e=None, q=3 * P, qe=None: lib.fmscan_readout_dot(sn, og, e, q, qe, *dims, 2, None)
+    assert dot(q=None) == E_NULL
+    assert dot(e=4 * P) == E_NULL                        # ext_grad without qe
+    assert dot(e=4 * P, qe=3 * P) == E_ALIAS
+    bw = lambda sn=P, r=2 * P, w=3 * P, og=4 * P, e=None, q=5 * P, qe=None, sg=6 * P: \
+        lib.fmscan_readout_backward(sn, r, w, og, e, q, qe, sg, *dims, 2, None)
+    assert bw(sg=None) == E_NULL
+    assert bw(q=None) == E_NULL                          # the norm's gradient needs q
+    assert bw(e=7 * P) == E_NULL                         # ... and qe when ext_grad is given
+    assert bw(sg=P) == E_ALIAS
 
 
 def test_workspace_bytes(lib):

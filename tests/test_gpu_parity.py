@@ -473,33 +473,97 @@ def test_seven_argument_backward_reproduces_reference_kernel(scan):
     check("gate grad", dg, gg, 1e-5)
 
 
-def test_fm_memory_layer(scan):
-    """The layer on top of the scan, forward and backward, against the same layer
-    built on the per-timestep PyTorch form in float64."""
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mem_norm", [True, False])
+def test_readout_kernels(scan, dtype, mem_norm):
+    """RMS norm + read-out and their gradients (four kernels) against the float64 oracle on
+    the same quantised inputs; shapes cover ragged tiles, D beyond and below a block's 16
+    rows, and lengths that force the element path."""
+    for (B, M, D, L), with_ext in [((2, 3, 5, 512), True), ((1, 2, 16, 8), False), ((2, 4, 40, 4096), True),
+                                   ((1, 33, 17, 1000), False), ((3, 2, 9, 2055), True),
+                                   ((1, 5, 130, 640), False)]:
+        gen = torch.Generator().manual_seed(B * 1000 + D)
+        states = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+        read = torch.randn(B, M, L, generator=gen).to(dtype).to(DEV)
+        out_grad = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        ext = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV) if (with_ext and mem_norm) else None
+        eps = 1e-6
+        out, normed, inv_rms = scan.fm_readout_forward(states, read, mem_norm, eps)
+        o_out, o_normed, o_inv = O.readout_forward(states, read, mem_norm, eps)
+        tag = f"{(B, M, D, L)} {dtype} norm={mem_norm}"
+        check(tag + " output", out, o_out, TOL[dtype])
+        if mem_norm:
+            check(tag + " normalised states", normed, o_normed, TOL[dtype])
+            check(tag + " inv_rms", inv_rms, o_inv, 1e-5)
+        else:
+            assert normed is None and inv_rms is None
+        # gradients: the kernels work from the stored (rounded) normalised states, the oracle
+        # from exact ones; the difference is inside the storage type's tolerance
+        states_n = normed if mem_norm else states
+        d_states, d_read = scan.fm_readout_backward(out_grad, ext, read, states_n, inv_rms)
+        o_ds, o_dr = O.readout_backward(out_grad, ext, read, states, mem_norm, eps)
+        check(tag + " d_states", d_states, o_ds, 2 * TOL[dtype])
+        check(tag + " d_read", d_read, o_dr, 2 * TOL[dtype])
+
+
+def test_readout_in_place_and_determinism(scan):
+    B, M, D, L, dt = 2, 8, 64, 2048, torch.bfloat16
+    gen = gpu_gen(5)
+    states = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    read = torch.randn(B, M, L, device=DEV, generator=gen).to(dt)
+    out1, n1, r1 = scan.fm_readout_forward(states, read)
+    out2, n2, r2 = scan.fm_readout_forward(states, read)
+    assert torch.equal(out1, out2) and torch.equal(n1, n2) and torch.equal(r1, r2)
+    # in place through the C interface: states_out == states
+    lib = scan.module
+    buf = states.clone()
+    out3 = torch.empty_like(out1)
+    rc = lib.fmscan_readout_forward(buf.data_ptr(), r1.data_ptr(), read.data_ptr(), buf.data_ptr(),
+                                    out3.data_ptr(), B, M, D, L, 2, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(buf, n1) and torch.equal(out3, out1)
+
+
+@pytest.mark.parametrize("dtype,mem_norm", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, True)])
+def test_fm_memory_layer(scan, dtype, mem_norm):
+    """The layer on top of the scan, forward and backward (gradients arriving at both
+    returned tensors), against the float64 oracle layer / the same layer written with the
+    PyTorch operations the reference names, in float64 on the CPU."""
     from fm.scan.fm_pytorch import fm_scan_pytorch
 
-    B, L, M, D = 2, 512, 4, 16
+    B, L, M, D = 2, 512, 4, 24
     gen = torch.Generator().manual_seed(13)
     mk = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float64)
-    alpha64 = torch.softmax(mk(B, L, M), dim=-1)
-    us64, os64, inp64 = torch.rand(B, L, 1, generator=gen, dtype=torch.float64), \
-        torch.rand(B, L, 1, generator=gen, dtype=torch.float64), mk(B, L, D)
+    q = lambda t: t.to(dtype).to(torch.float64)  # both sides start from the same quantised values
+    alpha64 = q(torch.softmax(mk(B, L, M), dim=-1))
+    us64, os64, inp64 = q(torch.rand(B, L, 1, generator=gen, dtype=torch.float64)), \
+        q(torch.rand(B, L, 1, generator=gen, dtype=torch.float64)), q(mk(B, L, D))
+    h064 = q(mk(B, M, D))
+    w_mem = q(mk(B, M, D, L)) * 0.1
     outs = {}
-    for name, dt, dev in (("gpu", torch.float32, DEV), ("ref", torch.float64, "cpu")):
-        a, u, o, i = (t.to(dt).to(dev).requires_grad_() for t in (alpha64, us64, os64, inp64))
+    for name, dt, dev in (("gpu", dtype, DEV), ("ref", torch.float64, "cpu")):
+        a, u, o, i, h0 = (t.to(dt).to(dev).requires_grad_() for t in (alpha64, us64, os64, inp64, h064))
         if name == "gpu":
-            y, mem = scan.fm_memory(a, u, o, i)
+            y, mem = scan.fm_memory(a, u, o, i, h0, mem_norm=mem_norm, norm_eps=1e-4)
+            assert y.shape == (B, L, D) and mem.shape == (B, M, D, L) and y.is_contiguous()
         else:
             tok = i.transpose(1, 2).contiguous()
             gate = 1.0 - (a * u).transpose(1, 2).contiguous()
-            mem = fm_scan_pytorch(gate, tok)
-            mem = mem * torch.rsqrt((mem ** 2).mean(dim=2, keepdim=True) + 1e-6)
+            mem = fm_scan_pytorch(gate, tok, h0)
+            if mem_norm:
+                mem = mem * torch.rsqrt((mem ** 2).mean(dim=2, keepdim=True) + 1e-4)
             y = torch.einsum("blm,bmdl->bld", a * o, mem)
-        y.square().sum().backward()
-        outs[name] = [y.detach(), mem.detach(), a.grad, u.grad, o.grad, i.grad]
+            o_y, o_mem = O.memory_forward(alpha64, us64, os64, inp64, h064, mem_norm, 1e-4)
+            np.testing.assert_allclose(y.detach().numpy(), o_y, rtol=1e-10, atol=1e-10)
+            np.testing.assert_allclose(mem.detach().numpy(), o_mem, rtol=1e-10, atol=1e-10)
+        acc = torch.float64 if name == "ref" else torch.float32
+        (y.to(acc).square().sum() + (mem.to(acc) * w_mem.to(dev).to(acc)).sum()).backward()
+        outs[name] = [y.detach(), mem.detach(), a.grad, u.grad, o.grad, i.grad, h0.grad]
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
     for t_gpu, t_ref, what in zip(outs["gpu"], outs["ref"], ("output", "memory", "d_alpha", "d_update_scale",
-                                                            "d_output_scale", "d_inputs")):
-        check(what, t_gpu, t_ref.numpy(), 1e-4)
+                                                            "d_output_scale", "d_inputs", "d_initial_state")):
+        check(what, t_gpu, t_ref.numpy(), tol)
 
 
 # ----------------------------------------------------------------------------- errors on the GPU

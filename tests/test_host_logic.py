@@ -40,6 +40,12 @@ def test_cpu_tensors_are_rejected_loudly():
         fm_scan_forward(g, x, torch.zeros(1, 1, 1), out)
     with pytest.raises(RuntimeError, match="GPU tensor"):
         fm_scan_backward(g, out, torch.zeros(1, 1, 1), out.clone(), out, x, out.clone())
+    from fm.scan.fm_scan import fm_memory, fm_readout
+
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fm_readout(out, g)
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        fm_memory(torch.rand(1, 32, 2), torch.rand(1, 32, 1), torch.rand(1, 32, 1), torch.rand(1, 32, 3))
 
 
 def test_fm_scan_shape_asserts_match_reference_behaviour():
@@ -55,14 +61,21 @@ def test_fm_scan_shape_asserts_match_reference_behaviour():
         fm_scan(torch.rand(2, 3, 32), torch.rand(2, 4, 32), torch.zeros(2, 4, 3))
 
 
-def test_fm_memory_layer_arithmetic(monkeypatch):
-    """fm_memory = gates 1 - alpha*update_scale, scan, RMS norm over D, read-out
-    einsum (reference fm_scan.py:117-131). Checked against a direct numpy
-    statement, with the scan served by the per-timestep PyTorch form."""
+def test_fm_memory_layer_wiring(monkeypatch):
+    """What fm_memory does around the two kernels' worth of work: gates 1 - alpha*update_scale
+    with time last, tokens with time last, read weights alpha*output_scale with time last, and
+    the output back to (B, L, D) (reference fm_scan.py:115-133). The scan is served by the
+    per-timestep PyTorch form and the read-out by the oracle here (no GPU); the result is
+    compared with a direct numpy statement of the layer."""
     import fm_amd.scan.fm_scan as impl
     from fm_amd.scan.fm_pytorch import fm_scan_pytorch
 
+    def readout_on_cpu(states, read, mem_norm, eps):
+        out, normed, _ = O.readout_forward(states.numpy(), read.numpy(), mem_norm, eps)
+        return torch.from_numpy(out), torch.from_numpy(normed)
+
     monkeypatch.setattr(impl, "fm_scan", fm_scan_pytorch)
+    monkeypatch.setattr(impl, "fm_readout", readout_on_cpu)
     gen = torch.Generator().manual_seed(0)
     B, L, M, D = 2, 16, 3, 5
     alpha = torch.softmax(torch.randn(B, L, M, generator=gen, dtype=torch.float64), dim=-1)
@@ -72,7 +85,7 @@ def test_fm_memory_layer_arithmetic(monkeypatch):
     h0 = torch.randn(B, M, D, generator=gen, dtype=torch.float64)
     for norm in (True, False):
         out, states = impl.fm_memory(alpha, us, os_, inp, h0, mem_norm=norm, norm_eps=1e-6)
-        assert out.shape == (B, L, D) and states.shape == (B, M, D, L)
+        assert out.shape == (B, L, D) and states.shape == (B, M, D, L) and out.is_contiguous()
         g = 1.0 - (alpha * us).numpy().transpose(0, 2, 1)
         h = O.forward(g, inp.numpy().transpose(0, 2, 1), h0.numpy())
         if norm:

@@ -231,6 +231,95 @@ def test_torch_loop_autograd_agrees_with_oracle():
     np.testing.assert_allclose(th.grad.numpy(), d_h0, rtol=1e-12, atol=1e-12)
 
 
+# ------------------------------------------------------------------ read-out of the layer
+
+def rand_readout(B, M, D, L, seed):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((B, M, D, L)), rng.standard_normal((B, M, L)),
+            rng.standard_normal((B, D, L)), rng.standard_normal((B, M, D, L)))
+
+
+def test_readout_forward_brute_force_and_invariants():
+    states, read, _, _ = rand_readout(2, 3, 4, 5, seed=21)
+    eps = 1e-3
+    out, normed, inv_rms = O.readout_forward(states, read, True, eps)
+    B, M, D, L = states.shape
+    for b in range(B):          # scalar loops straight from the formulas
+        for t in range(L):
+            for d in range(D):
+                acc = 0.0
+                for m in range(M):
+                    ms = sum(states[b, m, k, t] ** 2 for k in range(D)) / D
+                    acc += read[b, m, t] * states[b, m, d, t] / (ms + eps) ** 0.5
+                assert abs(acc - out[b, d, t]) < 1e-12
+    # eps = 0: unit mean square per slot and step, and invariance to the scale of the states
+    out0, normed0, _ = O.readout_forward(states, read, True, 0.0)
+    np.testing.assert_allclose((normed0 ** 2).mean(axis=2), 1.0, rtol=1e-13)
+    out1, _, _ = O.readout_forward(3.7 * states, read, True, 0.0)
+    np.testing.assert_allclose(out1, out0, rtol=1e-12, atol=1e-13)
+    # D = 1, eps = 0: the norm leaves the sign
+    s1, r1, _, _ = rand_readout(2, 3, 1, 6, seed=22)
+    o1, n1, _ = O.readout_forward(s1, r1, True, 0.0)
+    np.testing.assert_allclose(n1, np.sign(s1), rtol=1e-13)
+    np.testing.assert_allclose(o1[:, 0, :], (r1 * np.sign(s1[:, :, 0, :])).sum(axis=1), rtol=1e-12, atol=1e-13)
+    # no norm, read == 1: the plain sum over the slots
+    o2, n2, r2 = O.readout_forward(states, np.ones_like(read), False)
+    assert r2 is None and n2 is not None
+    np.testing.assert_allclose(o2, states.sum(axis=1), rtol=1e-13, atol=1e-13)
+
+
+@pytest.mark.parametrize("mem_norm", [True, False])
+@pytest.mark.parametrize("with_ext", [False, True])
+def test_readout_backward_matches_finite_differences(mem_norm, with_ext):
+    states, read, out_grad, ext = rand_readout(2, 3, 4, 5, seed=23)
+    ext = ext if with_ext else None
+    eps = 1e-2
+
+    def loss():
+        out, normed, _ = O.readout_forward(states, read, mem_norm, eps)
+        return float((out * out_grad).sum() + ((normed * ext).sum() if with_ext else 0.0))
+
+    d_states, d_read = O.readout_backward(out_grad, ext, read, states, mem_norm, eps)
+    np.testing.assert_allclose(d_states, fd_grad(loss, states), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(d_read, fd_grad(loss, read), rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("mem_norm", [True, False])
+def test_memory_layer_agrees_with_the_operations_the_reference_names(mem_norm):
+    """fm_memory written with the PyTorch operations of fm_scan.py:115-133 (the scan through
+    the per-timestep form) and differentiated by autograd: same outputs and gradients as the
+    oracle's layer, read-out gradients included."""
+    from fm_amd.scan.fm_pytorch import fm_scan_pytorch
+
+    rng = np.random.default_rng(24)
+    B, L, M, D = 2, 9, 3, 4
+    alpha = rng.random((B, L, M))
+    us, osc = rng.random((B, L, 1)), rng.standard_normal((B, L, 1))
+    x = rng.standard_normal((B, L, D))
+    h0 = rng.standard_normal((B, M, D))
+    w_out, w_mem = rng.standard_normal((B, L, D)), rng.standard_normal((B, M, D, L))
+    t = {k: torch.tensor(v, requires_grad=True) for k, v in dict(alpha=alpha, us=us, osc=osc, x=x, h0=h0).items()}
+    write = (t["alpha"] * t["us"]).transpose(1, 2).contiguous()
+    states = fm_scan_pytorch(1.0 - write, t["x"].transpose(1, 2).contiguous(), t["h0"])
+    raw = states
+    if mem_norm:
+        states = states * torch.rsqrt(torch.mean(states ** 2, dim=2, keepdim=True) + 1e-3)
+    out = torch.einsum("blm,bmdl->bld", t["alpha"] * t["osc"], states)
+    o_out, o_states = O.memory_forward(alpha, us, osc, x, h0, mem_norm, 1e-3)
+    np.testing.assert_allclose(out.detach().numpy(), o_out, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(states.detach().numpy(), o_states, rtol=1e-12, atol=1e-12)
+
+    raw.retain_grad()
+    ((out * torch.tensor(w_out)).sum() + (states * torch.tensor(w_mem)).sum()).backward()
+    read = np.ascontiguousarray(np.transpose(alpha * osc, (0, 2, 1)))
+    d_states, d_read = O.readout_backward(np.transpose(w_out, (0, 2, 1)), w_mem, read, raw.detach().numpy(),
+                                          mem_norm, 1e-3)
+    np.testing.assert_allclose(raw.grad.numpy(), d_states, rtol=1e-11, atol=1e-12)
+    # d read reaches alpha and output_scale: d osc[b,l] = sum_m alpha * d_read, checked through osc
+    d_osc = (np.transpose(d_read, (0, 2, 1)) * alpha).sum(axis=2, keepdims=True)
+    np.testing.assert_allclose(t["osc"].grad.numpy(), d_osc, rtol=1e-11, atol=1e-12)
+
+
 # ------------------------------------------------------------------ compiled oracle and port
 
 @pytest.mark.parametrize("plain", [False, True])
