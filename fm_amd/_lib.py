@@ -59,6 +59,8 @@ def load() -> ctypes.CDLL:
     lib.fmscan_readout_dot.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
     lib.fmscan_readout_backward.restype = c_int
     lib.fmscan_readout_backward.argtypes = [c_void_p] * 8 + dims + [c_int, c_void_p]
+    lib.fmscan_swap_last_two.restype = c_int
+    lib.fmscan_swap_last_two.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]
     got = lib.fmscan_abi_version()
     if got != ABI_VERSION:
         raise RuntimeError(f"libfmscan_hip.so has ABI version {got}, this package needs {ABI_VERSION}; "

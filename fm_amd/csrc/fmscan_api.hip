@@ -669,4 +669,27 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
     return launched("read-out (backward)");
 }
 
+int fmscan_swap_last_two(const void* src, void* dst, int64_t B, int64_t R, int64_t C, int element_size,
+                         void* stream) {
+    if (!src || !dst) return fail(FMSCAN_E_NULL, "fmscan_swap_last_two: src and dst must not be NULL");
+    if (B < 1 || R < 1 || C < 1) return fail(FMSCAN_E_SHAPE, "fmscan_swap_last_two: B, R, C must be >= 1");
+    if (element_size != 2 && element_size != 4)
+        return fail(FMSCAN_E_DTYPE, "fmscan_swap_last_two: element size must be 2 or 4 bytes (got %d)", element_size);
+    const int64_t tiles_r = (R + 63) / 64, tiles_c = (C + 63) / 64;
+    if (tiles_r > INT32_MAX || tiles_c > INT32_MAX || (__int128)B * tiles_r * tiles_c > (__int128)INT32_MAX ||
+        (__int128)B * R * C > ((__int128)1 << 46))
+        return fail(FMSCAN_E_SHAPE, "fmscan_swap_last_two: too many tiles for one launch");
+    const int64_t bytes = B * R * C * element_size;
+    if (overlap({"dst", dst, bytes}, {"src", src, bytes}))
+        return fail(FMSCAN_E_ALIAS, "fmscan_swap_last_two: dst overlaps src");
+    const unsigned grid = (unsigned)(B * tiles_r * tiles_c);
+    if (element_size == 2)
+        fmscan::swap_last_two_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, (uint16_t*)dst, R, C, (int32_t)tiles_c, (int32_t)tiles_r);
+    else
+        fmscan::swap_last_two_kernel<uint32_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint32_t*)src, (uint32_t*)dst, R, C, (int32_t)tiles_c, (int32_t)tiles_r);
+    return launched("swap of the last two axes");
+}
+
 }  // extern "C"

@@ -225,4 +225,30 @@ __global__ __launch_bounds__(256) void readout_backward_kernel(
     }
 }
 
+// dst[b, c, r] = src[b, r, c]: the layer takes (B, L, *) tensors and the kernels want time
+// last (reference fm_scan.py:117-118 does it with transpose().contiguous()). 64 x 64
+// tiles through LDS, so that both the reads and the writes are whole 128- or 256-byte
+// runs; U is an unsigned integer of the element's size.
+template <typename U>
+__global__ __launch_bounds__(256) void swap_last_two_kernel(const U* __restrict__ src, U* __restrict__ dst,
+                                                            int64_t R, int64_t C, int32_t tiles_c,
+                                                            int32_t tiles_r) {
+    __shared__ U tile[64][65];
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int64_t per_b = (int64_t)tiles_c * tiles_r;
+    const int64_t b = blockIdx.x / per_b;
+    const int64_t rest = blockIdx.x - b * per_b;
+    const int64_t r0 = (rest / tiles_c) * 64, c0 = (rest % tiles_c) * 64;
+    const U* __restrict__ s = src + b * R * C;
+    U* __restrict__ d = dst + b * R * C;
+#pragma unroll 4
+    for (int i = w; i < 64; i += 4)
+        if (r0 + i < R && c0 + lane < C) tile[i][lane] = s[(r0 + i) * C + c0 + lane];
+    __syncthreads();
+#pragma unroll 4
+    for (int i = w; i < 64; i += 4)
+        if (c0 + i < C && r0 + lane < R) d[(c0 + i) * R + r0 + lane] = tile[lane][i];
+}
+
 }  // namespace fmscan

@@ -417,6 +417,31 @@ def fm_readout(states, read, mem_norm=True, norm_eps=1e-6):
     return output, (normed if mem_norm else states)
 
 
+def _swap_last_two(t):
+    """Dense (B, C, R) copy of a (B, R, C) tensor: transpose(1, 2).contiguous() as one tiled kernel."""
+    _require(t.dim() == 3, "expected a (B, R, C) tensor")
+    _on_gpu("tensor", t, t.device)
+    _require(t.element_size() in (2, 4), f"Unsupported tensor dtype {t.dtype}")
+    t = t.contiguous()
+    B, R, C = t.shape
+    out = torch.empty((B, C, R), dtype=t.dtype, device=t.device)
+    if t.numel():
+        with _on_device(t.device):
+            _lib.check(module.fmscan_swap_last_two(t.data_ptr(), out.data_ptr(), B, R, C, t.element_size(),
+                                                   torch.cuda.current_stream(t.device).cuda_stream))
+    return out
+
+
+class _SwapLastTwo(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, t):
+        return _swap_last_two(t)
+
+    @staticmethod
+    def backward(ctx, grad):
+        return _swap_last_two(grad)
+
+
 def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True,
               norm_eps=1e-6):
     """The Factorization-Memory layer around the scan (reference fm_scan.py:102-133).
@@ -431,10 +456,11 @@ def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem
     Only the (B, L, *) tensors pass through PyTorch operations here; everything of size
     (B, M, D, L) is produced and consumed by the library's kernels.
     """
-    write = (alpha * update_scale).transpose(1, 2).contiguous()  # (B, M, L)
-    tokens = inputs.transpose(1, 2).contiguous()                 # (B, D, L)
+    swap = _SwapLastTwo.apply
+    write = swap(alpha * update_scale)                           # (B, M, L)
+    tokens = swap(inputs)                                        # (B, D, L)
     memory_states = fm_scan(1.0 - write, tokens, initial_state)  # decay gate = 1 - write weight
 
-    read = (alpha * output_scale).transpose(1, 2).contiguous()   # (B, M, L)
+    read = swap(alpha * output_scale)                            # (B, M, L)
     output, memory_states = fm_readout(memory_states, read, mem_norm, norm_eps)  # (B, D, L)
-    return output.transpose(1, 2).contiguous(), memory_states
+    return swap(output), memory_states

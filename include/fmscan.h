@@ -212,6 +212,14 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
                             const float* q, const float* qe, void* state_grad,
                             int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 
+/*
+ * dst[b, c, r] = src[b, r, c] for dense (B, R, C) -> (B, C, R): what fm_memory does to its
+ * (B, L, *) arguments and to its output with transpose(1, 2).contiguous() (reference
+ * fm/scan/fm_scan.py:117-118,131). element_size 2 or 4; src and dst must not overlap.
+ */
+int fmscan_swap_last_two(const void* src, void* dst, int64_t B, int64_t R, int64_t C,
+                         int element_size, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

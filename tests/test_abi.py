@@ -26,7 +26,7 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_reduced",
                                     "fmscan_forward", "fmscan_last_error", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
-                                    "fmscan_reduced_groups", "fmscan_workspace_bytes"]
+                                    "fmscan_reduced_groups", "fmscan_swap_last_two", "fmscan_workspace_bytes"]
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -135,6 +135,11 @@ def test_rejected_readout_arguments(lib):
     assert bw(q=None) == E_NULL                          # the norm's gradient needs q
     assert bw(e=7 * P) == E_NULL                         # ... and qe when ext_grad is given
     assert bw(sg=P) == E_ALIAS
+    sw = lambda src=P, dst=2 * P, es=2, R=5: lib.fmscan_swap_last_two(src, dst, 2, R, 7, es, None)
+    assert sw(dst=None) == E_NULL
+    assert sw(es=8) == E_DTYPE
+    assert sw(R=0) == E_SHAPE
+    assert sw(dst=P + 8) == E_ALIAS
 
 
 def test_workspace_bytes(lib):

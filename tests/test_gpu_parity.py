@@ -525,6 +525,15 @@ def test_readout_in_place_and_determinism(scan):
     assert torch.equal(buf, n1) and torch.equal(out3, out1)
 
 
+def test_swap_last_two_is_exact(scan):
+    from fm_amd.scan.fm_scan import _swap_last_two
+
+    for shape, dt in [((2, 5, 7), torch.float32), ((3, 64, 64), torch.bfloat16), ((1, 1000, 33), torch.float16),
+                      ((2, 129, 2048), torch.bfloat16), ((1, 1, 1), torch.float32)]:
+        t = torch.randn(*shape, device=DEV).to(dt)
+        assert torch.equal(_swap_last_two(t), t.transpose(1, 2).contiguous()), (shape, dt)
+
+
 @pytest.mark.parametrize("dtype,mem_norm", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, True)])
 def test_fm_memory_layer(scan, dtype, mem_norm):
     """The layer on top of the scan, forward and backward (gradients arriving at both

@@ -65,7 +65,8 @@ def test_fm_memory_layer_wiring(monkeypatch):
     """What fm_memory does around the two kernels' worth of work: gates 1 - alpha*update_scale
     with time last, tokens with time last, read weights alpha*output_scale with time last, and
     the output back to (B, L, D) (reference fm_scan.py:115-133). The scan is served by the
-    per-timestep PyTorch form and the read-out by the oracle here (no GPU); the result is
+    per-timestep PyTorch form, the read-out by the oracle and the axis swaps by PyTorch here
+    (no GPU); the result is
     compared with a direct numpy statement of the layer."""
     import fm_amd.scan.fm_scan as impl
     from fm_amd.scan.fm_pytorch import fm_scan_pytorch
@@ -76,6 +77,7 @@ def test_fm_memory_layer_wiring(monkeypatch):
 
     monkeypatch.setattr(impl, "fm_scan", fm_scan_pytorch)
     monkeypatch.setattr(impl, "fm_readout", readout_on_cpu)
+    monkeypatch.setattr(impl, "_swap_last_two", lambda t: t.transpose(1, 2).contiguous())
     gen = torch.Generator().manual_seed(0)
     B, L, M, D = 2, 16, 3, 5
     alpha = torch.softmax(torch.randn(B, L, M, generator=gen, dtype=torch.float64), dim=-1)
