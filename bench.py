@@ -16,6 +16,12 @@ time. `roofline` prices the backward kernel, the dominant one, from HIP events
 recorded around it inside the timed region. `cpu_baseline` times the compiled CPU
 port of the same scan (oracle/fmscan_cpu.c) on this host's cores on a bounded
 row sample of the same workload.
+
+`--workload layer` is a secondary measurement, the Factorization-Memory layer
+around the scan (`fm_memory`: scan, RMS norm over D, read-out over M) at the
+FM-native reading of configuration 5, (B, L, M, D) = (32, 2048, 32, 128) bfloat16:
+one step = forward + backward through autograd; the line also carries each
+kernel's own time and bandwidth from direct calls.
 """
 from __future__ import annotations
 
@@ -129,12 +135,101 @@ def reference_cpu_path(torch, g, x, G):
             "elements_per_s": round(n / (t2 - t0), 1), "fwd_s": round(t1 - t0, 3), "bwd_s": round(t2 - t1, 3)}
 
 
+LAYER = (32, 2048, 32, 128, "bfloat16")  # B, L, M, D
+
+
+def run_layer(torch, args) -> int:
+    import fm.scan.fm_scan as S
+
+    dev = torch.device("cuda", 0)
+    B, L, M, D, dtn = LAYER
+    dt = getattr(torch, dtn)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *sh: torch.randn(*sh, device=dev, generator=gen)
+    alpha = torch.softmax(rn(B, L, M), -1).to(dt).requires_grad_()
+    us = torch.rand(B, L, 1, device=dev, generator=gen).to(dt).requires_grad_()
+    osc = torch.rand(B, L, 1, device=dev, generator=gen).to(dt).requires_grad_()
+    inp = rn(B, L, D).to(dt).requires_grad_()
+    w_out = rn(B, L, D).to(dt)
+    leaves = (alpha, us, osc, inp)
+
+    def step():
+        out, _ = S.fm_memory(alpha, us, osc, inp)
+        out.backward(w_out)
+        for t in leaves:
+            t.grad = None
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # every kernel on its own, through the same Python entry points, HIP events around each
+    N, s = B * M * D * L, alpha.element_size()
+    gates = torch.rand(B, M, L, device=dev, generator=gen).to(dt)
+    tokens = rn(B, D, L).to(dt)
+    read = rn(B, M, L).to(dt)
+    og = rn(B, D, L).to(dt)
+    G = rn(B, M, D, L).to(dt)
+    zeros = torch.zeros(B, M, D, dtype=dt, device=dev)
+    states = torch.empty(B, M, D, L, dtype=dt, device=dev)
+    lib, st = S.module, torch.cuda.current_stream().cuda_stream
+    inv = torch.empty(B, M, L, device=dev)
+    q = torch.empty_like(inv)
+    normed, sg = torch.empty_like(states), torch.empty_like(states)
+    out = torch.empty(B, D, L, dtype=dt, device=dev)
+    code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
+    P = lambda t: t.data_ptr()
+    calls = {
+        "scan_forward_kernel": (s * N, lambda: S.fm_scan_forward(gates, tokens, zeros, states)),
+        "rowdot_kernel (inv_rms)": (s * N, lambda: lib.fmscan_readout_inv_rms(P(states), P(inv), B, M, D, L, code, 1e-6, st)),
+        "readout_forward_kernel": (2 * s * N, lambda: lib.fmscan_readout_forward(
+            P(states), P(inv), P(read), P(normed), P(out), B, M, D, L, code, st)),
+        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, B, M, D, L, code, st)),
+        "readout_backward_kernel": (2 * s * N, lambda: lib.fmscan_readout_backward(
+            P(normed), P(inv), P(read), P(og), None, P(q), None, P(sg), B, M, D, L, code, st)),
+        "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 8, lambda: S.fm_scan_backward_reduced(
+            gates, G, zeros, states, tokens)),
+    }
+    kernels = {}
+    for name, (nbytes, call) in calls.items():
+        for _ in range(3):
+            call()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record()
+        for _ in range(10):
+            call()
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / 10
+        kernels[name] = {"ms": round(ms, 4), "algorithmic_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
+    dom = kernels["scan_backward_reduced_kernel"]
+    result = {
+        "metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
+        "value": round(N / (ms_per_step * 1e-3) / 1e9, 2), "unit": "Gelem/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 storage, f32 arithmetic", "data": "synthetic",
+        "config": {"workload": f"layer: fm_memory (B,L,M,D)=({B},{L},{M},{D}) {dtn}, mem_norm, fwd+bwd via autograd",
+                   "elements": N},
+        "kernels": kernels,
+        "roofline": {"kernel": "scan_backward_reduced_kernel", "bound": "hbm", "achieved": dom["GBps"],
+                     "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom["GBps"] / PEAK_HBM_GBPS, 4),
+                     "algorithmic_bytes": dom["algorithmic_bytes"], "traffic": None},
+    }
+    print(json.dumps(result), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["layer"])
     ap.add_argument("--waves-per-row", type=int, default=0, help="0 = library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--probe", action="store_true",
@@ -156,6 +251,8 @@ def main() -> int:
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.workload == "layer":
+        return run_layer(torch, args)
     B, Cn, T, dtn = WORKLOADS[args.workload]
     g, x, G = make_inputs(torch, args.workload, dev)
     rows = B * Cn
