@@ -527,12 +527,20 @@ __global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
 // (C KiB at a time), which the memory likes, at C tiles of accumulators.
 // HBM traffic: G and h once (2s per element) plus 4/DG bytes per element of partials,
 // against 6s for the unfused kernel plus the two torch.sum passes.
-template <typename T, int DG, int C, int R, bool PLAIN>
+//
+// LAYER: the gradient that arrives at the states is not read but made on the spot from what
+// the layer around the scan holds (reference fm/scan/fm_scan.py:124-131 differentiated):
+//   G[b,m,d,t] = coef_out[b,m,t] * layer_out_grad[b,d,t] - coef_self[b,m,t] * out_grad[b,m,d,t]
+// where `out_grad` then carries the normalised states; the (B, M, D, L) gradient tensor is
+// never written or read.
+template <typename T, int DG, int C, int R, bool PLAIN, bool LAYER>
 __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved,
     const T* __restrict__ tokens, float* __restrict__ gate_partial /* (B, M, NG, L) */,
-    const T* __restrict__ h0, T* __restrict__ h0_grad, int32_t M, int32_t D, int64_t L) {
+    const T* __restrict__ h0, T* __restrict__ h0_grad, const T* __restrict__ coef_out /* (B, M, L) */,
+    const T* __restrict__ coef_self /* (B, M, L) */, const T* __restrict__ layer_out_grad /* (B, D, L) */,
+    int32_t M, int32_t D, int64_t L) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     constexpr int SLICE = TILE / DG;  // elements of a summed tile each wave adds up and stores
@@ -561,6 +569,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
         mycarry[m] = first_prop_grad ? Elem<T>::widen(first_prop_grad[(b * M + m) * D + d]) : 0.0f;
 
     const T* __restrict__ xrow = tokens + (b * D + d) * L;  // never read when PLAIN
+    const T* __restrict__ yrow = layer_out_grad + (b * D + d) * L;  // never read unless LAYER
     T* __restrict__ dxrow = token_grad + (b * D + d) * L;
 
     // What a step loads, exactly as it arrives: anything computed from a loaded value at
@@ -569,6 +578,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     // choice of h[-1] are therefore applied when the entry is used.
     struct Entry {
         u32x4 g, G, h, x;
+        u32x4 co, cs, y;  // LAYER only
         T hb;
     };
     // Where a visit is: chunk `chunk` of row (b, m, d), with the offsets that go with it
@@ -611,6 +621,12 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
         e.h = load16<T, true>(at(hrow + tw));
         e.x = u32x4{0u, 0u, 0u, 0u};
         if constexpr (!PLAIN) e.x = load16<T, false>(at(xrow + tw));
+        e.co = e.cs = e.y = u32x4{0u, 0u, 0u, 0u};
+        if constexpr (LAYER) {
+            e.co = load16<T, false>(at(coef_out + c.goff + tw));
+            e.cs = load16<T, false>(at(coef_self + c.goff + tw));
+            e.y = load16<T, false>(at(yrow + tw));
+        }
         // h just before the tile (h[-1] at the start of the row): one address for the whole wave
         const T* src = tw > 0 ? hrow + (tw - 1) : (h0 != nullptr ? h0 + c.row : hrow);
         e.hb = *src;
@@ -629,7 +645,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
 
     __syncthreads();  // carries are in place
 
-    float dtok[C][E], xf[HOIST ? C : 1][E];
+    float dtok[C][E], xf[HOIST ? C : 1][E], yf[HOIST ? C : 1][E];
 #pragma unroll
     for (int i = 0; i < C; ++i) {
 #pragma unroll
@@ -638,7 +654,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
 #pragma unroll
     for (int i = 0; i < (HOIST ? C : 1); ++i) {
 #pragma unroll
-        for (int j = 0; j < E; ++j) xf[i][j] = 0.0f;
+        for (int j = 0; j < E; ++j) xf[i][j] = yf[i][j] = 0.0f;
     }
     int parity = 0;
     const int32_t visits = nchunks * M;  // the host checks that this fits
@@ -657,7 +673,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                 const int64_t tw = (int64_t)k * TILE;
                 if (tw + TILE > L && tw + lane_off >= L) {  // short or absent tile: nothing there
                     cur.g = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
-                    cur.G = cur.h = cur.x = u32x4{0u, 0u, 0u, 0u};
+                    cur.G = cur.h = cur.x = cur.co = cur.cs = cur.y = u32x4{0u, 0u, 0u, 0u};
                 }
                 const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(cur.hb) : 0.0f;
                 float g[E], G[E], h[E], p[E], xs[E];
@@ -669,6 +685,21 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                         if (m == 0) Elem<T>::unpack(cur.x, xf[i]);  // the M rows share their tokens
                     } else {
                         Elem<T>::unpack(cur.x, xs);
+                    }
+                }
+                if constexpr (LAYER) {
+                    float co[E], cs[E], ys[E];
+                    Elem<T>::unpack(cur.co, co);
+                    Elem<T>::unpack(cur.cs, cs);
+                    if constexpr (HOIST) {
+                        if (m == 0) Elem<T>::unpack(cur.y, yf[i]);  // shared by the M rows, like the tokens
+                    } else {
+                        Elem<T>::unpack(cur.y, ys);
+                    }
+#pragma unroll
+                    for (int j = 0; j < E; ++j) {
+                        const float y = HOIST ? yf[HOIST ? i : 0][j] : ys[j];
+                        G[j] = __builtin_fmaf(-cs[j], G[j], co[j] * y);  // G[] held the normalised state
                     }
                 }
 #pragma unroll

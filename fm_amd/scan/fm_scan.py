@@ -25,7 +25,8 @@ import torch
 from .. import _lib
 
 __all__ = ["fm_scan_forward", "fm_scan_backward", "fm_scan_backward_reduced", "FM_Scan", "fm_scan",
-           "fm_readout_forward", "fm_readout_backward", "FM_Readout", "fm_readout", "fm_memory", "module"]
+           "fm_readout_forward", "fm_readout_backward", "FM_Readout", "fm_readout", "FM_Layer", "fm_layer",
+           "fm_memory", "module"]
 
 _DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16,
            torch.bfloat16: _lib.DTYPE_BF16}
@@ -261,34 +262,40 @@ class FM_Scan(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         tokens, gates, states, initial_state = ctx.saved_tensors
-        B, M, D, L = states.shape
-        assert states.is_contiguous()
-        assert gates.is_contiguous()
+        return _scan_gradients(gates, tokens, states, initial_state, grad_output, ctx.needs_input_grad[2])
 
-        first_prop_grad = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
-        grad_output = grad_output.contiguous()
-        # The reference leaves the initial state's gradient unconnected (fm_scan.py:80-81); it
-        # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
-        d_initial_state = torch.empty_like(first_prop_grad) if ctx.needs_input_grad[2] else None
 
-        if _reduced_ok(gates, tokens, states, grad_output):
-            # both sums are real: one kernel produces d_gates and d_tokens directly
-            d_gates, d_tokens = fm_scan_backward_reduced(
-                gates, grad_output, first_prop_grad, states, tokens,
-                initial_state=initial_state, initial_state_grad=d_initial_state)
-            return d_gates, d_tokens, d_initial_state
+def _scan_gradients(gates, tokens, states, initial_state, grad_output, want_initial_state_grad):
+    """(d_gates (B, M, L), d_tokens (B, D, L), d_initial_state or None) from the gradient of the
+    states (reference fm_scan.py:61-81)."""
+    B, M, D, L = states.shape
+    assert states.is_contiguous()
+    assert gates.is_contiguous()
 
-        per_pair_gates = torch.empty_like(states)   # (B, M, D, L)
-        per_pair_tokens = torch.empty_like(states)  # (B, M, D, L)
-        fm_scan_backward(gates, grad_output, first_prop_grad, per_pair_tokens, states, tokens,
-                         per_pair_gates, initial_state=initial_state,
-                         initial_state_grad=d_initial_state)
+    first_prop_grad = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
+    grad_output = grad_output.contiguous()
+    # The reference leaves the initial state's gradient unconnected (fm_scan.py:80-81); it
+    # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
+    d_initial_state = torch.empty_like(first_prop_grad) if want_initial_state_grad else None
 
-        # (B, M, D, L) -> (B, M, L) and (B, D, L); a sum over an axis of length one
-        # is the same tensor, so it is returned as a view without another pass
-        d_gates = per_pair_gates.view(B, M, L) if D == 1 else per_pair_gates.sum(dim=2)
-        d_tokens = per_pair_tokens.view(B, D, L) if M == 1 else per_pair_tokens.sum(dim=1)
+    if _reduced_ok(gates, tokens, states, grad_output):
+        # both sums are real: one kernel produces d_gates and d_tokens directly
+        d_gates, d_tokens = fm_scan_backward_reduced(
+            gates, grad_output, first_prop_grad, states, tokens,
+            initial_state=initial_state, initial_state_grad=d_initial_state)
         return d_gates, d_tokens, d_initial_state
+
+    per_pair_gates = torch.empty_like(states)   # (B, M, D, L)
+    per_pair_tokens = torch.empty_like(states)  # (B, M, D, L)
+    fm_scan_backward(gates, grad_output, first_prop_grad, per_pair_tokens, states, tokens,
+                     per_pair_gates, initial_state=initial_state,
+                     initial_state_grad=d_initial_state)
+
+    # (B, M, D, L) -> (B, M, L) and (B, D, L); a sum over an axis of length one
+    # is the same tensor, so it is returned as a view without another pass
+    d_gates = per_pair_gates.view(B, M, L) if D == 1 else per_pair_gates.sum(dim=2)
+    d_tokens = per_pair_tokens.view(B, D, L) if M == 1 else per_pair_tokens.sum(dim=1)
+    return d_gates, d_tokens, d_initial_state
 
 
 def fm_scan(gates, tokens, initial_state=None):
@@ -417,6 +424,94 @@ def fm_readout(states, read, mem_norm=True, norm_eps=1e-6):
     return output, (normed if mem_norm else states)
 
 
+class FM_Layer(torch.autograd.Function):
+    """output, memory_states = FM_Layer.apply(gates, tokens, initial_state, read, mem_norm, norm_eps)
+
+    Scan, RMS norm and read-out of the layer as one node of the autograd graph (reference
+    fm_scan.py:121-131): gates, read (B, M, L), tokens (B, D, L), initial_state (B, M, D) or
+    None -> output (B, D, L), memory states as the layer returns them (B, M, D, L). One node,
+    because backward then needs no (B, M, D, L) gradient tensor between the read-out and
+    the scan: when nothing but `output` feeds the loss, the scan's backward kernel makes that
+    gradient itself from the output's gradient, the normalised states and two per-slot
+    coefficient vectors.
+    """
+
+    @staticmethod
+    def forward(ctx, gates, tokens, initial_state, read, mem_norm=True, norm_eps=1e-6):
+        B_g, M, L_g = gates.shape
+        B, D, L = tokens.shape
+        assert L_g == L
+        assert B_g == B
+        assert gates.is_contiguous()
+        assert tokens.is_contiguous()
+        given_state = initial_state is not None
+        if given_state:
+            assert initial_state.shape == (B, M, D)
+            assert initial_state.is_contiguous()
+        else:
+            initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
+        states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
+        fm_scan_forward(gates, tokens, initial_state, states)
+        output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps)
+        ctx.mem_norm = bool(mem_norm)
+        ctx.save_for_backward(tokens, gates, states, initial_state if given_state else None, read, normed,
+                              inv_rms)
+        ctx.set_materialize_grads(False)
+        return output, (normed if mem_norm else states)
+
+    @staticmethod
+    def backward(ctx, out_grad, ext_grad):
+        tokens, gates, states, initial_state, read, normed, inv_rms = ctx.saved_tensors
+        if out_grad is None and ext_grad is None:
+            return None, None, None, None, None, None
+        B, M, D, L = states.shape
+        want_h0 = ctx.needs_input_grad[2]
+        states_n = normed if ctx.mem_norm else states
+        if out_grad is not None:
+            out_grad = out_grad.contiguous()
+
+        if ext_grad is None and _reduced_ok(gates, tokens, states, states_n) and _aligned(read, out_grad):
+            # only the output feeds the loss: the states' gradient is made inside the scan's kernel
+            dev, code = states.device, _dtype_code(states)
+            q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
+            groups = module.fmscan_reduced_groups(D)
+            d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
+            partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
+            zeros = torch.zeros((B, M, D), dtype=gates.dtype, device=dev)
+            d_h0 = torch.empty_like(zeros) if want_h0 else None
+            with _on_device(dev):
+                stream = torch.cuda.current_stream(dev).cuda_stream
+                _lib.check(module.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(), None,
+                                                     q.data_ptr(), None, B, M, D, L, code, stream))
+                if ctx.mem_norm:
+                    coef = inv_rms * read  # float32
+                    coef_out = coef.to(gates.dtype)
+                    coef_self = (coef * q).mul_(1.0 / D).to(gates.dtype)
+                else:
+                    coef_out, coef_self = read, torch.zeros_like(read)
+                _lib.check(module.fmscan_backward_layer(
+                    gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
+                    out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(), states.data_ptr(),
+                    tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0), B, M, D, L, code, 0,
+                    stream))
+            return partial.sum(dim=2).to(gates.dtype), d_tokens, d_h0, q.to(gates.dtype), None, None
+
+        if out_grad is None:
+            out_grad = torch.zeros((B, D, L), dtype=states.dtype, device=states.device)
+        # the norm's gradient never sees ext_grad without the norm: the states are returned as they are
+        state_grad, read_grad = fm_readout_backward(
+            out_grad, ext_grad.contiguous() if (ext_grad is not None and ctx.mem_norm) else None, read, states_n,
+            inv_rms)
+        if ext_grad is not None and not ctx.mem_norm:
+            state_grad += ext_grad
+        d_gates, d_tokens, d_h0 = _scan_gradients(gates, tokens, states, initial_state, state_grad, want_h0)
+        return d_gates, d_tokens, d_h0, read_grad, None, None
+
+
+def _aligned(*tensors):
+    return all(t.data_ptr() % 16 == 0 for t in tensors)
+
+
 def _swap_last_two(t):
     """Dense (B, C, R) copy of a (B, R, C) tensor: transpose(1, 2).contiguous() as one tiled kernel."""
     _require(t.dim() == 3, "expected a (B, R, C) tensor")
@@ -442,6 +537,11 @@ class _SwapLastTwo(torch.autograd.Function):
         return _swap_last_two(grad)
 
 
+def fm_layer(gates, tokens, initial_state, read, mem_norm=True, norm_eps=1e-6):
+    """(output (B, D, L), memory states (B, M, D, L)) of scan + RMS norm + read-out, time last."""
+    return FM_Layer.apply(gates, tokens, initial_state, read, mem_norm, norm_eps)
+
+
 def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True,
               norm_eps=1e-6):
     """The Factorization-Memory layer around the scan (reference fm_scan.py:102-133).
@@ -459,8 +559,7 @@ def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem
     swap = _SwapLastTwo.apply
     write = swap(alpha * update_scale)                           # (B, M, L)
     tokens = swap(inputs)                                        # (B, D, L)
-    memory_states = fm_scan(1.0 - write, tokens, initial_state)  # decay gate = 1 - write weight
-
     read = swap(alpha * output_scale)                            # (B, M, L)
-    output, memory_states = fm_readout(memory_states, read, mem_norm, norm_eps)  # (B, D, L)
+    # decay gate = 1 - write weight; scan, norm and read-out in one autograd node
+    output, memory_states = fm_layer(1.0 - write, tokens, initial_state, read, mem_norm, norm_eps)
     return swap(output), memory_states

@@ -167,6 +167,27 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
                             int dtype, unsigned flags, void* stream);
 
 /*
+ * fmscan_backward_reduced for a scan inside the Factorization-Memory layer (reference
+ * fm/scan/fm_scan.py:121-131 differentiated as one piece): the gradient arriving at the
+ * scanned states is not passed as a (B, M, D, L) tensor but made inside the kernel,
+ *   G[b,m,d,t] = coef_out[b,m,t] * out_grad[b,d,t] - coef_self[b,m,t] * states_n[b,m,d,t],
+ * which is the gradient of the RMS norm and read-out (fmscan_readout_backward without
+ * ext_grad) when coef_out = inv_rms * read and coef_self = inv_rms * read * q / D, and of
+ * the read-out alone when coef_out = read, coef_self = 0 and states_n = cached_output.
+ *   states_n   (B, M, D, L)  the normalised states      coef_out, coef_self  (B, M, L)
+ *   out_grad   (B, D, L)     gradient of the layer's output, time last
+ * all of the call's dtype. Everything else, and the limits, as fmscan_backward_reduced.
+ */
+int fmscan_backward_layer(const void* gates, const void* states_n,
+                          const void* coef_out, const void* coef_self, const void* out_grad,
+                          const void* first_prop_grad, void* token_grad,
+                          const void* cached_output, const void* input_tokens,
+                          float* gate_grad_partial,
+                          const void* initial_state, void* initial_state_grad,
+                          int64_t B, int64_t M, int64_t D, int64_t L,
+                          int dtype, unsigned flags, void* stream);
+
+/*
  * The read-out of the Factorization-Memory layer (reference fm/scan/fm_scan.py:124-131,
  * inside fm_memory): RMS norm of the scanned states over the D axis of every memory slot
  *   inv_rms[b,m,t] = rsqrt(mean_d states[b,m,d,t]^2 + eps)            (:126)

@@ -23,7 +23,8 @@ def declared_functions():
 
 
 def test_header_declares_the_expected_entry_points():
-    assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_reduced",
+    assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
+                                    "fmscan_backward_reduced",
                                     "fmscan_forward", "fmscan_last_error", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
                                     "fmscan_reduced_groups", "fmscan_swap_last_two", "fmscan_workspace_bytes"]
@@ -97,6 +98,13 @@ def test_rejected_arguments(lib):
     assert red(dx=4 * P) == E_ALIAS
     assert red(L=7) == _const("FMSCAN_E_UNALIGNED")
     assert red(g=P + 4) == _const("FMSCAN_E_UNALIGNED")
+    lay = lambda **k: lib.fmscan_backward_layer(
+        P, 2 * P, k.get("co", 7 * P), k.get("cs", 8 * P), k.get("og", 9 * P), None, k.get("dx", 3 * P), 4 * P, 5 * P,
+        6 * P, None, None, 2, 2, 2, 8, 0, 0, None)
+    assert lay(co=None) == E_NULL
+    assert lay(cs=None) == E_NULL
+    assert lay(og=None) == E_NULL
+    assert lay(dx=9 * P) == E_ALIAS                   # token_grad on top of the layer's out_grad
     assert lib.fmscan_reduced_groups(128) == 16 and lib.fmscan_reduced_groups(9) == 2
     assert fwd(lib, out=P) == E_ALIAS                 # out on top of gates
     assert fwd(lib, out=2 * P + 16) == E_ALIAS        # out inside tokens

@@ -525,6 +525,46 @@ def test_readout_in_place_and_determinism(scan):
     assert torch.equal(buf, n1) and torch.equal(out3, out1)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mem_norm", [True, False])
+def test_layer_backward_kernel_equals_the_two_step_route(scan, dtype, mem_norm):
+    """fmscan_backward_layer (states' gradient made inside the scan's backward kernel) against
+    fmscan_readout_backward followed by fmscan_backward_reduced, and against the oracle."""
+    for (B, M, D, L) in [(2, 3, 5, 512), (1, 2, 16, 8), (2, 4, 24, 4096), (1, 5, 9, 1000), (2, 3, 4, 2568)]:
+        gen = torch.Generator().manual_seed(7 * M + D)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        read = torch.randn(B, M, L, generator=gen).to(dtype).to(DEV)
+        og = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        zeros = torch.zeros(B, M, D, dtype=dtype, device=DEV)
+        states = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        scan.fm_scan_forward(g, x, h0, states)
+        out, normed, inv_rms = scan.fm_readout_forward(states, read, mem_norm, 1e-5)
+        states_n = normed if mem_norm else states
+        # two steps: a (B, M, D, L) gradient in between
+        sg, d_read = scan.fm_readout_backward(og, None, read, states_n, inv_rms)
+        dh0_a = torch.empty_like(zeros)
+        dg_a, dx_a = scan.fm_scan_backward_reduced(g, sg, zeros, states, x, initial_state=h0, initial_state_grad=dh0_a)
+        # one step, through the autograd node
+        leaves = [t.clone().requires_grad_() for t in (g, x, h0, read)]
+        out_b, _ = scan.fm_layer(*leaves[:3], leaves[3], mem_norm, 1e-5)
+        assert torch.equal(out_b, out)
+        out_b.backward(og)
+        tag = f"{(B, M, D, L)} {dtype} norm={mem_norm}"
+        tol = 4 * TOL[dtype]
+        check(tag + " d_gates vs two steps", leaves[0].grad, dg_a.double().cpu().numpy(), tol)
+        check(tag + " d_tokens vs two steps", leaves[1].grad, dx_a.double().cpu().numpy(), tol)
+        check(tag + " d_initial_state vs two steps", leaves[2].grad, dh0_a.double().cpu().numpy(), tol)
+        check(tag + " d_read vs two steps", leaves[3].grad, d_read.double().cpu().numpy(), tol)
+        # oracle: read-out gradient, then the scan's
+        o_sg, o_dr = O.readout_backward(og, None, read, states, mem_norm, 1e-5)
+        tg, gg, delta = O.backward_per_row(g, o_sg, states, x, None, h0, False)
+        check(tag + " d_gates", leaves[0].grad, gg.sum(axis=2), tol)
+        check(tag + " d_tokens", leaves[1].grad, tg.sum(axis=1), tol)
+        check(tag + " d_read", leaves[3].grad, o_dr, tol)
+
+
 def test_swap_last_two_is_exact(scan):
     from fm_amd.scan.fm_scan import _swap_last_two
 
@@ -534,11 +574,14 @@ def test_swap_last_two_is_exact(scan):
         assert torch.equal(_swap_last_two(t), t.transpose(1, 2).contiguous()), (shape, dt)
 
 
+@pytest.mark.parametrize("mem_in_loss", [True, False])
 @pytest.mark.parametrize("dtype,mem_norm", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, True)])
-def test_fm_memory_layer(scan, dtype, mem_norm):
-    """The layer on top of the scan, forward and backward (gradients arriving at both
-    returned tensors), against the float64 oracle layer / the same layer written with the
-    PyTorch operations the reference names, in float64 on the CPU."""
+def test_fm_memory_layer(scan, dtype, mem_norm, mem_in_loss):
+    """The layer on top of the scan, forward and backward, against the float64 oracle layer /
+    the same layer written with the PyTorch operations the reference names, in float64 on the
+    CPU. With the returned memory states in the loss the states' gradient is a tensor between
+    the read-out's and the scan's backward kernels; with the output alone it is made inside
+    the scan's backward kernel."""
     from fm.scan.fm_pytorch import fm_scan_pytorch
 
     B, L, M, D = 2, 512, 4, 24
@@ -567,7 +610,10 @@ def test_fm_memory_layer(scan, dtype, mem_norm):
             np.testing.assert_allclose(y.detach().numpy(), o_y, rtol=1e-10, atol=1e-10)
             np.testing.assert_allclose(mem.detach().numpy(), o_mem, rtol=1e-10, atol=1e-10)
         acc = torch.float64 if name == "ref" else torch.float32
-        (y.to(acc).square().sum() + (mem.to(acc) * w_mem.to(dev).to(acc)).sum()).backward()
+        loss = y.to(acc).square().sum()
+        if mem_in_loss:
+            loss = loss + (mem.to(acc) * w_mem.to(dev).to(acc)).sum()
+        loss.backward()
         outs[name] = [y.detach(), mem.detach(), a.grad, u.grad, o.grad, i.grad, h0.grad]
     tol = 1e-4 if dtype == torch.float32 else 3e-2
     for t_gpu, t_ref, what in zip(outs["gpu"], outs["ref"], ("output", "memory", "d_alpha", "d_update_scale",

@@ -68,15 +68,16 @@ def test_fm_memory_layer_wiring(monkeypatch):
     per-timestep PyTorch form, the read-out by the oracle and the axis swaps by PyTorch here
     (no GPU); the result is
     compared with a direct numpy statement of the layer."""
+    # (scan + norm + read-out are one call in the product, `fm_layer`: that is what is served here)
     import fm_amd.scan.fm_scan as impl
     from fm_amd.scan.fm_pytorch import fm_scan_pytorch
 
-    def readout_on_cpu(states, read, mem_norm, eps):
+    def layer_on_cpu(gates, tokens, initial_state, read, mem_norm, eps):
+        states = fm_scan_pytorch(gates, tokens, initial_state)
         out, normed, _ = O.readout_forward(states.numpy(), read.numpy(), mem_norm, eps)
         return torch.from_numpy(out), torch.from_numpy(normed)
 
-    monkeypatch.setattr(impl, "fm_scan", fm_scan_pytorch)
-    monkeypatch.setattr(impl, "fm_readout", readout_on_cpu)
+    monkeypatch.setattr(impl, "fm_layer", layer_on_cpu)
     monkeypatch.setattr(impl, "_swap_last_two", lambda t: t.transpose(1, 2).contiguous())
     gen = torch.Generator().manual_seed(0)
     B, L, M, D = 2, 16, 3, 5
