@@ -182,6 +182,8 @@ def run_layer(torch, args) -> int:
     q = torch.empty_like(inv)
     normed, sg = torch.empty_like(states), torch.empty_like(states)
     out = torch.empty(B, D, L, dtype=dt, device=dev)
+    coef, dtok = rn(B, M, L).to(dt), torch.empty(B, D, L, dtype=dt, device=dev)
+    partial = torch.empty(B, M, lib.fmscan_reduced_groups(D), L, device=dev)
     code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
     P = lambda t: t.data_ptr()
     calls = {
@@ -194,6 +196,11 @@ def run_layer(torch, args) -> int:
             P(normed), P(inv), P(read), P(og), None, P(q), None, P(sg), B, M, D, L, code, st)),
         "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 8, lambda: S.fm_scan_backward_reduced(
             gates, G, zeros, states, tokens)),
+        # what the layer's backward runs when only its output feeds the loss: the kernel above in
+        # the form that makes the states' gradient itself (no readout_backward_kernel, no G)
+        "scan_backward_reduced_kernel (layer form)": (2 * s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
+            P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), P(states), P(tokens), P(partial),
+            None, None, B, M, D, L, code, 0, st)),
     }
     kernels = {}
     for name, (nbytes, call) in calls.items():
@@ -207,7 +214,7 @@ def run_layer(torch, args) -> int:
         torch.cuda.synchronize()
         ms = ev[0].elapsed_time(ev[1]) / 10
         kernels[name] = {"ms": round(ms, 4), "algorithmic_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
-    dom = kernels["scan_backward_reduced_kernel"]
+    dom = kernels["scan_backward_reduced_kernel (layer form)"]
     result = {
         "metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
         "value": round(N / (ms_per_step * 1e-3) / 1e9, 2), "unit": "Gelem/s", "n_gpus": 1, "steps": args.steps,
@@ -216,7 +223,7 @@ def run_layer(torch, args) -> int:
         "config": {"workload": f"layer: fm_memory (B,L,M,D)=({B},{L},{M},{D}) {dtn}, mem_norm, fwd+bwd via autograd",
                    "elements": N},
         "kernels": kernels,
-        "roofline": {"kernel": "scan_backward_reduced_kernel", "bound": "hbm", "achieved": dom["GBps"],
+        "roofline": {"kernel": "scan_backward_reduced_kernel (layer form)", "bound": "hbm", "achieved": dom["GBps"],
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom["GBps"] / PEAK_HBM_GBPS, 4),
                      "algorithmic_bytes": dom["algorithmic_bytes"], "traffic": None},
     }
