@@ -191,7 +191,7 @@ def run_layer(torch, args) -> int:
         "rowdot_kernel (inv_rms)": (s * N, lambda: lib.fmscan_readout_inv_rms(P(states), P(inv), B, M, D, L, code, 1e-6, st)),
         "readout_forward_kernel": (2 * s * N, lambda: lib.fmscan_readout_forward(
             P(states), P(inv), P(read), P(normed), P(out), B, M, D, L, code, st)),
-        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, B, M, D, L, code, st)),
+        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, None, None, None, None, B, M, D, L, code, st)),
         "readout_backward_kernel": (2 * s * N, lambda: lib.fmscan_readout_backward(
             P(normed), P(inv), P(read), P(og), None, P(q), None, P(sg), B, M, D, L, code, st)),
         "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 8, lambda: S.fm_scan_backward_reduced(

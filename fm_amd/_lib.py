@@ -58,7 +58,11 @@ def load() -> ctypes.CDLL:
     lib.fmscan_readout_forward.restype = c_int
     lib.fmscan_readout_forward.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
     lib.fmscan_readout_dot.restype = c_int
-    lib.fmscan_readout_dot.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
+    lib.fmscan_readout_dot.argtypes = [c_void_p] * 9 + dims + [c_int, c_void_p]
+    lib.fmscan_layer_prepare.restype = c_int
+    lib.fmscan_layer_prepare.argtypes = [c_void_p] * 5 + [c_int64] * 3 + [c_int, c_void_p]
+    lib.fmscan_layer_finish.restype = c_int
+    lib.fmscan_layer_finish.argtypes = [c_void_p, c_int64] + [c_void_p] * 7 + [c_int64] * 3 + [c_int, c_void_p]
     lib.fmscan_readout_backward.restype = c_int
     lib.fmscan_readout_backward.argtypes = [c_void_p] * 8 + dims + [c_int, c_void_p]
     lib.fmscan_swap_last_two.restype = c_int

@@ -584,8 +584,8 @@ int fmscan_readout_inv_rms(const void* states, float* inv_rms, int64_t B, int64_
         with_bool(vec, [&](auto vt) {
             fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kSumSq, false, decltype(vt)::value>
                 <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>((const T*)states, nullptr, nullptr, inv_rms,
-                                                                      nullptr, (int32_t)M, (int32_t)D, L,
-                                                                      rs.tiles, eps);
+                                                                      nullptr, nullptr, nullptr, nullptr, nullptr,
+                                                                      (int32_t)M, (int32_t)D, L, rs.tiles, eps);
         });
     });
     return launched("read-out (inverse rms)");
@@ -628,20 +628,28 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
 }
 
 int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad, float* q, float* qe,
-                       int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
+                       const float* inv_rms, const void* read, void* coef_out, void* coef_self, int64_t B,
+                       int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
     ReadoutShape rs;
     if (int rc = parse_readout("fmscan_readout_dot", B, M, D, L, dtype, &rs)) return rc;
     if (!states_n || !out_grad || !q)
         return fail(FMSCAN_E_NULL, "fmscan_readout_dot: states_n, out_grad and q must not be NULL");
     if (ext_grad && !qe) return fail(FMSCAN_E_NULL, "fmscan_readout_dot: qe must not be NULL with ext_grad");
-    const int64_t full = B * M * D * L * rs.esize;
-    const Range outs[] = {{"q", q, B * M * L * 4}, {"qe", ext_grad ? qe : nullptr, B * M * L * 4}};
+    if ((coef_out || coef_self) && (!coef_out || !coef_self || !read))
+        return fail(FMSCAN_E_NULL, "fmscan_readout_dot: coef_out, coef_self and read go together");
+    const int64_t full = B * M * D * L * rs.esize, slot = B * M * L;
+    const Range outs[] = {{"q", q, slot * 4}, {"qe", ext_grad ? qe : nullptr, slot * 4},
+                          {"coef_out", coef_out, slot * rs.esize}, {"coef_self", coef_self, slot * rs.esize}};
     const Range ins[] = {{"states_n", states_n, full}, {"out_grad", out_grad, B * D * L * rs.esize},
-                         {"ext_grad", ext_grad, full}};
+                         {"ext_grad", ext_grad, full}, {"inv_rms", coef_out ? inv_rms : nullptr, slot * 4},
+                         {"read", coef_out ? read : nullptr, slot * rs.esize}};
     for (const Range& o : outs)
         for (const Range& in : ins)
             if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", o.name, in.name);
-    if (overlap(outs[0], outs[1])) return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: q overlaps qe");
+    for (int i = 0; i < 4; ++i)
+        for (int j = i + 1; j < 4; ++j)
+            if (overlap(outs[i], outs[j]))
+                return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", outs[i].name, outs[j].name);
     const bool vec = vector_path(rs, {states_n, out_grad, ext_grad});
     const unsigned grid = (unsigned)(B * M * rs.tiles);
     with_dtype(dtype, [&](auto tt) {
@@ -649,9 +657,9 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
         with_bool(ext_grad != nullptr, [&](auto et) {
             with_bool(vec, [&](auto vt) {
                 fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kDot, decltype(et)::value, decltype(vt)::value>
-                    <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>((const T*)states_n, (const T*)out_grad,
-                                                                          (const T*)ext_grad, q, qe, (int32_t)M,
-                                                                          (int32_t)D, L, rs.tiles, 0.0f);
+                    <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>(
+                        (const T*)states_n, (const T*)out_grad, (const T*)ext_grad, q, qe, inv_rms, (const T*)read,
+                        (T*)coef_out, (T*)coef_self, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
             });
         });
     });
@@ -701,6 +709,70 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
         });
     });
     return launched("read-out (backward)");
+}
+
+int fmscan_layer_prepare(const void* alpha, const void* update_scale, const void* output_scale, void* gates,
+                         void* read, int64_t B, int64_t L, int64_t M, int dtype, void* stream) {
+    Problem pb;
+    if (int rc = parse(B, M, 1, L, dtype, 0, &pb)) return rc;
+    if (!alpha || !update_scale || !output_scale || !gates || !read)
+        return fail(FMSCAN_E_NULL, "fmscan_layer_prepare: no argument may be NULL");
+    const int64_t tiles_t = (L + 63) / 64, tiles_m = (M + 63) / 64;
+    if ((__int128)B * tiles_t * tiles_m > (__int128)INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "fmscan_layer_prepare: too many tiles for one launch");
+    const int64_t big = B * L * M * pb.esize, small = B * L * pb.esize;
+    const Range outs[] = {{"gates", gates, big}, {"read", read, big}};
+    const Range ins[] = {{"alpha", alpha, big}, {"update_scale", update_scale, small},
+                         {"output_scale", output_scale, small}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "fmscan_layer_prepare: %s overlaps %s", o.name, in.name);
+    if (overlap(outs[0], outs[1])) return fail(FMSCAN_E_ALIAS, "fmscan_layer_prepare: gates overlaps read");
+    const unsigned grid = (unsigned)(B * tiles_t * tiles_m);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        fmscan::layer_prepare_kernel<T><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const T*)alpha, (const T*)update_scale, (const T*)output_scale, (T*)gates, (T*)read, L, M,
+            (int32_t)tiles_t, (int32_t)tiles_m);
+    });
+    return launched("layer (prepare)");
+}
+
+int fmscan_layer_finish(const float* gate_grad_partial, int64_t G, const float* read_grad, const void* alpha,
+                        const void* update_scale, const void* output_scale, void* alpha_grad,
+                        void* update_scale_grad, void* output_scale_grad, int64_t B, int64_t L, int64_t M,
+                        int dtype, void* stream) {
+    Problem pb;
+    if (int rc = parse(B, M, 1, L, dtype, 0, &pb)) return rc;
+    if (G < 1 || G > INT32_MAX) return fail(FMSCAN_E_SHAPE, "fmscan_layer_finish: G must be >= 1");
+    if (!gate_grad_partial || !read_grad || !alpha || !update_scale || !output_scale || !alpha_grad ||
+        !update_scale_grad || !output_scale_grad)
+        return fail(FMSCAN_E_NULL, "fmscan_layer_finish: no argument may be NULL");
+    const int64_t tiles_t = (L + 63) / 64;
+    if ((__int128)B * tiles_t > (__int128)INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "fmscan_layer_finish: too many tiles for one launch");
+    const int64_t big = B * L * M * pb.esize, small = B * L * pb.esize;
+    const Range outs[] = {{"alpha_grad", alpha_grad, big}, {"update_scale_grad", update_scale_grad, small},
+                          {"output_scale_grad", output_scale_grad, small}};
+    const Range ins[] = {{"gate_grad_partial", gate_grad_partial, B * M * G * L * 4},
+                         {"read_grad", read_grad, B * M * L * 4}, {"alpha", alpha, big},
+                         {"update_scale", update_scale, small}, {"output_scale", output_scale, small}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "fmscan_layer_finish: %s overlaps %s", o.name, in.name);
+    for (int i = 0; i < 3; ++i)
+        for (int j = i + 1; j < 3; ++j)
+            if (overlap(outs[i], outs[j]))
+                return fail(FMSCAN_E_ALIAS, "fmscan_layer_finish: %s overlaps %s", outs[i].name, outs[j].name);
+    const unsigned grid = (unsigned)(B * tiles_t);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        fmscan::layer_finish_kernel<T><<<grid, 256, 0, (hipStream_t)stream>>>(
+            gate_grad_partial, (int32_t)G, read_grad, (const T*)alpha, (const T*)update_scale,
+            (const T*)output_scale, (T*)alpha_grad, (T*)update_scale_grad, (T*)output_scale_grad, L, M,
+            (int32_t)tiles_t);
+    });
+    return launched("layer (finish)");
 }
 
 int fmscan_swap_last_two(const void* src, void* dst, int64_t B, int64_t R, int64_t C, int element_size,

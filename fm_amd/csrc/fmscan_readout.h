@@ -50,8 +50,9 @@ template <typename T, int WV, RowDot MODE, bool EXT, bool VEC>
 __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
     const T* __restrict__ states /* (B, M, D, L) */, const T* __restrict__ out_grad /* (B, D, L) */,
     const T* __restrict__ ext_grad /* (B, M, D, L) */, float* __restrict__ result /* (B, M, L) */,
-    float* __restrict__ result_ext /* (B, M, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles,
-    float eps) {
+    float* __restrict__ result_ext /* (B, M, L) */, const float* __restrict__ inv_rms /* (B, M, L) */,
+    const T* __restrict__ read /* (B, M, L) */, T* __restrict__ coef_out, T* __restrict__ coef_self,
+    int32_t M, int32_t D, int64_t L, int32_t tiles, float eps) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     __shared__ float part[EXT ? 2 : 1][WV][TILE];
@@ -102,6 +103,15 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
         if constexpr (MODE == RowDot::kSumSq) s = 1.0f / __builtin_sqrtf(s / (float)D + eps);
         result[bm * L + t] = s;
         if constexpr (EXT) result_ext[bm * L + t] = se;
+        if constexpr (MODE == RowDot::kDot) {
+            // what scan_backward_reduced_kernel<..., LAYER> takes: the states' gradient is
+            // coef_out * out_grad - coef_self * normalised state
+            if (coef_out != nullptr) {
+                const float c = (inv_rms ? inv_rms[bm * L + t] : 1.0f) * (float)read[bm * L + t];
+                coef_out[bm * L + t] = (T)c;
+                coef_self[bm * L + t] = (T)(inv_rms ? c * s / (float)D : 0.0f);
+            }
+        }
     }
 }
 
@@ -249,6 +259,97 @@ __global__ __launch_bounds__(256) void swap_last_two_kernel(const U* __restrict_
 #pragma unroll 4
     for (int i = w; i < 64; i += 4)
         if (c0 + i < C && r0 + lane < R) d[(c0 + i) * R + r0 + lane] = tile[lane][i];
+}
+
+// gates[b, m, t] = 1 - alpha[b, t, m] * update_scale[b, t], read[b, m, t] = alpha[b, t, m] *
+// output_scale[b, t] (reference fm_scan.py:116,118-119,130: two products, two transposed
+// copies and a subtraction). 64 x 64 tiles of (t, m) through LDS; float32 arithmetic, one
+// rounding. grid: B * tiles_t * tiles_m.
+template <typename T>
+__global__ __launch_bounds__(256) void layer_prepare_kernel(
+    const T* __restrict__ alpha /* (B, L, M) */, const T* __restrict__ update_scale /* (B, L) */,
+    const T* __restrict__ output_scale /* (B, L) */, T* __restrict__ gates /* (B, M, L) */,
+    T* __restrict__ read /* (B, M, L) */, int64_t L, int64_t M, int32_t tiles_t, int32_t tiles_m) {
+    __shared__ float tg[64][65], tr[64][65];
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int64_t per_b = (int64_t)tiles_t * tiles_m;
+    const int64_t b = blockIdx.x / per_b;
+    const int64_t rest = blockIdx.x - b * per_b;
+    const int64_t t0 = (rest / tiles_m) * 64, m0 = (rest % tiles_m) * 64;
+#pragma unroll 4
+    for (int i = w; i < 64; i += 4) {
+        const int64_t t = t0 + i;
+        if (t < L && m0 + lane < M) {
+            const float a = (float)alpha[(b * L + t) * M + m0 + lane];
+            tg[i][lane] = 1.0f - a * (float)update_scale[b * L + t];
+            tr[i][lane] = a * (float)output_scale[b * L + t];
+        }
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int i = w; i < 64; i += 4) {
+        const int64_t m = m0 + i;
+        if (m < M && t0 + lane < L) {
+            gates[(b * M + m) * L + t0 + lane] = (T)tg[lane][i];
+            read[(b * M + m) * L + t0 + lane] = (T)tr[lane][i];
+        }
+    }
+}
+
+// The gradients of those lines: with dg = sum over the G partials of the gates' gradient
+// and dr the gradient of read (both (B, M, L), float32),
+//   alpha_grad[b,t,m] = dr * output_scale - dg * update_scale
+//   update_scale_grad[b,t] = -sum_m dg * alpha,   output_scale_grad[b,t] = sum_m dr * alpha.
+// A block is one b and 64 consecutive t; its four waves share the m of each 64-wide tile.
+template <typename T>
+__global__ __launch_bounds__(256) void layer_finish_kernel(
+    const float* __restrict__ gate_grad_partial /* (B, M, G, L) */, int32_t G,
+    const float* __restrict__ read_grad /* (B, M, L) */, const T* __restrict__ alpha /* (B, L, M) */,
+    const T* __restrict__ update_scale, const T* __restrict__ output_scale, T* __restrict__ alpha_grad,
+    T* __restrict__ update_scale_grad, T* __restrict__ output_scale_grad, int64_t L, int64_t M,
+    int32_t tiles_t) {
+    __shared__ float ta[64][65], td[64][65], red[2][4][64];
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int64_t b = blockIdx.x / tiles_t;
+    const int64_t t0 = (blockIdx.x - b * tiles_t) * 64;
+    const int64_t t = t0 + lane;  // the step this lane owns in the (m, t) view
+    const float us = t < L ? (float)update_scale[b * L + t] : 0.0f;
+    const float os = t < L ? (float)output_scale[b * L + t] : 0.0f;
+    float d_us = 0.0f, d_os = 0.0f;
+    for (int64_t m0 = 0; m0 < M; m0 += 64) {
+        __syncthreads();  // the tiles of the round before are no longer read
+#pragma unroll 4
+        for (int i = w; i < 64; i += 4)  // alpha tile, rows are steps
+            ta[i][lane] = (t0 + i < L && m0 + lane < M) ? (float)alpha[(b * L + t0 + i) * M + m0 + lane] : 0.0f;
+        __syncthreads();
+#pragma unroll 2
+        for (int i = w; i < 64; i += 4) {  // row i of this round: slot m0 + i, lanes are steps
+            const int64_t m = m0 + i;
+            float dg = 0.0f, dr = 0.0f;
+            if (m < M && t < L) {
+                const float* __restrict__ p = gate_grad_partial + ((b * M + m) * G) * L + t;
+                for (int32_t g = 0; g < G; ++g) dg += p[(int64_t)g * L];
+                dr = read_grad[(b * M + m) * L + t];
+            }
+            const float a = ta[lane][i];
+            td[lane][i] = dr * os - dg * us;
+            d_us -= dg * a;
+            d_os += dr * a;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int i = w; i < 64; i += 4)
+            if (t0 + i < L && m0 + lane < M) alpha_grad[(b * L + t0 + i) * M + m0 + lane] = (T)td[i][lane];
+    }
+    red[0][w][lane] = d_us;
+    red[1][w][lane] = d_os;
+    __syncthreads();
+    if (w == 0 && t < L) {
+        update_scale_grad[b * L + t] = (T)(red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane]);
+        output_scale_grad[b * L + t] = (T)(red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane]);
+    }
 }
 
 }  // namespace fmscan

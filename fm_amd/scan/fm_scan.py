@@ -26,7 +26,7 @@ from .. import _lib
 
 __all__ = ["fm_scan_forward", "fm_scan_backward", "fm_scan_backward_reduced", "FM_Scan", "fm_scan",
            "fm_readout_forward", "fm_readout_backward", "FM_Readout", "fm_readout", "FM_Layer", "fm_layer",
-           "fm_memory", "module"]
+           "FM_Memory", "fm_memory", "module"]
 
 _DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16,
            torch.bfloat16: _lib.DTYPE_BF16}
@@ -348,13 +348,14 @@ def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6):
     return output, normed, inv_rms
 
 
-def fm_readout_backward(out_grad, ext_grad, read, states_n, inv_rms):
+def fm_readout_backward(out_grad, ext_grad, read, states_n, inv_rms, *, read_grad_float32=False):
     """Gradients of fm_readout_forward.
 
     out_grad (B, D, L): gradient of the output; ext_grad (B, M, D, L) or None: gradient that
     arrives at the returned (normalised) states; states_n: the normalised states (the scanned
     states themselves without the norm); inv_rms (B, M, L) float32 or None without the norm.
-    Returns (state_grad (B, M, D, L), read_grad (B, M, L)).
+    Returns (state_grad (B, M, D, L), read_grad (B, M, L)); read_grad stays in the float32 it
+    is accumulated in when `read_grad_float32` is set.
     """
     dev = states_n.device
     for name, t in (("out_grad", out_grad), ("ext_grad", ext_grad), ("read", read), ("states_n", states_n),
@@ -380,12 +381,12 @@ def fm_readout_backward(out_grad, ext_grad, read, states_n, inv_rms):
             stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(module.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(),
                                                  None if qe is None else ext_grad.data_ptr(), q.data_ptr(),
-                                                 _ptr(qe), B, M, D, L, code, stream))
+                                                 _ptr(qe), None, None, None, None, B, M, D, L, code, stream))
             _lib.check(module.fmscan_readout_backward(states_n.data_ptr(), _ptr(inv_rms), read.data_ptr(),
                                                       out_grad.data_ptr(), _ptr(ext_grad), q.data_ptr(),
                                                       _ptr(qe), state_grad.data_ptr(), B, M, D, L, code,
                                                       stream))
-    return state_grad, q.to(states_n.dtype)
+    return state_grad, (q if read_grad_float32 else q.to(states_n.dtype))
 
 
 class FM_Readout(torch.autograd.Function):
@@ -424,38 +425,91 @@ def fm_readout(states, read, mem_norm=True, norm_eps=1e-6):
     return output, (normed if mem_norm else states)
 
 
+def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
+    """Scan, RMS norm and read-out (reference fm_scan.py:121-131), time last. Returns what the
+    layer hands back and what its gradient needs."""
+    B_g, M, L_g = gates.shape
+    B, D, L = tokens.shape
+    assert L_g == L
+    assert B_g == B
+    assert gates.is_contiguous()
+    assert tokens.is_contiguous()
+    given_state = initial_state is not None
+    if given_state:
+        assert initial_state.shape == (B, M, D)
+        assert initial_state.is_contiguous()
+    else:
+        initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
+    states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
+    fm_scan_forward(gates, tokens, initial_state, states)
+    output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps)
+    return output, states, normed, inv_rms, (initial_state if given_state else None)
+
+
+def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms, out_grad, ext_grad,
+                     want_initial_state_grad):
+    """Gradients of _layer_forward from those of its two results (either may be None, not both):
+    (gate_grad_partial (B, M, G, L) float32, to be summed over G; d_tokens (B, D, L);
+    d_initial_state or None; read_grad (B, M, L) float32).
+
+    When nothing but the output feeds the loss, no (B, M, D, L) gradient tensor exists between
+    the read-out and the scan: the scan's backward kernel makes it from the output's gradient,
+    the normalised states and two per-slot coefficient vectors.
+    """
+    B, M, D, L = states.shape
+    mem_norm = inv_rms is not None
+    states_n = normed if mem_norm else states
+    dev, dtype = states.device, states.dtype
+    if out_grad is not None:
+        out_grad = out_grad.contiguous()
+
+    if ext_grad is None and _reduced_ok(gates, tokens, states, states_n) and _aligned(read, out_grad):
+        code = _dtype_code(states)
+        q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
+        coef_out, coef_self = torch.empty_like(read), torch.empty_like(read)
+        groups = module.fmscan_reduced_groups(D)
+        d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
+        partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
+        zeros = torch.zeros((B, M, D), dtype=dtype, device=dev)
+        d_h0 = torch.empty_like(zeros) if want_initial_state_grad else None
+        with _on_device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            _lib.check(module.fmscan_readout_dot(
+                states_n.data_ptr(), out_grad.data_ptr(), None, q.data_ptr(), None, _ptr(inv_rms),
+                read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), B, M, D, L, code, stream))
+            _lib.check(module.fmscan_backward_layer(
+                gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
+                out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(), states.data_ptr(),
+                tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0), B, M, D, L, code, 0,
+                stream))
+        return partial, d_tokens, d_h0, q
+
+    if out_grad is None:
+        out_grad = torch.zeros((B, D, L), dtype=dtype, device=dev)
+    # without the norm the states are returned as they are: ext_grad reaches them unchanged
+    state_grad, q = fm_readout_backward(
+        out_grad, ext_grad.contiguous() if (ext_grad is not None and mem_norm) else None, read, states_n,
+        inv_rms, read_grad_float32=True)
+    if ext_grad is not None and not mem_norm:
+        state_grad += ext_grad
+    d_gates, d_tokens, d_h0 = _scan_gradients(gates, tokens, states, initial_state, state_grad,
+                                              want_initial_state_grad)
+    return d_gates.float().unsqueeze(2), d_tokens, d_h0, q
+
+
 class FM_Layer(torch.autograd.Function):
     """output, memory_states = FM_Layer.apply(gates, tokens, initial_state, read, mem_norm, norm_eps)
 
     Scan, RMS norm and read-out of the layer as one node of the autograd graph (reference
-    fm_scan.py:121-131): gates, read (B, M, L), tokens (B, D, L), initial_state (B, M, D) or
-    None -> output (B, D, L), memory states as the layer returns them (B, M, D, L). One node,
-    because backward then needs no (B, M, D, L) gradient tensor between the read-out and
-    the scan: when nothing but `output` feeds the loss, the scan's backward kernel makes that
-    gradient itself from the output's gradient, the normalised states and two per-slot
-    coefficient vectors.
+    fm_scan.py:121-131), time last: gates, read (B, M, L), tokens (B, D, L), initial_state
+    (B, M, D) or None -> output (B, D, L), memory states as the layer returns them (B, M, D, L).
     """
 
     @staticmethod
     def forward(ctx, gates, tokens, initial_state, read, mem_norm=True, norm_eps=1e-6):
-        B_g, M, L_g = gates.shape
-        B, D, L = tokens.shape
-        assert L_g == L
-        assert B_g == B
-        assert gates.is_contiguous()
-        assert tokens.is_contiguous()
-        given_state = initial_state is not None
-        if given_state:
-            assert initial_state.shape == (B, M, D)
-            assert initial_state.is_contiguous()
-        else:
-            initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
-        states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
-        fm_scan_forward(gates, tokens, initial_state, states)
-        output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps)
-        ctx.mem_norm = bool(mem_norm)
-        ctx.save_for_backward(tokens, gates, states, initial_state if given_state else None, read, normed,
-                              inv_rms)
+        output, states, normed, inv_rms, kept_state = _layer_forward(gates, tokens, initial_state, read,
+                                                                     mem_norm, norm_eps)
+        ctx.save_for_backward(tokens, gates, states, kept_state, read, normed, inv_rms)
         ctx.set_materialize_grads(False)
         return output, (normed if mem_norm else states)
 
@@ -464,48 +518,71 @@ class FM_Layer(torch.autograd.Function):
         tokens, gates, states, initial_state, read, normed, inv_rms = ctx.saved_tensors
         if out_grad is None and ext_grad is None:
             return None, None, None, None, None, None
-        B, M, D, L = states.shape
-        want_h0 = ctx.needs_input_grad[2]
-        states_n = normed if ctx.mem_norm else states
-        if out_grad is not None:
-            out_grad = out_grad.contiguous()
+        partial, d_tokens, d_h0, q = _layer_gradients(gates, tokens, states, initial_state, read, normed,
+                                                      inv_rms, out_grad, ext_grad, ctx.needs_input_grad[2])
+        d_gates = partial.sum(dim=2) if partial.shape[2] > 1 else partial.squeeze(2)
+        return d_gates.to(gates.dtype), d_tokens, d_h0, q.to(gates.dtype), None, None
 
-        if ext_grad is None and _reduced_ok(gates, tokens, states, states_n) and _aligned(read, out_grad):
-            # only the output feeds the loss: the states' gradient is made inside the scan's kernel
-            dev, code = states.device, _dtype_code(states)
-            q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
-            groups = module.fmscan_reduced_groups(D)
-            d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
-            partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
-            zeros = torch.zeros((B, M, D), dtype=gates.dtype, device=dev)
-            d_h0 = torch.empty_like(zeros) if want_h0 else None
+
+class FM_Memory(torch.autograd.Function):
+    """output (B, L, D), memory_states (B, M, D, L) = FM_Memory.apply(alpha, update_scale,
+    output_scale, inputs, initial_state, mem_norm, norm_eps): the whole layer (reference
+    fm_scan.py:102-133) as one node, every step of it a kernel of the library."""
+
+    @staticmethod
+    def forward(ctx, alpha, update_scale, output_scale, inputs, initial_state, mem_norm=True, norm_eps=1e-6):
+        dev = alpha.device
+        for name, t in (("alpha", alpha), ("update_scale", update_scale), ("output_scale", output_scale),
+                        ("inputs", inputs)):
+            _on_gpu(name, t, dev)
+            _require(t.dtype == alpha.dtype, f"{name} has dtype {t.dtype}, alpha has {alpha.dtype}")
+        _require(alpha.dim() == 3 and inputs.dim() == 3, "alpha must be (B, L, M) and inputs (B, L, D)")
+        B, L, M = alpha.shape
+        _require(tuple(update_scale.shape) == (B, L, 1) and tuple(output_scale.shape) == (B, L, 1),
+                 f"update_scale and output_scale must be {(B, L, 1)}")
+        _require(inputs.shape[:2] == (B, L), f"inputs must be (B, L, D) with B, L = {(B, L)}")
+        alpha, update_scale, output_scale = alpha.contiguous(), update_scale.contiguous(), output_scale.contiguous()
+        code = _dtype_code(alpha)
+        gates = torch.empty((B, M, L), dtype=alpha.dtype, device=dev)
+        read = torch.empty_like(gates)
+        if gates.numel():
             with _on_device(dev):
-                stream = torch.cuda.current_stream(dev).cuda_stream
-                _lib.check(module.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(), None,
-                                                     q.data_ptr(), None, B, M, D, L, code, stream))
-                if ctx.mem_norm:
-                    coef = inv_rms * read  # float32
-                    coef_out = coef.to(gates.dtype)
-                    coef_self = (coef * q).mul_(1.0 / D).to(gates.dtype)
-                else:
-                    coef_out, coef_self = read, torch.zeros_like(read)
-                _lib.check(module.fmscan_backward_layer(
-                    gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
-                    out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(), states.data_ptr(),
-                    tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0), B, M, D, L, code, 0,
-                    stream))
-            return partial.sum(dim=2).to(gates.dtype), d_tokens, d_h0, q.to(gates.dtype), None, None
+                _lib.check(module.fmscan_layer_prepare(
+                    alpha.data_ptr(), update_scale.data_ptr(), output_scale.data_ptr(), gates.data_ptr(),
+                    read.data_ptr(), B, L, M, code, torch.cuda.current_stream(dev).cuda_stream))
+        tokens = _swap_last_two(inputs)
+        output, states, normed, inv_rms, kept_state = _layer_forward(gates, tokens, initial_state, read,
+                                                                     mem_norm, norm_eps)
+        ctx.save_for_backward(alpha, update_scale, output_scale, tokens, gates, states, kept_state, read, normed,
+                              inv_rms)
+        ctx.set_materialize_grads(False)
+        return _swap_last_two(output), (normed if mem_norm else states)
 
-        if out_grad is None:
-            out_grad = torch.zeros((B, D, L), dtype=states.dtype, device=states.device)
-        # the norm's gradient never sees ext_grad without the norm: the states are returned as they are
-        state_grad, read_grad = fm_readout_backward(
-            out_grad, ext_grad.contiguous() if (ext_grad is not None and ctx.mem_norm) else None, read, states_n,
-            inv_rms)
-        if ext_grad is not None and not ctx.mem_norm:
-            state_grad += ext_grad
-        d_gates, d_tokens, d_h0 = _scan_gradients(gates, tokens, states, initial_state, state_grad, want_h0)
-        return d_gates, d_tokens, d_h0, read_grad, None, None
+    @staticmethod
+    def backward(ctx, out_grad, ext_grad):
+        (alpha, update_scale, output_scale, tokens, gates, states, initial_state, read, normed,
+         inv_rms) = ctx.saved_tensors
+        if out_grad is None and ext_grad is None:
+            return None, None, None, None, None, None, None
+        partial, d_tokens, d_h0, q = _layer_gradients(
+            gates, tokens, states, initial_state, read, normed, inv_rms,
+            None if out_grad is None else _swap_last_two(out_grad), ext_grad, ctx.needs_input_grad[4])
+        B, L, M = alpha.shape
+        dev = alpha.device
+        d_alpha = torch.empty_like(alpha)
+        d_update_scale, d_output_scale = torch.empty_like(update_scale), torch.empty_like(output_scale)
+        if partial.shape[2] > 16:
+            # many groups of d: the finishing kernel walks them one by one, a reduction does better
+            partial = partial.sum(dim=2, keepdim=True)
+        partial = partial.contiguous()
+        if alpha.numel():
+            with _on_device(dev):
+                _lib.check(module.fmscan_layer_finish(
+                    partial.data_ptr(), partial.shape[2], q.data_ptr(), alpha.data_ptr(), update_scale.data_ptr(),
+                    output_scale.data_ptr(), d_alpha.data_ptr(), d_update_scale.data_ptr(),
+                    d_output_scale.data_ptr(), B, L, M, _dtype_code(alpha),
+                    torch.cuda.current_stream(dev).cuda_stream))
+        return d_alpha, d_update_scale, d_output_scale, _swap_last_two(d_tokens), d_h0, None, None
 
 
 def _aligned(*tensors):
@@ -553,13 +630,9 @@ def fm_memory(alpha, update_scale, output_scale, inputs, initial_state=None, mem
         initial_state (B, M, D), optional
     Returns (output (B, L, D), memory_states (B, M, D, L)).
 
-    Only the (B, L, *) tensors pass through PyTorch operations here; everything of size
-    (B, M, D, L) is produced and consumed by the library's kernels.
+    The steps of the reference, each a kernel here: decay gates 1 - alpha * update_scale and read
+    weights alpha * output_scale with time last (:116-119,130), tokens with time last (:117), the
+    scan (:121), the RMS norm over D (:124-127), the read-out over the M slots and its way back to
+    (B, L, D) (:130-131).
     """
-    swap = _SwapLastTwo.apply
-    write = swap(alpha * update_scale)                           # (B, M, L)
-    tokens = swap(inputs)                                        # (B, D, L)
-    read = swap(alpha * output_scale)                            # (B, M, L)
-    # decay gate = 1 - write weight; scan, norm and read-out in one autograd node
-    output, memory_states = fm_layer(1.0 - write, tokens, initial_state, read, mem_norm, norm_eps)
-    return swap(output), memory_states
+    return FM_Memory.apply(alpha, update_scale, output_scale, inputs, initial_state, mem_norm, norm_eps)

@@ -213,6 +213,10 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
  *                           (float32; it is the gradient of `read`) and, when ext_grad
  *                           (a gradient arriving at the returned memory states,
  *                           (B, M, D, L)) is not NULL, qe = sum_d ext_grad * states_n.
+ *                           With coef_out and coef_self ((B, M, L), the call's dtype)
+ *                           not NULL it also writes what fmscan_backward_layer takes:
+ *                           coef_out = inv_rms * read, coef_self = coef_out * q / D
+ *                           (inv_rms NULL: coef_out = read, coef_self = 0).
  * fmscan_readout_backward:  state_grad (B, M, D, L) = gradient of the scanned states:
  *                           dn = read * out_grad (+ ext_grad);
  *                           with the norm  inv_rms * (dn - states_n * (read*q + qe) / D),
@@ -227,11 +231,34 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
                            int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad,
                        float* q, float* qe,
+                       const float* inv_rms, const void* read, void* coef_out, void* coef_self,
                        int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 int fmscan_readout_backward(const void* states_n, const float* inv_rms, const void* read,
                             const void* out_grad, const void* ext_grad,
                             const float* q, const float* qe, void* state_grad,
                             int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
+
+/*
+ * The layer's small tensors (reference fm/scan/fm_scan.py:116,118-119,130 and their
+ * gradients): alpha (B, L, M), update_scale and output_scale (B, L, 1), all of the call's
+ * dtype.
+ * fmscan_layer_prepare:  gates[b,m,t] = 1 - alpha[b,t,m] * update_scale[b,t] and
+ *                        read[b,m,t] = alpha[b,t,m] * output_scale[b,t], both (B, M, L).
+ * fmscan_layer_finish:   from the gradient of gates, given as G float32 partials
+ *                        (B, M, G, L) to be summed (what fmscan_backward_reduced and
+ *                        fmscan_backward_layer write; G = 1 for a plain (B, M, L) gradient),
+ *                        and of read (B, M, L) float32 (q of fmscan_readout_dot):
+ *                        alpha_grad = read_grad * output_scale - gate_grad * update_scale,
+ *                        update_scale_grad = -sum_m gate_grad * alpha,
+ *                        output_scale_grad = sum_m read_grad * alpha.
+ */
+int fmscan_layer_prepare(const void* alpha, const void* update_scale, const void* output_scale,
+                         void* gates, void* read,
+                         int64_t B, int64_t L, int64_t M, int dtype, void* stream);
+int fmscan_layer_finish(const float* gate_grad_partial, int64_t G, const float* read_grad,
+                        const void* alpha, const void* update_scale, const void* output_scale,
+                        void* alpha_grad, void* update_scale_grad, void* output_scale_grad,
+                        int64_t B, int64_t L, int64_t M, int dtype, void* stream);
 
 /*
  * dst[b, c, r] = src[b, r, c] for dense (B, R, C) -> (B, C, R): what fm_memory does to its

@@ -25,7 +25,8 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
                                     "fmscan_backward_reduced",
-                                    "fmscan_forward", "fmscan_last_error", "fmscan_readout_backward",
+                                    "fmscan_forward", "fmscan_last_error", "fmscan_layer_finish",
+                                    "fmscan_layer_prepare", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
                                     "fmscan_reduced_groups", "fmscan_swap_last_two", "fmscan_workspace_bytes"]
 
@@ -133,10 +134,22 @@ def test_rejected_readout_arguments(lib):
     assert fw(o=P) == E_ALIAS
     assert fw(so=3 * P) == E_ALIAS                       # normalised states on top of read
     assert b"overlaps" in lib.fmscan_last_error()
-    dot = lambda sn=P, og=2 * P, e=None, q=3 * P, qe=None: lib.fmscan_readout_dot(sn, og, e, q, qe, *dims, 2, None)
+    dot = lambda sn=P, og=2 * P, e=None, q=3 * P, qe=None, r=None, w=None, co=None, cs=None: \
+        lib.fmscan_readout_dot(sn, og, e, q, qe, r, w, co, cs, *dims, 2, None)
     assert dot(q=None) == E_NULL
     assert dot(e=4 * P) == E_NULL                        # ext_grad without qe
     assert dot(e=4 * P, qe=3 * P) == E_ALIAS
+    assert dot(co=5 * P) == E_NULL                       # coef_out without coef_self and read
+    assert dot(w=6 * P, co=5 * P, cs=5 * P) == E_ALIAS
+    prep = lambda a=P, u=2 * P, o=3 * P, g=4 * P, r=5 * P, M=3: lib.fmscan_layer_prepare(a, u, o, g, r, 2, 64, M, 2, None)
+    assert prep(r=None) == E_NULL
+    assert prep(M=0) == E_SHAPE
+    assert prep(g=P) == E_ALIAS
+    fin = lambda p=P, G=2, q=2 * P, a=3 * P, u=4 * P, o=5 * P, da=6 * P, du=7 * P, do=8 * P: \
+        lib.fmscan_layer_finish(p, G, q, a, u, o, da, du, do, 2, 64, 3, 2, None)
+    assert fin(q=None) == E_NULL
+    assert fin(G=0) == E_SHAPE
+    assert fin(du=6 * P) == E_ALIAS
     bw = lambda sn=P, r=2 * P, w=3 * P, og=4 * P, e=None, q=5 * P, qe=None, sg=6 * P: \
         lib.fmscan_readout_backward(sn, r, w, og, e, q, qe, sg, *dims, 2, None)
     assert bw(sg=None) == E_NULL

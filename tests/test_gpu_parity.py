@@ -565,6 +565,39 @@ def test_layer_backward_kernel_equals_the_two_step_route(scan, dtype, mem_norm):
         check(tag + " d_read", leaves[3].grad, o_dr, tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_layer_prepare_and_finish_kernels(scan, dtype):
+    """The layer's small tensors: gates and read weights with time last, and the gradients of
+    alpha and the two scales from those of gates (as partial sums) and read; against the same
+    formulas in float64."""
+    lib, st = scan.module, torch.cuda.current_stream().cuda_stream
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    for (B, L, M, G) in [(2, 64, 3, 1), (1, 1000, 33, 2), (3, 130, 70, 3), (2, 2048, 32, 16), (1, 5, 1, 1)]:
+        gen = torch.Generator().manual_seed(L + M)
+        alpha = torch.softmax(torch.randn(B, L, M, generator=gen), -1).to(dtype).to(DEV)
+        us = torch.rand(B, L, 1, generator=gen).to(dtype).to(DEV)
+        osc = torch.randn(B, L, 1, generator=gen).to(dtype).to(DEV)
+        gates, read = torch.empty(B, M, L, dtype=dtype, device=DEV), torch.empty(B, M, L, dtype=dtype, device=DEV)
+        assert lib.fmscan_layer_prepare(alpha.data_ptr(), us.data_ptr(), osc.data_ptr(), gates.data_ptr(),
+                                        read.data_ptr(), B, L, M, code, st) == 0
+        a64, u64, o64 = (O.to_f64(t) for t in (alpha, us, osc))
+        tag = f"{(B, L, M, G)} {dtype}"
+        check(tag + " gates", gates, np.transpose(1.0 - a64 * u64, (0, 2, 1)), 1e-6 if dtype == torch.float32 else 4e-3)
+        check(tag + " read", read, np.transpose(a64 * o64, (0, 2, 1)), 1e-6 if dtype == torch.float32 else 4e-3)
+        partial = torch.randn(B, M, G, L, generator=gen).to(DEV)
+        q = torch.randn(B, M, L, generator=gen).to(DEV)
+        d_alpha, d_us, d_os = torch.empty_like(alpha), torch.empty_like(us), torch.empty_like(osc)
+        assert lib.fmscan_layer_finish(partial.data_ptr(), G, q.data_ptr(), alpha.data_ptr(), us.data_ptr(),
+                                       osc.data_ptr(), d_alpha.data_ptr(), d_us.data_ptr(), d_os.data_ptr(),
+                                       B, L, M, code, st) == 0
+        dg = np.transpose(O.to_f64(partial).sum(axis=2), (0, 2, 1))  # (B, L, M)
+        dr = np.transpose(O.to_f64(q), (0, 2, 1))
+        tol = 1e-5 if dtype == torch.float32 else 4e-3
+        check(tag + " d_alpha", d_alpha, dr * o64 - dg * u64, tol)
+        check(tag + " d_update_scale", d_us, -(dg * a64).sum(axis=2, keepdims=True), tol)
+        check(tag + " d_output_scale", d_os, (dr * a64).sum(axis=2, keepdims=True), tol)
+
+
 def test_swap_last_two_is_exact(scan):
     from fm_amd.scan.fm_scan import _swap_last_two
 

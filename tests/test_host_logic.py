@@ -60,39 +60,3 @@ def test_fm_scan_shape_asserts_match_reference_behaviour():
     with pytest.raises(AssertionError):  # initial state of the wrong shape
         fm_scan(torch.rand(2, 3, 32), torch.rand(2, 4, 32), torch.zeros(2, 4, 3))
 
-
-def test_fm_memory_layer_wiring(monkeypatch):
-    """What fm_memory does around the two kernels' worth of work: gates 1 - alpha*update_scale
-    with time last, tokens with time last, read weights alpha*output_scale with time last, and
-    the output back to (B, L, D) (reference fm_scan.py:115-133). The scan is served by the
-    per-timestep PyTorch form, the read-out by the oracle and the axis swaps by PyTorch here
-    (no GPU); the result is
-    compared with a direct numpy statement of the layer."""
-    # (scan + norm + read-out are one call in the product, `fm_layer`: that is what is served here)
-    import fm_amd.scan.fm_scan as impl
-    from fm_amd.scan.fm_pytorch import fm_scan_pytorch
-
-    def layer_on_cpu(gates, tokens, initial_state, read, mem_norm, eps):
-        states = fm_scan_pytorch(gates, tokens, initial_state)
-        out, normed, _ = O.readout_forward(states.numpy(), read.numpy(), mem_norm, eps)
-        return torch.from_numpy(out), torch.from_numpy(normed)
-
-    monkeypatch.setattr(impl, "fm_layer", layer_on_cpu)
-    monkeypatch.setattr(impl, "_swap_last_two", lambda t: t.transpose(1, 2).contiguous())
-    gen = torch.Generator().manual_seed(0)
-    B, L, M, D = 2, 16, 3, 5
-    alpha = torch.softmax(torch.randn(B, L, M, generator=gen, dtype=torch.float64), dim=-1)
-    us = torch.rand(B, L, 1, generator=gen, dtype=torch.float64)
-    os_ = torch.rand(B, L, 1, generator=gen, dtype=torch.float64)
-    inp = torch.randn(B, L, D, generator=gen, dtype=torch.float64)
-    h0 = torch.randn(B, M, D, generator=gen, dtype=torch.float64)
-    for norm in (True, False):
-        out, states = impl.fm_memory(alpha, us, os_, inp, h0, mem_norm=norm, norm_eps=1e-6)
-        assert out.shape == (B, L, D) and states.shape == (B, M, D, L) and out.is_contiguous()
-        g = 1.0 - (alpha * us).numpy().transpose(0, 2, 1)
-        h = O.forward(g, inp.numpy().transpose(0, 2, 1), h0.numpy())
-        if norm:
-            h = h / np.sqrt((h ** 2).mean(axis=2, keepdims=True) + 1e-6)
-        ref = np.einsum("blm,bmdl->bld", (alpha * os_).numpy(), h)
-        np.testing.assert_allclose(states.numpy(), h, rtol=1e-12, atol=1e-12)
-        np.testing.assert_allclose(out.numpy(), ref, rtol=1e-12, atol=1e-12)
