@@ -69,7 +69,7 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
 #pragma unroll 4
     for (int32_t d = w; d < D; d += WV) {
         float h[E];
-        Elem<T>::unpack(load_chunk<T, VEC, MODE == RowDot::kSumSq>(states + (bm * D + d) * L, t0, L, 0u), h);
+        Elem<T>::unpack(load_chunk<T, VEC, true>(states + (bm * D + d) * L, t0, L, 0u), h);
         if constexpr (MODE == RowDot::kSumSq) {
 #pragma unroll
             for (int i = 0; i < E; ++i) acc[i] = __builtin_fmaf(h[i], h[i], acc[i]);
@@ -330,7 +330,16 @@ __global__ __launch_bounds__(256) void layer_finish_kernel(
             float dg = 0.0f, dr = 0.0f;
             if (m < M && t < L) {
                 const float* __restrict__ p = gate_grad_partial + ((b * M + m) * G) * L + t;
-                for (int32_t g = 0; g < G; ++g) dg += p[(int64_t)g * L];
+                float d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;  // four loads in flight per lane
+                int32_t g = 0;
+                for (; g + 4 <= G; g += 4) {
+                    dg += p[(int64_t)g * L];
+                    d1 += p[(int64_t)(g + 1) * L];
+                    d2 += p[(int64_t)(g + 2) * L];
+                    d3 += p[(int64_t)(g + 3) * L];
+                }
+                for (; g < G; ++g) dg += p[(int64_t)g * L];
+                dg = (dg + d1) + (d2 + d3);
                 dr = read_grad[(b * M + m) * L + t];
             }
             const float a = ta[lane][i];
