@@ -49,7 +49,7 @@ def gpu_gen(seed=0):
 
 
 def baseline_inputs(cfg, dtype=None):
-    """(gates, tokens, out_grad) of BASELINE config `cfg` as (rows, 1, L) / (rows, 1, 1, L)
+    """(gates, tokens, out_grad) of benchmark configuration `cfg` (1-5) as (rows, 1, L) / (rows, 1, 1, L)
     tensors: a (B, C, T) problem is the zero-copy fold B' = B*C, M = D = 1."""
     gen = gpu_gen(0)
     rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
@@ -102,7 +102,7 @@ def oracle_rows(g, x, G, out, idx, h0=None, fpg=None, plain=False):
     return h_ref, tg, gg
 
 
-# ----------------------------------------------------------------------------- BASELINE configs
+# ----------------------------------------------------------------------------- the five benchmark configurations
 
 @pytest.mark.parametrize("cfg", [1, 2, 3, 4, 5])
 def test_baseline_config(scan, cfg):
