@@ -199,7 +199,7 @@ def run_layer(torch, args) -> int:
         # what the layer's backward runs when only its output feeds the loss: the kernel above in
         # the form that makes the states' gradient itself (no readout_backward_kernel, no G)
         "scan_backward_reduced_kernel (layer form)": (2 * s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
-            P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), P(states), P(tokens), P(partial),
+            P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), None, P(inv), P(tokens), P(partial),
             None, None, B, M, D, L, code, 0, st)),
     }
     kernels = {}

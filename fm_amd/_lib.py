@@ -51,7 +51,7 @@ def load() -> ctypes.CDLL:
     lib.fmscan_backward_reduced.restype = c_int
     lib.fmscan_backward_reduced.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     lib.fmscan_backward_layer.restype = c_int
-    lib.fmscan_backward_layer.argtypes = [c_void_p] * 12 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
+    lib.fmscan_backward_layer.argtypes = [c_void_p] * 13 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     dims = [c_int64] * 4
     lib.fmscan_readout_inv_rms.restype = c_int
     lib.fmscan_readout_inv_rms.argtypes = [c_void_p] * 2 + dims + [c_int, c_float, c_void_p]

@@ -428,16 +428,21 @@ int64_t fmscan_reduced_groups(int64_t D) { return D < 1 ? 0 : (D + kReducedGroup
 static int backward_reduced(const char* who, const void* gates, const void* out_grad, const void* first_prop_grad,
                             void* token_grad, const void* cached_output, const void* input_tokens,
                             float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
-                            const void* coef_out, const void* coef_self, const void* layer_out_grad, int64_t B,
-                            int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, void* stream) {
+                            const void* coef_out, const void* coef_self, const void* layer_out_grad,
+                            const float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                            unsigned flags, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
     if (flags & ~FMSCAN_FLAG_PLAIN)
         return fail(FMSCAN_E_FLAGS, "%s: only FMSCAN_FLAG_PLAIN is understood here", who);
-    if (!gates || !out_grad || !token_grad || !cached_output || !gate_grad_partial)
+    const bool layer = coef_out != nullptr;
+    const bool recover = layer && !cached_output;  // the states come back from states_n / inv_rms
+    if (!gates || !out_grad || !token_grad || (!cached_output && !recover) || !gate_grad_partial)
         return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
                     "be NULL", who, coef_out ? "states_n" : "out_grad");
-    const bool layer = coef_out != nullptr;
+    if (recover && !inv_rms)
+        return fail(FMSCAN_E_NULL, "%s: without cached_output the states are states_n / inv_rms: inv_rms must "
+                    "not be NULL", who);
     if (layer && (!coef_self || !layer_out_grad))
         return fail(FMSCAN_E_NULL, "%s: coef_self and out_grad must not be NULL", who);
     if (!pb.plain && !input_tokens)
@@ -457,7 +462,8 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                          {"initial_state", initial_state, pb.rows * pb.esize},
                          {"coef_out", coef_out, B * M * L * pb.esize},
                          {"coef_self", layer ? coef_self : nullptr, B * M * L * pb.esize},
-                         {"out_grad", layer ? layer_out_grad : nullptr, B * D * L * pb.esize}};
+                         {"out_grad", layer ? layer_out_grad : nullptr, B * D * L * pb.esize},
+                         {"inv_rms", recover ? inv_rms : nullptr, B * M * L * 4}};
     for (const Range& o : outs)
         for (const Range& in : ins)
             if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
@@ -466,7 +472,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
             if (overlap(outs[i], outs[j]))
                 return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, outs[i].name, outs[j].name);
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
-                     aligned16(token_grad) && aligned16(cached_output) &&
+                     aligned16(token_grad) && aligned16(cached_output) && (!recover || aligned16(inv_rms)) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial) &&
                      (!layer || (aligned16(coef_out) && aligned16(coef_self) && aligned16(layer_out_grad)));
     if (!vec)
@@ -483,22 +489,23 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
         using T = typename decltype(tt)::type;
         auto go = [&](auto pt, auto lt, auto ct) {
             auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, decltype(ct)::value, kReducedDepth,
-                                                             decltype(pt)::value, decltype(lt)::value>;
+                                                             decltype(pt)::value, decltype(lt)::value>;  // lt: 0 plain call, 1 layer, 2 layer + recovered states
             if (lds > 48u * 1024u)
                 (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             kern<<<grid, 64 * kReducedGroup, lds, (hipStream_t)stream>>>(
                 (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
                 (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
                 (T*)initial_state_grad, (const T*)coef_out, (const T*)coef_self, (const T*)layer_out_grad,
-                (int32_t)M, (int32_t)D, L);
+                recover ? inv_rms : nullptr, (int32_t)M, (int32_t)D, L);
         };
         auto with_plain = [&](auto lt, auto ct) {
             if (pb.plain) go(BoolTag<true>{}, lt, ct);
             else go(BoolTag<false>{}, lt, ct);
         };
-        // the layer form holds three more loads per ring entry: two tiles per visit instead of four
-        if (layer) with_plain(BoolTag<true>{}, IntTag<kLayerChunk>{});
-        else with_plain(BoolTag<false>{}, IntTag<kReducedChunk>{});
+        // the layer forms hold three more loads per ring entry: two tiles per visit instead of four
+        if (recover) with_plain(IntTag<2>{}, IntTag<kLayerChunk>{});
+        else if (layer) with_plain(IntTag<1>{}, IntTag<kLayerChunk>{});
+        else with_plain(IntTag<0>{}, IntTag<kReducedChunk>{});
     });
     return launched(who);
 }
@@ -510,18 +517,18 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
                             void* stream) {
     return backward_reduced("fmscan_backward_reduced", gates, out_grad, first_prop_grad, token_grad, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, nullptr, nullptr,
-                            nullptr, B, M, D, L, dtype, flags, stream);
+                            nullptr, nullptr, B, M, D, L, dtype, flags, stream);
 }
 
 int fmscan_backward_layer(const void* gates, const void* states_n, const void* coef_out, const void* coef_self,
                           const void* out_grad, const void* first_prop_grad, void* token_grad,
-                          const void* cached_output, const void* input_tokens, float* gate_grad_partial,
-                          const void* initial_state, void* initial_state_grad, int64_t B, int64_t M, int64_t D,
-                          int64_t L, int dtype, unsigned flags, void* stream) {
+                          const void* cached_output, const float* inv_rms, const void* input_tokens,
+                          float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                          int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, void* stream) {
     if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer: coef_out must not be NULL");
     return backward_reduced("fmscan_backward_layer", gates, states_n, first_prop_grad, token_grad, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
-                            out_grad, B, M, D, L, dtype, flags, stream);
+                            out_grad, inv_rms, B, M, D, L, dtype, flags, stream);
 }
 
 }  // extern "C"

@@ -456,15 +456,15 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
     the read-out and the scan: the scan's backward kernel makes it from the output's gradient,
     the normalised states and two per-slot coefficient vectors.
     """
-    B, M, D, L = states.shape
     mem_norm = inv_rms is not None
-    states_n = normed if mem_norm else states
-    dev, dtype = states.device, states.dtype
+    states_n = normed if mem_norm else states  # with the norm, `states` is None: not kept
+    B, M, D, L = states_n.shape
+    dev, dtype = states_n.device, states_n.dtype
     if out_grad is not None:
         out_grad = out_grad.contiguous()
 
-    if ext_grad is None and _reduced_ok(gates, tokens, states, states_n) and _aligned(read, out_grad):
-        code = _dtype_code(states)
+    if ext_grad is None and _reduced_ok(gates, tokens, states_n, states_n) and _aligned(read, out_grad):
+        code = _dtype_code(states_n)
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         coef_out, coef_self = torch.empty_like(read), torch.empty_like(read)
         groups = module.fmscan_reduced_groups(D)
@@ -479,9 +479,10 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
                 read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), B, M, D, L, code, stream))
             _lib.check(module.fmscan_backward_layer(
                 gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
-                out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(), states.data_ptr(),
-                tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0), B, M, D, L, code, 0,
-                stream))
+                out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(),
+                None if mem_norm else states.data_ptr(),  # with the norm: states = states_n / inv_rms
+                _ptr(inv_rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0),
+                B, M, D, L, code, 0, stream))
         return partial, d_tokens, d_h0, q
 
     if out_grad is None:
@@ -492,6 +493,8 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         inv_rms, read_grad_float32=True)
     if ext_grad is not None and not mem_norm:
         state_grad += ext_grad
+    if mem_norm:  # the scanned states were not kept: take them back from the normalised ones
+        states = normed * (1.0 / inv_rms).to(dtype).unsqueeze(2)
     d_gates, d_tokens, d_h0 = _scan_gradients(gates, tokens, states, initial_state, state_grad,
                                               want_initial_state_grad)
     return d_gates.float().unsqueeze(2), d_tokens, d_h0, q
@@ -509,7 +512,9 @@ class FM_Layer(torch.autograd.Function):
     def forward(ctx, gates, tokens, initial_state, read, mem_norm=True, norm_eps=1e-6):
         output, states, normed, inv_rms, kept_state = _layer_forward(gates, tokens, initial_state, read,
                                                                      mem_norm, norm_eps)
-        ctx.save_for_backward(tokens, gates, states, kept_state, read, normed, inv_rms)
+        # with the norm, the normalised states (returned anyway) and inv_rms stand in for the
+        # scanned states: nothing else of size (B, M, D, L) is kept for backward
+        ctx.save_for_backward(tokens, gates, None if mem_norm else states, kept_state, read, normed, inv_rms)
         ctx.set_materialize_grads(False)
         return output, (normed if mem_norm else states)
 
@@ -553,8 +558,8 @@ class FM_Memory(torch.autograd.Function):
         tokens = _swap_last_two(inputs)
         output, states, normed, inv_rms, kept_state = _layer_forward(gates, tokens, initial_state, read,
                                                                      mem_norm, norm_eps)
-        ctx.save_for_backward(alpha, update_scale, output_scale, tokens, gates, states, kept_state, read, normed,
-                              inv_rms)
+        ctx.save_for_backward(alpha, update_scale, output_scale, tokens, gates, None if mem_norm else states,
+                              kept_state, read, normed, inv_rms)
         ctx.set_materialize_grads(False)
         return _swap_last_two(output), (normed if mem_norm else states)
 

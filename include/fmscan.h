@@ -176,13 +176,17 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
  * the read-out alone when coef_out = read, coef_self = 0 and states_n = cached_output.
  *   states_n   (B, M, D, L)  the normalised states      coef_out, coef_self  (B, M, L)
  *   out_grad   (B, D, L)     gradient of the layer's output, time last
- * all of the call's dtype. Everything else, and the limits, as fmscan_backward_reduced.
+ * all of the call's dtype. cached_output may be NULL when inv_rms ((B, M, L) float32, as
+ * fmscan_readout_inv_rms wrote it) is given: the scanned states are then taken back from
+ * the normalised ones, states_n / inv_rms, and the layer need not keep them (the reference
+ * keeps them for autograd, fm/scan/fm_scan.py:53-55). Everything else, and the limits, as
+ * fmscan_backward_reduced.
  */
 int fmscan_backward_layer(const void* gates, const void* states_n,
                           const void* coef_out, const void* coef_self, const void* out_grad,
                           const void* first_prop_grad, void* token_grad,
-                          const void* cached_output, const void* input_tokens,
-                          float* gate_grad_partial,
+                          const void* cached_output, const float* inv_rms,
+                          const void* input_tokens, float* gate_grad_partial,
                           const void* initial_state, void* initial_state_grad,
                           int64_t B, int64_t M, int64_t D, int64_t L,
                           int dtype, unsigned flags, void* stream);

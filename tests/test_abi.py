@@ -100,11 +100,13 @@ def test_rejected_arguments(lib):
     assert red(L=7) == _const("FMSCAN_E_UNALIGNED")
     assert red(g=P + 4) == _const("FMSCAN_E_UNALIGNED")
     lay = lambda **k: lib.fmscan_backward_layer(
-        P, 2 * P, k.get("co", 7 * P), k.get("cs", 8 * P), k.get("og", 9 * P), None, k.get("dx", 3 * P), 4 * P, 5 * P,
-        6 * P, None, None, 2, 2, 2, 8, 0, 0, None)
+        P, 2 * P, k.get("co", 7 * P), k.get("cs", 8 * P), k.get("og", 9 * P), None, k.get("dx", 3 * P),
+        k.get("h", 4 * P), k.get("r", None), 5 * P, 6 * P, None, None, 2, 2, 2, 8, 0, 0, None)
     assert lay(co=None) == E_NULL
     assert lay(cs=None) == E_NULL
     assert lay(og=None) == E_NULL
+    assert lay(h=None) == E_NULL                      # no saved states and no inv_rms to take them back with
+    assert lay(h=None, r=3 * P) == E_ALIAS            # inv_rms under token_grad
     assert lay(dx=9 * P) == E_ALIAS                   # token_grad on top of the layer's out_grad
     assert lib.fmscan_reduced_groups(128) == 16 and lib.fmscan_reduced_groups(9) == 2
     assert fwd(lib, out=P) == E_ALIAS                 # out on top of gates

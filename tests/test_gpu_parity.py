@@ -598,6 +598,26 @@ def test_layer_prepare_and_finish_kernels(scan, dtype):
         check(tag + " d_output_scale", d_os, (dr * a64).sum(axis=2, keepdims=True), tol)
 
 
+def test_layer_keeps_no_second_copy_of_the_states(scan):
+    """With the norm, backward works from the normalised states the layer returns (and inv_rms):
+    the scanned states are not kept. Measured as allocated memory across the forward pass."""
+    B, L, M, D, dt = 2, 4096, 8, 64, torch.bfloat16
+    gen = gpu_gen(11)
+    alpha = torch.softmax(torch.randn(B, L, M, device=DEV, generator=gen), -1).to(dt).requires_grad_()
+    us = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt).requires_grad_()
+    osc = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt).requires_grad_()
+    inp = torch.randn(B, L, D, device=DEV, generator=gen).to(dt).requires_grad_()
+    states_bytes = B * M * D * L * 2
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    out, mem = scan.fm_memory(alpha, us, osc, inp)
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated() - before
+    assert states_bytes <= held < 1.5 * states_bytes, (held, states_bytes)
+    out.sum().backward()  # and the gradients still come out
+    assert all(t.grad is not None and torch.isfinite(t.grad.float()).all() for t in (alpha, us, osc, inp))
+
+
 def test_swap_last_two_is_exact(scan):
     from fm_amd.scan.fm_scan import _swap_last_two
 
