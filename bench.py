@@ -180,6 +180,7 @@ def run_layer(torch, args) -> int:
     lib, st = S.module, torch.cuda.current_stream().cuda_stream
     inv = torch.empty(B, M, L, device=dev)
     q = torch.empty_like(inv)
+    rms = torch.full_like(read, 1.5)  # 1 / inv_rms: takes the scanned states back from the normalised ones
     normed, sg = torch.empty_like(states), torch.empty_like(states)
     out = torch.empty(B, D, L, dtype=dt, device=dev)
     coef, dtok = rn(B, M, L).to(dt), torch.empty(B, D, L, dtype=dt, device=dev)
@@ -191,7 +192,7 @@ def run_layer(torch, args) -> int:
         "rowdot_kernel (inv_rms)": (s * N, lambda: lib.fmscan_readout_inv_rms(P(states), P(inv), B, M, D, L, code, 1e-6, st)),
         "readout_forward_kernel": (2 * s * N, lambda: lib.fmscan_readout_forward(
             P(states), P(inv), P(read), P(normed), P(out), B, M, D, L, code, st)),
-        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, None, None, None, None, B, M, D, L, code, st)),
+        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, None, None, None, None, None, B, M, D, L, code, st)),
         "readout_backward_kernel": (2 * s * N, lambda: lib.fmscan_readout_backward(
             P(normed), P(inv), P(read), P(og), None, P(q), None, P(sg), B, M, D, L, code, st)),
         "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 8, lambda: S.fm_scan_backward_reduced(
@@ -199,7 +200,7 @@ def run_layer(torch, args) -> int:
         # what the layer's backward runs when only its output feeds the loss: the kernel above in
         # the form that makes the states' gradient itself (no readout_backward_kernel, no G)
         "scan_backward_reduced_kernel (layer form)": (2 * s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
-            P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), None, P(inv), P(tokens), P(partial),
+            P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
             None, None, B, M, D, L, code, 0, st)),
     }
     kernels = {}

@@ -58,7 +58,7 @@ def load() -> ctypes.CDLL:
     lib.fmscan_readout_forward.restype = c_int
     lib.fmscan_readout_forward.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
     lib.fmscan_readout_dot.restype = c_int
-    lib.fmscan_readout_dot.argtypes = [c_void_p] * 9 + dims + [c_int, c_void_p]
+    lib.fmscan_readout_dot.argtypes = [c_void_p] * 10 + dims + [c_int, c_void_p]
     lib.fmscan_layer_prepare.restype = c_int
     lib.fmscan_layer_prepare.argtypes = [c_void_p] * 5 + [c_int64] * 3 + [c_int, c_void_p]
     lib.fmscan_layer_finish.restype = c_int

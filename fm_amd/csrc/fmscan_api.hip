@@ -429,19 +429,19 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                             void* token_grad, const void* cached_output, const void* input_tokens,
                             float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
                             const void* coef_out, const void* coef_self, const void* layer_out_grad,
-                            const float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                            const void* rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
                             unsigned flags, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
     if (flags & ~FMSCAN_FLAG_PLAIN)
         return fail(FMSCAN_E_FLAGS, "%s: only FMSCAN_FLAG_PLAIN is understood here", who);
     const bool layer = coef_out != nullptr;
-    const bool recover = layer && !cached_output;  // the states come back from states_n / inv_rms
+    const bool recover = layer && !cached_output;  // the states come back from states_n * rms
     if (!gates || !out_grad || !token_grad || (!cached_output && !recover) || !gate_grad_partial)
         return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
                     "be NULL", who, coef_out ? "states_n" : "out_grad");
-    if (recover && !inv_rms)
-        return fail(FMSCAN_E_NULL, "%s: without cached_output the states are states_n / inv_rms: inv_rms must "
+    if (recover && !rms)
+        return fail(FMSCAN_E_NULL, "%s: without cached_output the states are states_n * rms: rms must "
                     "not be NULL", who);
     if (layer && (!coef_self || !layer_out_grad))
         return fail(FMSCAN_E_NULL, "%s: coef_self and out_grad must not be NULL", who);
@@ -463,7 +463,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                          {"coef_out", coef_out, B * M * L * pb.esize},
                          {"coef_self", layer ? coef_self : nullptr, B * M * L * pb.esize},
                          {"out_grad", layer ? layer_out_grad : nullptr, B * D * L * pb.esize},
-                         {"inv_rms", recover ? inv_rms : nullptr, B * M * L * 4}};
+                         {"rms", recover ? rms : nullptr, B * M * L * pb.esize}};
     for (const Range& o : outs)
         for (const Range& in : ins)
             if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
@@ -472,7 +472,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
             if (overlap(outs[i], outs[j]))
                 return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, outs[i].name, outs[j].name);
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
-                     aligned16(token_grad) && aligned16(cached_output) && (!recover || aligned16(inv_rms)) &&
+                     aligned16(token_grad) && aligned16(cached_output) && (!recover || aligned16(rms)) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial) &&
                      (!layer || (aligned16(coef_out) && aligned16(coef_self) && aligned16(layer_out_grad)));
     if (!vec)
@@ -496,7 +496,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                 (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
                 (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
                 (T*)initial_state_grad, (const T*)coef_out, (const T*)coef_self, (const T*)layer_out_grad,
-                recover ? inv_rms : nullptr, (int32_t)M, (int32_t)D, L);
+                (const T*)(recover ? rms : nullptr), (int32_t)M, (int32_t)D, L);
         };
         auto with_plain = [&](auto lt, auto ct) {
             if (pb.plain) go(BoolTag<true>{}, lt, ct);
@@ -522,13 +522,13 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
 
 int fmscan_backward_layer(const void* gates, const void* states_n, const void* coef_out, const void* coef_self,
                           const void* out_grad, const void* first_prop_grad, void* token_grad,
-                          const void* cached_output, const float* inv_rms, const void* input_tokens,
+                          const void* cached_output, const void* rms, const void* input_tokens,
                           float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
                           int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, void* stream) {
     if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer: coef_out must not be NULL");
     return backward_reduced("fmscan_backward_layer", gates, states_n, first_prop_grad, token_grad, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
-                            out_grad, inv_rms, B, M, D, L, dtype, flags, stream);
+                            out_grad, rms, B, M, D, L, dtype, flags, stream);
 }
 
 }  // extern "C"
@@ -592,7 +592,7 @@ int fmscan_readout_inv_rms(const void* states, float* inv_rms, int64_t B, int64_
             fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kSumSq, false, decltype(vt)::value>
                 <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>((const T*)states, nullptr, nullptr, inv_rms,
                                                                       nullptr, nullptr, nullptr, nullptr, nullptr,
-                                                                      (int32_t)M, (int32_t)D, L, rs.tiles, eps);
+                                                                      nullptr, (int32_t)M, (int32_t)D, L, rs.tiles, eps);
         });
     });
     return launched("read-out (inverse rms)");
@@ -635,8 +635,8 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
 }
 
 int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad, float* q, float* qe,
-                       const float* inv_rms, const void* read, void* coef_out, void* coef_self, int64_t B,
-                       int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
+                       const float* inv_rms, const void* read, void* coef_out, void* coef_self, void* rms_out,
+                       int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
     ReadoutShape rs;
     if (int rc = parse_readout("fmscan_readout_dot", B, M, D, L, dtype, &rs)) return rc;
     if (!states_n || !out_grad || !q)
@@ -644,17 +644,19 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
     if (ext_grad && !qe) return fail(FMSCAN_E_NULL, "fmscan_readout_dot: qe must not be NULL with ext_grad");
     if ((coef_out || coef_self) && (!coef_out || !coef_self || !read))
         return fail(FMSCAN_E_NULL, "fmscan_readout_dot: coef_out, coef_self and read go together");
+    if (rms_out && !inv_rms) return fail(FMSCAN_E_NULL, "fmscan_readout_dot: rms_out needs inv_rms");
     const int64_t full = B * M * D * L * rs.esize, slot = B * M * L;
     const Range outs[] = {{"q", q, slot * 4}, {"qe", ext_grad ? qe : nullptr, slot * 4},
-                          {"coef_out", coef_out, slot * rs.esize}, {"coef_self", coef_self, slot * rs.esize}};
+                          {"coef_out", coef_out, slot * rs.esize}, {"coef_self", coef_self, slot * rs.esize},
+                          {"rms_out", rms_out, slot * rs.esize}};
     const Range ins[] = {{"states_n", states_n, full}, {"out_grad", out_grad, B * D * L * rs.esize},
-                         {"ext_grad", ext_grad, full}, {"inv_rms", coef_out ? inv_rms : nullptr, slot * 4},
+                         {"ext_grad", ext_grad, full}, {"inv_rms", (coef_out || rms_out) ? inv_rms : nullptr, slot * 4},
                          {"read", coef_out ? read : nullptr, slot * rs.esize}};
     for (const Range& o : outs)
         for (const Range& in : ins)
             if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", o.name, in.name);
-    for (int i = 0; i < 4; ++i)
-        for (int j = i + 1; j < 4; ++j)
+    for (int i = 0; i < 5; ++i)
+        for (int j = i + 1; j < 5; ++j)
             if (overlap(outs[i], outs[j]))
                 return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", outs[i].name, outs[j].name);
     const bool vec = vector_path(rs, {states_n, out_grad, ext_grad});
@@ -666,7 +668,7 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
                 fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kDot, decltype(et)::value, decltype(vt)::value>
                     <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>(
                         (const T*)states_n, (const T*)out_grad, (const T*)ext_grad, q, qe, inv_rms, (const T*)read,
-                        (T*)coef_out, (T*)coef_self, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
+                        (T*)coef_out, (T*)coef_self, (T*)rms_out, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
             });
         });
     });

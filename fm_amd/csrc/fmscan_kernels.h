@@ -533,7 +533,7 @@ __global__ __launch_bounds__(64 * R) void scan_aggregate_kernel(
 //   G[b,m,d,t] = coef_out[b,m,t] * layer_out_grad[b,d,t] - coef_self[b,m,t] * out_grad[b,m,d,t]
 // where `out_grad` then carries the normalised states; the (B, M, D, L) gradient tensor is
 // never written or read. LAYER == 2: the scanned states themselves are not read either
-// (h_saved is NULL) but taken back from the normalised ones, h = out_grad / inv_rms, so that
+// (h_saved is NULL) but taken back from the normalised ones, h = out_grad * rms, so that
 // the layer has to keep nothing of size (B, M, D, L) besides the states it returns.
 template <typename T, int DG, int C, int R, bool PLAIN, int LAYER>
 __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
@@ -542,7 +542,7 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const T* __restrict__ tokens, float* __restrict__ gate_partial /* (B, M, NG, L) */,
     const T* __restrict__ h0, T* __restrict__ h0_grad, const T* __restrict__ coef_out /* (B, M, L) */,
     const T* __restrict__ coef_self /* (B, M, L) */, const T* __restrict__ layer_out_grad /* (B, D, L) */,
-    const float* __restrict__ inv_rms /* (B, M, L) */, int32_t M, int32_t D, int64_t L) {
+    const T* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     constexpr int SLICE = TILE / DG;  // elements of a summed tile each wave adds up and stores
@@ -581,9 +581,9 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     struct Entry {
         u32x4 g, G, h, x;
         u32x4 co, cs, y;  // LAYER only
-        u32x4 ra, rb;     // LAYER == 2: inv_rms of the chunk's steps (float32: two loads for 8 steps)
+        u32x4 rr;         // LAYER == 2: rms of the chunk's steps
         T hb;
-        float hbr;        // LAYER == 2: inv_rms at the step hb belongs to
+        T hbr;            // LAYER == 2: rms at the step hb belongs to
     };
     // Where a visit is: chunk `chunk` of row (b, m, d), with the offsets that go with it
     // kept as running sums in scalar registers (a 64-bit product per step would run on the
@@ -633,13 +633,11 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
             e.cs = load16<T, false>(at(coef_self + c.goff + tw));
             e.y = load16<T, false>(at(yrow + tw));
         }
-        e.ra = e.rb = u32x4{0u, 0u, 0u, 0u};
-        e.hbr = 1.0f;
+        e.rr = u32x4{0u, 0u, 0u, 0u};
+        e.hbr = e.hb;
         if constexpr (LAYER == 2) {
-            const char* rrow = reinterpret_cast<const char*>(inv_rms + c.goff + tw) + loff * (4u / (uint32_t)sizeof(T));
-            e.ra = *reinterpret_cast<const u32x4*>(rrow);
-            if constexpr (E == 8) e.rb = *reinterpret_cast<const u32x4*>(rrow + 16);
-            e.hbr = inv_rms[c.goff + (tw > 0 ? tw - 1 : 0)];
+            e.rr = load16<T, false>(at(rms + c.goff + tw));
+            e.hbr = rms[c.goff + (tw > 0 ? tw - 1 : 0)];
         }
         // h just before the tile (h[-1] at the start of the row): one address for the whole wave
         const T* src = tw > 0 ? hrow + (tw - 1) : (h0 != nullptr ? h0 + c.row : hrow);
@@ -688,11 +686,11 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                 if (tw + TILE > L && tw + lane_off >= L) {  // short or absent tile: nothing there
                     cur.g = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
                     cur.G = cur.h = cur.x = cur.co = cur.cs = cur.y = u32x4{0u, 0u, 0u, 0u};
-                    cur.ra = cur.rb = u32x4{0x3f800000u, 0x3f800000u, 0x3f800000u, 0x3f800000u};
+                    cur.rr = u32x4{0u, 0u, 0u, 0u};
                 }
                 float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(cur.hb) : 0.0f;
                 if constexpr (LAYER == 2) {
-                    if (k > 0) hb *= __builtin_amdgcn_rcpf(cur.hbr);  // at k == 0 it is the initial state itself
+                    if (k > 0) hb *= Elem<T>::widen(cur.hbr);  // at k == 0 it is the initial state itself
                 }
                 float g[E], G[E], h[E], p[E], xs[E];
                 Elem<T>::unpack(cur.g, g);
@@ -705,14 +703,11 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
                         Elem<T>::unpack(cur.x, xs);
                     }
                 }
-                if constexpr (LAYER == 2) {  // h = normalised state / inv_rms (G[] holds the normalised state)
-                    float inv[E];
-                    inv[0] = u2f(cur.ra.x); inv[1] = u2f(cur.ra.y); inv[2] = u2f(cur.ra.z); inv[3] = u2f(cur.ra.w);
-                    if constexpr (E == 8) {
-                        inv[4] = u2f(cur.rb.x); inv[5] = u2f(cur.rb.y); inv[6] = u2f(cur.rb.z); inv[7] = u2f(cur.rb.w);
-                    }
+                if constexpr (LAYER == 2) {  // h = normalised state * rms (G[] holds the normalised state)
+                    float r[E];
+                    Elem<T>::unpack(cur.rr, r);
 #pragma unroll
-                    for (int j = 0; j < E; ++j) h[j] = G[j] * __builtin_amdgcn_rcpf(inv[j]);
+                    for (int j = 0; j < E; ++j) h[j] = G[j] * r[j];
                 }
                 if constexpr (LAYER != 0) {
                     float co[E], cs[E], ys[E];

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
     const T* __restrict__ ext_grad /* (B, M, D, L) */, float* __restrict__ result /* (B, M, L) */,
     float* __restrict__ result_ext /* (B, M, L) */, const float* __restrict__ inv_rms /* (B, M, L) */,
     const T* __restrict__ read /* (B, M, L) */, T* __restrict__ coef_out, T* __restrict__ coef_self,
-    int32_t M, int32_t D, int64_t L, int32_t tiles, float eps) {
+    T* __restrict__ rms_out /* (B, M, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles, float eps) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     __shared__ float part[EXT ? 2 : 1][WV][TILE];
@@ -111,6 +111,8 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
                 coef_out[bm * L + t] = (T)c;
                 coef_self[bm * L + t] = (T)(inv_rms ? c * s / (float)D : 0.0f);
             }
+            // ... and what takes the scanned states back from the normalised ones
+            if (rms_out != nullptr) rms_out[bm * L + t] = (T)(1.0f / inv_rms[bm * L + t]);
         }
     }
 }

@@ -317,12 +317,13 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6):
+def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6, *, in_place=False):
     """RMS norm over D and read-out over M of scanned states (reference fm_scan.py:124-131).
 
     states (B, M, D, L), read (B, M, L) = (alpha * output_scale) with time last; same dtype,
     contiguous, on one GPU. Returns (output (B, D, L), normalised states (B, M, D, L) or None
-    without the norm, inv_rms (B, M, L) float32 or None).
+    without the norm, inv_rms (B, M, L) float32 or None). `in_place` writes the normalised states
+    over `states` (for callers that need the scanned states no longer).
     """
     dev = states.device
     for name, t in (("states", states), ("read", read)):
@@ -334,7 +335,7 @@ def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6):
     _require(tuple(read.shape) == (B, M, L), f"read must be {(B, M, L)}, got {tuple(read.shape)}")
     code = _dtype_code(states)
     output = torch.empty((B, D, L), dtype=states.dtype, device=dev)
-    normed = torch.empty_like(states) if mem_norm else None
+    normed = (states if in_place else torch.empty_like(states)) if mem_norm else None
     inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev) if mem_norm else None
     if states.numel():
         with _on_device(dev):
@@ -381,7 +382,7 @@ def fm_readout_backward(out_grad, ext_grad, read, states_n, inv_rms, *, read_gra
             stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(module.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(),
                                                  None if qe is None else ext_grad.data_ptr(), q.data_ptr(),
-                                                 _ptr(qe), None, None, None, None, B, M, D, L, code, stream))
+                                                 _ptr(qe), None, None, None, None, None, B, M, D, L, code, stream))
             _lib.check(module.fmscan_readout_backward(states_n.data_ptr(), _ptr(inv_rms), read.data_ptr(),
                                                       out_grad.data_ptr(), _ptr(ext_grad), q.data_ptr(),
                                                       _ptr(qe), state_grad.data_ptr(), B, M, D, L, code,
@@ -442,8 +443,10 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
         initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
     states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
     fm_scan_forward(gates, tokens, initial_state, states)
-    output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps)
-    return output, states, normed, inv_rms, (initial_state if given_state else None)
+    # with the norm the scanned states are needed no longer (backward takes them back from the
+    # normalised ones): normalise in place, one (B, M, D, L) tensor at any time
+    output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps, in_place=bool(mem_norm))
+    return output, (None if mem_norm else states), normed, inv_rms, (initial_state if given_state else None)
 
 
 def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms, out_grad, ext_grad,
@@ -467,6 +470,7 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         code = _dtype_code(states_n)
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         coef_out, coef_self = torch.empty_like(read), torch.empty_like(read)
+        rms = torch.empty_like(read) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
         groups = module.fmscan_reduced_groups(D)
         d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
@@ -476,12 +480,12 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
             stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(module.fmscan_readout_dot(
                 states_n.data_ptr(), out_grad.data_ptr(), None, q.data_ptr(), None, _ptr(inv_rms),
-                read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), B, M, D, L, code, stream))
+                read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), _ptr(rms), B, M, D, L, code, stream))
             _lib.check(module.fmscan_backward_layer(
                 gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
                 out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(),
-                None if mem_norm else states.data_ptr(),  # with the norm: states = states_n / inv_rms
-                _ptr(inv_rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0),
+                None if mem_norm else states.data_ptr(),  # with the norm: states = states_n * rms
+                _ptr(rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0),
                 B, M, D, L, code, 0, stream))
         return partial, d_tokens, d_h0, q
 

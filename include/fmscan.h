@@ -176,16 +176,16 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
  * the read-out alone when coef_out = read, coef_self = 0 and states_n = cached_output.
  *   states_n   (B, M, D, L)  the normalised states      coef_out, coef_self  (B, M, L)
  *   out_grad   (B, D, L)     gradient of the layer's output, time last
- * all of the call's dtype. cached_output may be NULL when inv_rms ((B, M, L) float32, as
- * fmscan_readout_inv_rms wrote it) is given: the scanned states are then taken back from
- * the normalised ones, states_n / inv_rms, and the layer need not keep them (the reference
- * keeps them for autograd, fm/scan/fm_scan.py:53-55). Everything else, and the limits, as
+ * all of the call's dtype. cached_output may be NULL when rms ((B, M, L), 1 / inv_rms:
+ * fmscan_readout_dot writes it) is given: the scanned states are then taken back from the
+ * normalised ones, states_n * rms, and the layer need not keep them (the reference keeps
+ * them for autograd, fm/scan/fm_scan.py:53-55). Everything else, and the limits, as
  * fmscan_backward_reduced.
  */
 int fmscan_backward_layer(const void* gates, const void* states_n,
                           const void* coef_out, const void* coef_self, const void* out_grad,
                           const void* first_prop_grad, void* token_grad,
-                          const void* cached_output, const float* inv_rms,
+                          const void* cached_output, const void* rms,
                           const void* input_tokens, float* gate_grad_partial,
                           const void* initial_state, void* initial_state_grad,
                           int64_t B, int64_t M, int64_t D, int64_t L,
@@ -220,7 +220,8 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
  *                           With coef_out and coef_self ((B, M, L), the call's dtype)
  *                           not NULL it also writes what fmscan_backward_layer takes:
  *                           coef_out = inv_rms * read, coef_self = coef_out * q / D
- *                           (inv_rms NULL: coef_out = read, coef_self = 0).
+ *                           (inv_rms NULL: coef_out = read, coef_self = 0), and with rms_out
+ *                           ((B, M, L), the call's dtype) not NULL, rms_out = 1 / inv_rms.
  * fmscan_readout_backward:  state_grad (B, M, D, L) = gradient of the scanned states:
  *                           dn = read * out_grad (+ ext_grad);
  *                           with the norm  inv_rms * (dn - states_n * (read*q + qe) / D),
@@ -236,6 +237,7 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
 int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad,
                        float* q, float* qe,
                        const float* inv_rms, const void* read, void* coef_out, void* coef_self,
+                       void* rms_out,
                        int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 int fmscan_readout_backward(const void* states_n, const float* inv_rms, const void* read,
                             const void* out_grad, const void* ext_grad,

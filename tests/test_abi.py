@@ -136,13 +136,14 @@ def test_rejected_readout_arguments(lib):
     assert fw(o=P) == E_ALIAS
     assert fw(so=3 * P) == E_ALIAS                       # normalised states on top of read
     assert b"overlaps" in lib.fmscan_last_error()
-    dot = lambda sn=P, og=2 * P, e=None, q=3 * P, qe=None, r=None, w=None, co=None, cs=None: \
-        lib.fmscan_readout_dot(sn, og, e, q, qe, r, w, co, cs, *dims, 2, None)
+    dot = lambda sn=P, og=2 * P, e=None, q=3 * P, qe=None, r=None, w=None, co=None, cs=None, rms=None: \
+        lib.fmscan_readout_dot(sn, og, e, q, qe, r, w, co, cs, rms, *dims, 2, None)
     assert dot(q=None) == E_NULL
     assert dot(e=4 * P) == E_NULL                        # ext_grad without qe
     assert dot(e=4 * P, qe=3 * P) == E_ALIAS
     assert dot(co=5 * P) == E_NULL                       # coef_out without coef_self and read
     assert dot(w=6 * P, co=5 * P, cs=5 * P) == E_ALIAS
+    assert dot(rms=7 * P) == E_NULL                      # rms_out without inv_rms
     prep = lambda a=P, u=2 * P, o=3 * P, g=4 * P, r=5 * P, M=3: lib.fmscan_layer_prepare(a, u, o, g, r, 2, 64, M, 2, None)
     assert prep(r=None) == E_NULL
     assert prep(M=0) == E_SHAPE
