@@ -240,6 +240,9 @@ def main() -> int:
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["layer"])
     ap.add_argument("--waves-per-row", type=int, default=0, help="0 = library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture one step in a HIP graph and time its replays (what a launch-bound "
+                         "caller, e.g. the small configuration 1, gets without the per-call Python cost)")
     ap.add_argument("--probe", action="store_true",
                     help="for rocprofv3 --pmc runs: a few launches of an elementwise copy of known "
                          "size (torch.neg, reads and writes one tensor), then of the two scan "
@@ -335,6 +338,25 @@ def main() -> int:
                      "algorithmic_bytes": bwd_bytes,
                      "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.workload)},
     }
+    if args.graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        result["graph_replay"] = {"ms_per_step": round(graph_ms, 4),
+                                  "GBps": round(9 * s * N / (graph_ms * 1e-3) / 1e9, 1)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, g, x, G)
         if args.workload == "cfg1":

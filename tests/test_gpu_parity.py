@@ -676,6 +676,44 @@ def test_fm_memory_layer(scan, dtype, mem_norm, mem_in_loss):
         check(what, t_gpu, t_ref.numpy(), tol)
 
 
+def test_calls_can_be_captured_in_a_graph(scan):
+    """The entry points only enqueue kernels on the given stream (no allocation, no memset, no
+    synchronisation), so a forward + backward pair can be captured once and replayed. Every
+    replay is checked against the eager result, with eager work in between."""
+    B, M, D, L, dt = 2, 4, 8, 4096, torch.bfloat16
+    gen = gpu_gen(3)
+    g = torch.rand(B, M, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(B, D, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    z = torch.zeros(B, M, D, dtype=dt, device=DEV)
+    out, dx, dg = (torch.empty(B, M, D, L, dtype=dt, device=DEV) for _ in range(3))
+
+    def run():
+        scan.fm_scan_forward(g, x, z, out)
+        scan.fm_scan_backward(g, G, z, dx, out, x, dg)
+
+    run()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (out, dx, dg)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()  # warm-up on the capturing stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run()
+    for k in range(3):
+        for t in (out, dx, dg):
+            t.fill_(float(k))          # eager work between replays; also wipes the previous results
+        x.mul_(1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref, name in zip((out, dx, dg), want, ("states", "token grad", "gate grad")):
+            assert torch.equal(got, ref), (k, name)
+
+
 # ----------------------------------------------------------------------------- errors on the GPU
 
 def test_argument_errors_on_gpu(scan):
