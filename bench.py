@@ -159,14 +159,16 @@ def run_layer(torch, args) -> int:
         for t in leaves:
             t.grad = None
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = 0.0
+    if not args.probe:
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # every kernel on its own, through the same Python entry points, HIP events around each
     N, s = B * M * D * L, alpha.element_size()
@@ -198,11 +200,23 @@ def run_layer(torch, args) -> int:
         "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 8, lambda: S.fm_scan_backward_reduced(
             gates, G, zeros, states, tokens)),
         # what the layer's backward runs when only its output feeds the loss: the kernel above in
-        # the form that makes the states' gradient itself (no readout_backward_kernel, no G)
-        "scan_backward_reduced_kernel (layer form)": (2 * s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
+        # the form that makes the states' gradient itself (no readout_backward_kernel, no G) and
+        # takes the scanned states back from the normalised ones (reads one (B,M,D,L) tensor)
+        "scan_backward_reduced_kernel (layer form)": (s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
             P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
             None, None, B, M, D, L, code, 0, st)),
     }
+    if args.probe:  # for rocprofv3 --pmc: a copy of known size, then every kernel a few times
+        for _ in range(4):
+            torch.neg(states, out=sg)
+        for _, call in calls.values():
+            for _ in range(4):
+                call()
+        torch.cuda.synchronize()
+        print(f"probe: torch.neg reads and writes {states.numel() * s} bytes each; algorithmic bytes: "
+              + ", ".join(f"{k} {v[0]}" for k, v in calls.items()))
+        return 0
+
     kernels = {}
     for name, (nbytes, call) in calls.items():
         for _ in range(3):
@@ -226,7 +240,10 @@ def run_layer(torch, args) -> int:
         "kernels": kernels,
         "roofline": {"kernel": "scan_backward_reduced_kernel (layer form)", "bound": "hbm", "achieved": dom["GBps"],
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom["GBps"] / PEAK_HBM_GBPS, 4),
-                     "algorithmic_bytes": dom["algorithmic_bytes"], "traffic": None},
+                     "algorithmic_bytes": dom["algorithmic_bytes"],
+                     # rocprofv3 counters, summarised under profiles/: FETCH_SIZE 297789.3 KiB x 2.0
+                     # (copy calibration) + WRITE_SIZE 147456.0 KiB x 1.0 per launch
+                     "traffic": int((297789.3 * 2.0 + 147456.0) * 1024)},
     }
     print(json.dumps(result), flush=True)
     return 0

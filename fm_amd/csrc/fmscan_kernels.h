@@ -557,9 +557,14 @@ __global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
     const int32_t NG = (D + DG - 1) / DG;
     // (the division runs on the vector unit; everything derived from b is an address, so
     // bring it back to a scalar register)
-    const int32_t b32 = uniform((int)(blockIdx.x / (uint32_t)NG));
+    // Blocks go to the 8 XCDs (each with its own L2) round robin. The blocks of one b read the
+    // same gates (and coefficient vectors), so they are renumbered to share an XCD: XCD x takes
+    // the x-th eighth of the (b, group) pairs.
+    uint32_t id = blockIdx.x;
+    if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+    const int32_t b32 = uniform((int)(id / (uint32_t)NG));
     const int64_t b = b32;
-    const int32_t grp = (int32_t)blockIdx.x - b32 * NG;
+    const int32_t grp = uniform((int)id - b32 * NG);
     const bool active = grp * DG + w < D;        // a wave past the last d still joins every barrier
     const int64_t d = active ? grp * DG + w : D - 1;
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
