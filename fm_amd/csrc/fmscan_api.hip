@@ -123,9 +123,9 @@ Grid throttled_grid(const void* kern, std::atomic<uint64_t>& last_set, int64_t s
 // encodes: one or two waves per row stream best when there are many rows of moderate
 // length; long rows want eight waves side by side so that fewer rows are open at a
 // time; with few rows a block per row keeps every compute unit busy. One to two waves
-// per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few rows that even eight waves per row leave
-// compute units idle (fewer than 32 rows), and a workspace to hold the segment pairs,
-// rows are cut into segments (two passes).
+// per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few rows
+// that even eight waves per row leave compute units idle (fewer than 32 rows), and a
+// workspace to hold the segment pairs, rows are cut into segments (two passes).
 struct Tuning {
     unsigned waves, blocks_per_cu, depth;
     int32_t nseg;       // segments per row (1 = the row is scanned in one piece)

@@ -598,6 +598,29 @@ def test_layer_prepare_and_finish_kernels(scan, dtype):
         check(tag + " d_output_scale", d_os, (dr * a64).sum(axis=2, keepdims=True), tol)
 
 
+def test_scan_then_readout_equals_the_one_node_layer(scan):
+    """fm_scan followed by fm_readout (two autograd nodes, a (B, M, D, L) gradient between them) and
+    fm_layer (one node) are the same function: same values, gradients within the storage type's
+    rounding of each other."""
+    B, M, D, L, dt = 2, 4, 24, 2048, torch.bfloat16
+    gen = gpu_gen(17)
+    mk = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    g0, x0, h0, r0 = torch.sigmoid(mk(B, M, L) + 2).to(dt), mk(B, D, L).to(dt), mk(B, M, D).to(dt), mk(B, M, L).to(dt)
+    w = mk(B, D, L).to(dt)
+    grads = []
+    for route in ("two nodes", "one node"):
+        g, x, h, r = (t.clone().requires_grad_() for t in (g0, x0, h0, r0))
+        if route == "two nodes":
+            out, mem = scan.fm_readout(scan.fm_scan(g, x, h), r, True, 1e-5)
+        else:
+            out, mem = scan.fm_layer(g, x, h, r, True, 1e-5)
+        out.backward(w)
+        grads.append([out.detach(), mem.detach(), g.grad, x.grad, h.grad, r.grad])
+    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
+    for a, b, name in zip(grads[0][2:], grads[1][2:], ("d_gates", "d_tokens", "d_initial_state", "d_read")):
+        check(name, b, a.double().cpu().numpy(), 2e-2)
+
+
 def test_layer_keeps_no_second_copy_of_the_states(scan):
     """With the norm, backward works from the normalised states the layer returns (and inv_rms):
     the scanned states are not kept. Measured as allocated memory across the forward pass."""
