@@ -100,9 +100,8 @@ __device__ __forceinline__ u32x4 load16(const T* __restrict__ p) {
 
 // The VEC form never branches around its load: a chunk outside [0, L) reads the last
 // chunk of the row instead and is replaced by `fill` afterwards. A load that is only
-// sometimes issued would make the compiler wait for every outstanding load before each
-// use (it can no longer count how many newer ones are in flight), which throws the
-// prefetch distance away.
+// sometimes issued makes the compiler wait for every outstanding load before each use
+// (it can no longer count how many newer ones are in flight).
 template <typename T, bool VEC, bool ONCE>
 __device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t0, int64_t L,
                                             uint32_t fill) {
