@@ -187,8 +187,8 @@ __global__ __launch_bounds__(64 * W * R) void scan_forward_kernel(
     };
 
     // The steady part of the row runs without a single conditional memory operation and
-    // without bound checks (measured: 5-10 % faster than the checked loop, which waits for
-    // every load in flight before each use because it can no longer count the newer ones).
+    // without bound checks (measured faster than the checked loop, which waits for every
+    // load in flight before each use because it can no longer count the newer ones).
     // It covers the tiles whose prefetch target is still a whole tile; the rest of the row
     // takes the checked path. What the unrolled body does not do is wait tile by tile: the
     // compiler moves the first use of all P entries to its top, so the loads are waited
