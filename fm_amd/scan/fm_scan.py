@@ -31,9 +31,24 @@ __all__ = ["fm_scan_forward", "fm_scan_backward", "fm_scan_backward_reduced", "F
 _DTYPES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16,
            torch.bfloat16: _lib.DTYPE_BF16}
 
+class _Extension:
+    """Stands where the reference's `module` stands (fm_scan.py:18-35, the object load_inline
+    returns): `module.fm_scan_forward` and `module.fm_scan_backward` are the two extension
+    functions; every other attribute is an entry point of libfmscan_hip.so."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def __getattr__(self, name):
+        if name in ("fm_scan_forward", "fm_scan_backward"):
+            return globals()[name]
+        return getattr(self._lib, name)
+
+
 # the library is loaded when this module is imported, as the reference builds and
 # loads its extension at import (fm_scan.py:18-33); a missing library is an error here
-module = _lib.load()
+_raw = _lib.load()
+module = _Extension(_raw)
 
 
 def _require(cond: bool, what: str) -> None:
@@ -83,7 +98,7 @@ def _workspace(B, M, D, L, code, flags, device):
     None when the library scans every row in one piece."""
     if B * M * D >= 32 and not (flags >> _lib.FLAG_SEGMENTS_SHIFT):
         return None, 0  # rows are only cut on request or when there are very few of them
-    need = module.fmscan_workspace_bytes(B, M, D, L, code, flags)
+    need = _raw.fmscan_workspace_bytes(B, M, D, L, code, flags)
     if not need:
         return None, 0
     return torch.empty(need, dtype=torch.uint8, device=device), need
@@ -116,7 +131,7 @@ def fm_scan_forward(gates, tokens, initial_state, out, *, plain=False, waves_per
     with _on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         ws, ws_bytes = _workspace(B, M, D, L, code, flags, dev)
-        _lib.check(module.fmscan_forward(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+        _lib.check(_raw.fmscan_forward(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
                                          out.data_ptr(), B, M, D, L, code, flags,
                                          None if ws is None else ws.data_ptr(), ws_bytes, stream))
     return out
@@ -165,7 +180,7 @@ def fm_scan_backward(gates, outGrad, firstPropGrad, tokenGradOut, cached_output,
     with _on_device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         ws, ws_bytes = _workspace(B, M, D, L, code, flags, dev)
-        _lib.check(module.fmscan_backward(
+        _lib.check(_raw.fmscan_backward(
             gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), tokenGradOut.data_ptr(),
             cached_output.data_ptr(), input_tokens.data_ptr(), gateGradOut.data_ptr(),
             None if initial_state is None else initial_state.data_ptr(),
@@ -210,13 +225,13 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
         if t is not None:
             _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
     code = _dtype_code(gates)
-    groups = module.fmscan_reduced_groups(D)
+    groups = _raw.fmscan_reduced_groups(D)
     d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
     partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
     if cached_output.numel():
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            _lib.check(module.fmscan_backward_reduced(
+            _lib.check(_raw.fmscan_backward_reduced(
                 gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), d_tokens.data_ptr(),
                 cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(),
                 None if initial_state is None else initial_state.data_ptr(),
@@ -341,9 +356,9 @@ def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6, *, in_place=F
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             if mem_norm:
-                _lib.check(module.fmscan_readout_inv_rms(states.data_ptr(), inv_rms.data_ptr(), B, M, D, L,
+                _lib.check(_raw.fmscan_readout_inv_rms(states.data_ptr(), inv_rms.data_ptr(), B, M, D, L,
                                                          code, float(norm_eps), stream))
-            _lib.check(module.fmscan_readout_forward(states.data_ptr(), _ptr(inv_rms), read.data_ptr(),
+            _lib.check(_raw.fmscan_readout_forward(states.data_ptr(), _ptr(inv_rms), read.data_ptr(),
                                                      _ptr(normed), output.data_ptr(), B, M, D, L, code,
                                                      stream))
     return output, normed, inv_rms
@@ -380,10 +395,10 @@ def fm_readout_backward(out_grad, ext_grad, read, states_n, inv_rms, *, read_gra
     if states_n.numel():
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            _lib.check(module.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(),
+            _lib.check(_raw.fmscan_readout_dot(states_n.data_ptr(), out_grad.data_ptr(),
                                                  None if qe is None else ext_grad.data_ptr(), q.data_ptr(),
                                                  _ptr(qe), None, None, None, None, None, B, M, D, L, code, stream))
-            _lib.check(module.fmscan_readout_backward(states_n.data_ptr(), _ptr(inv_rms), read.data_ptr(),
+            _lib.check(_raw.fmscan_readout_backward(states_n.data_ptr(), _ptr(inv_rms), read.data_ptr(),
                                                       out_grad.data_ptr(), _ptr(ext_grad), q.data_ptr(),
                                                       _ptr(qe), state_grad.data_ptr(), B, M, D, L, code,
                                                       stream))
@@ -471,17 +486,17 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         coef_out, coef_self = torch.empty_like(read), torch.empty_like(read)
         rms = torch.empty_like(read) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
-        groups = module.fmscan_reduced_groups(D)
+        groups = _raw.fmscan_reduced_groups(D)
         d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
         zeros = torch.zeros((B, M, D), dtype=dtype, device=dev)
         d_h0 = torch.empty_like(zeros) if want_initial_state_grad else None
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            _lib.check(module.fmscan_readout_dot(
+            _lib.check(_raw.fmscan_readout_dot(
                 states_n.data_ptr(), out_grad.data_ptr(), None, q.data_ptr(), None, _ptr(inv_rms),
                 read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), _ptr(rms), B, M, D, L, code, stream))
-            _lib.check(module.fmscan_backward_layer(
+            _lib.check(_raw.fmscan_backward_layer(
                 gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
                 out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(),
                 None if mem_norm else states.data_ptr(),  # with the norm: states = states_n * rms
@@ -556,7 +571,7 @@ class FM_Memory(torch.autograd.Function):
         read = torch.empty_like(gates)
         if gates.numel():
             with _on_device(dev):
-                _lib.check(module.fmscan_layer_prepare(
+                _lib.check(_raw.fmscan_layer_prepare(
                     alpha.data_ptr(), update_scale.data_ptr(), output_scale.data_ptr(), gates.data_ptr(),
                     read.data_ptr(), B, L, M, code, torch.cuda.current_stream(dev).cuda_stream))
         tokens = _swap_last_two(inputs)
@@ -586,7 +601,7 @@ class FM_Memory(torch.autograd.Function):
         partial = partial.contiguous()
         if alpha.numel():
             with _on_device(dev):
-                _lib.check(module.fmscan_layer_finish(
+                _lib.check(_raw.fmscan_layer_finish(
                     partial.data_ptr(), partial.shape[2], q.data_ptr(), alpha.data_ptr(), update_scale.data_ptr(),
                     output_scale.data_ptr(), d_alpha.data_ptr(), d_update_scale.data_ptr(),
                     d_output_scale.data_ptr(), B, L, M, _dtype_code(alpha),
@@ -608,7 +623,7 @@ def _swap_last_two(t):
     out = torch.empty((B, C, R), dtype=t.dtype, device=t.device)
     if t.numel():
         with _on_device(t.device):
-            _lib.check(module.fmscan_swap_last_two(t.data_ptr(), out.data_ptr(), B, R, C, t.element_size(),
+            _lib.check(_raw.fmscan_swap_last_two(t.data_ptr(), out.data_ptr(), B, R, C, t.element_size(),
                                                    torch.cuda.current_stream(t.device).cuda_stream))
     return out
 

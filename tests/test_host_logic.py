@@ -1,6 +1,5 @@
-"""Host-side behaviour that needs no GPU: import paths, argument checks of the
-extension functions and of FM_Scan, and the layer arithmetic of fm_memory around
-the scan (with the scan itself replaced by the per-timestep PyTorch form)."""
+"""Host-side behaviour that needs no GPU: import paths, the `module` object, argument
+checks of the extension functions and of FM_Scan, loud failure on CPU tensors."""
 import numpy as np
 import pytest
 import torch
@@ -27,6 +26,18 @@ def test_product_does_not_import_the_oracle():
     root = Path(__file__).resolve().parent.parent
     res = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True)
     assert res.returncode == 0, res.stdout + res.stderr
+
+
+def test_module_stands_in_for_the_reference_extension():
+    """`module` is what load_inline returns in the reference (fm_scan.py:18-35): it carries the
+    two extension functions; here it also gives access to the library's C entry points."""
+    import fm.scan.fm_scan as m
+
+    assert m.module.fm_scan_forward is m.fm_scan_forward
+    assert m.module.fm_scan_backward is m.fm_scan_backward
+    assert m.module.fmscan_abi_version() >= 3
+    with pytest.raises(AttributeError):
+        m.module.no_such_entry_point
 
 
 def test_cpu_tensors_are_rejected_loudly():
