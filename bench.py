@@ -234,7 +234,7 @@ def run_layer(torch, args) -> int:
         "metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
         "value": round(N / (ms_per_step * 1e-3) / 1e9, 2), "unit": "Gelem/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16 storage, f32 arithmetic", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32", "storage_dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"layer: fm_memory (B,L,M,D)=({B},{L},{M},{D}) {dtn}, mem_norm, fwd+bwd via autograd",
                    "elements": N},
         "kernels": kernels,
@@ -340,7 +340,8 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"bfloat16": "bf16", "float32": "f32", "float16": "f16"}[dtn] + " storage, f32 arithmetic",
+        "dtype": "f32",  # the arithmetic type; tensors are stored as storage_dtype
+        "storage_dtype": {"bfloat16": "bf16", "float32": "f32", "float16": "f16"}[dtn],
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: (B,C,T)=({B},{Cn},{T}) {dtn}, fwd+bwd, passed as "
                                f"{rows} rows with M=D=1, FM form h=g*h+(1-g)*x",
