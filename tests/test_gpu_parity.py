@@ -699,6 +699,31 @@ def test_fm_memory_layer(scan, dtype, mem_norm, mem_in_loss):
         check(what, t_gpu, t_ref.numpy(), tol)
 
 
+def test_kernels_follow_the_current_stream(scan):
+    """Every call reads torch's current stream when it is made (the reference extension does the
+    same, fm_scan.cuh:271): work issued under a side stream is ordered there, not on the
+    default stream."""
+    B, L, M, D, dt = 2, 2048, 4, 32, torch.bfloat16
+    gen = gpu_gen(23)
+    alpha = torch.softmax(torch.randn(B, L, M, device=DEV, generator=gen), -1).to(dt)
+    us = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt)
+    osc = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt)
+    inp = torch.randn(B, L, D, device=DEV, generator=gen).to(dt)
+    want_out, want_mem = scan.fm_memory(alpha, us, osc, inp)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        # a long-running kernel first: were the layer's kernels on another stream, they would
+        # read `late` before it is written
+        big = torch.randn(64 * 1024 * 1024, device=DEV)
+        for _ in range(8):
+            big = big * 1.0001
+        late = (inp.float() + big[: inp.numel()].view_as(inp) * 0.0).to(dt)
+        out, mem = scan.fm_memory(alpha, us, osc, late)
+    side.synchronize()
+    assert torch.equal(out, want_out) and torch.equal(mem, want_mem)
+
+
 def test_calls_can_be_captured_in_a_graph(scan):
     """The entry points only enqueue kernels on the given stream (no allocation, no memset, no
     synchronisation), so a forward + backward pair can be captured once and replayed. Every
