@@ -71,3 +71,18 @@ def test_fm_scan_shape_asserts_match_reference_behaviour():
     with pytest.raises(AssertionError):  # initial state of the wrong shape
         fm_scan(torch.rand(2, 3, 32), torch.rand(2, 4, 32), torch.zeros(2, 4, 3))
 
+
+
+def test_bench_refuses_more_than_one_gpu_and_no_gpu():
+    """bench.py runs on one GPU: asked for more it says so and exits; without a GPU it says
+    that the scan has no CPU path to benchmark (it never falls back to the CPU checker)."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = Path(__file__).resolve().parents[1] / "bench.py"
+    two = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True)
+    assert two.returncode == 2 and "one GPU" in two.stderr and not two.stdout.strip()
+    if not torch.cuda.is_available():
+        one = subprocess.run([sys.executable, str(bench)], capture_output=True, text=True)
+        assert one.returncode == 1 and "no GPU" in one.stderr and not one.stdout.strip()
