@@ -245,8 +245,35 @@ def run_layer(torch, args) -> int:
                      # (copy calibration) + WRITE_SIZE 147456.0 KiB x 1.0 per launch
                      "traffic": int((297789.3 * 2.0 + 147456.0) * 1024)},
     }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = layer_cpu_baseline(torch, alpha, us, osc, inp, w_out)
     print(json.dumps(result), flush=True)
     return 0
+
+
+def layer_cpu_baseline(torch, alpha, us, osc, inp, w_out, batch=4):
+    """The float64 numpy oracle of the layer (forward, then the gradients of the read-out and of
+    the scan) on the first `batch` batch elements of the same inputs: one core, sequential in t."""
+    sys.path.insert(0, str(ROOT / "oracle"))
+    import numpy as np
+
+    import fm_scan_oracle as O
+
+    a, u, o, x, w = (O.to_f64(t.detach()[:batch]) for t in (alpha, us, osc, inp, w_out))
+    t0 = time.perf_counter()
+    write = np.ascontiguousarray(np.transpose(a * u, (0, 2, 1)))
+    tokens = np.ascontiguousarray(np.transpose(x, (0, 2, 1)))
+    read = np.ascontiguousarray(np.transpose(a * o, (0, 2, 1)))
+    gates = 1.0 - write
+    states = O.forward(gates, tokens)
+    out, normed, _ = O.readout_forward(states, read, True, 1e-6)
+    state_grad, read_grad = O.readout_backward(np.transpose(w, (0, 2, 1)), None, read, states, True, 1e-6)
+    O.backward(gates, tokens, state_grad, states=states)
+    el = time.perf_counter() - t0
+    n = states.size
+    return {"value": round(n / el / 1e9, 4), "unit": "Gelem/s", "cores": 1, "kind": "port",
+            "sample": f"first {batch} of {alpha.shape[0]} batch elements ({n} elements of the states), forward + "
+                      f"backward once in {el:.1f} s, float64 numpy oracle oracle/fm_scan_oracle.py"}
 
 
 def main() -> int:
