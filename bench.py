@@ -251,7 +251,7 @@ def run_layer(torch, args) -> int:
     return 0
 
 
-def layer_cpu_baseline(torch, alpha, us, osc, inp, w_out, batch=4):
+def layer_cpu_baseline(torch, alpha, us, osc, inp, w_out, batch=16):
     """The float64 numpy oracle of the layer (forward, then the gradients of the read-out and of
     the scan) on the first `batch` batch elements of the same inputs: one core, sequential in t."""
     sys.path.insert(0, str(ROOT / "oracle"))
