@@ -566,6 +566,15 @@ bool vector_path(const ReadoutShape& rs, std::initializer_list<const void*> poin
     return true;
 }
 
+// As for the scan kernels: an untouched slice of dynamic LDS per block bounds how many blocks
+// (rows that stream at once) a compute unit holds.
+constexpr unsigned kReadoutBlocksPerCU = 4;  // measured on the layer shapes of bench.py
+template <typename K>
+unsigned capped_lds(K kern, std::atomic<uint64_t>& last_set) {
+    if (kReadoutBlocksPerCU == 0) return 0;
+    return throttled_grid((const void*)kern, last_set, 1, 1, kReadoutBlocksPerCU).lds;
+}
+
 template <typename F>
 void with_bool(bool v, F&& f) {
     if (v) f(BoolTag<true>{});
@@ -624,10 +633,11 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
         using T = typename decltype(tt)::type;
         with_bool(inv_rms != nullptr, [&](auto nt) {
             with_bool(vec, [&](auto vt) {
-                fmscan::readout_forward_kernel<T, kReadoutRows, decltype(nt)::value, decltype(vt)::value>
-                    <<<grid, 256, 0, (hipStream_t)stream>>>((const T*)states, inv_rms, (const T*)read,
-                                                            (T*)states_out, (T*)output, (int32_t)M, (int32_t)D,
-                                                            L, rs.tiles);
+                auto kern = fmscan::readout_forward_kernel<T, kReadoutRows, decltype(nt)::value, decltype(vt)::value>;
+                static std::atomic<uint64_t> last_set{~0ull};
+                kern<<<grid, 256, capped_lds(kern, last_set), (hipStream_t)stream>>>(
+                    (const T*)states, inv_rms, (const T*)read, (T*)states_out, (T*)output, (int32_t)M, (int32_t)D,
+                    L, rs.tiles);
             });
         });
     });
@@ -707,12 +717,12 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
         with_bool(norm, [&](auto nt) {
             with_bool(ext_grad != nullptr, [&](auto et) {
                 with_bool(vec, [&](auto vt) {
-                    fmscan::readout_backward_kernel<T, kReadoutRows, decltype(nt)::value, decltype(et)::value,
-                                                    decltype(vt)::value>
-                        <<<grid, 256, 0, (hipStream_t)stream>>>((const T*)states_n, inv_rms, (const T*)read,
-                                                                (const T*)out_grad, (const T*)ext_grad, q, qe,
-                                                                (T*)state_grad, (int32_t)M, (int32_t)D, L,
-                                                                rs.tiles);
+                    auto kern = fmscan::readout_backward_kernel<T, kReadoutRows, decltype(nt)::value,
+                                                                decltype(et)::value, decltype(vt)::value>;
+                    static std::atomic<uint64_t> last_set{~0ull};
+                    kern<<<grid, 256, capped_lds(kern, last_set), (hipStream_t)stream>>>(
+                        (const T*)states_n, inv_rms, (const T*)read, (const T*)out_grad, (const T*)ext_grad, q, qe,
+                        (T*)state_grad, (int32_t)M, (int32_t)D, L, rs.tiles);
                 });
             });
         });
