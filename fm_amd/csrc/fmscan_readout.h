@@ -263,6 +263,35 @@ __global__ __launch_bounds__(256) void swap_last_two_kernel(const U* __restrict_
         if (c0 + i < C && r0 + lane < R) d[(c0 + i) * R + r0 + lane] = tile[lane][i];
 }
 
+// The same for 2-byte elements when R and C are even and both pointers 4-byte aligned: every
+// lane moves two neighbouring elements (4 bytes) on both sides, half a wave per row, so a wave
+// instruction covers two 128-byte runs instead of one.
+__global__ __launch_bounds__(256) void swap_last_two_pairs_kernel(const uint16_t* __restrict__ src,
+                                                                  uint16_t* __restrict__ dst, int64_t R, int64_t C,
+                                                                  int32_t tiles_c, int32_t tiles_r) {
+    __shared__ uint16_t tile[64][66];  // 132-byte rows: 4-byte aligned, odd in 4-byte words
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    const int half = lane >> 5, pair = lane & 31;
+    const int64_t per_b = (int64_t)tiles_c * tiles_r;
+    const int64_t b = blockIdx.x / per_b;
+    const int64_t rest = blockIdx.x - b * per_b;
+    const int64_t r0 = (rest / tiles_c) * 64, c0 = (rest % tiles_c) * 64;
+    const uint16_t* __restrict__ s = src + b * R * C;
+    uint16_t* __restrict__ d = dst + b * R * C;
+#pragma unroll 4
+    for (int i = 2 * w + half; i < 64; i += 8)
+        if (r0 + i < R && c0 + 2 * pair < C)
+            *reinterpret_cast<uint32_t*>(&tile[i][2 * pair]) =
+                *reinterpret_cast<const uint32_t*>(s + (r0 + i) * C + c0 + 2 * pair);
+    __syncthreads();
+#pragma unroll 4
+    for (int j = 2 * w + half; j < 64; j += 8)
+        if (c0 + j < C && r0 + 2 * pair < R)
+            *reinterpret_cast<uint32_t*>(d + (c0 + j) * R + r0 + 2 * pair) =
+                (uint32_t)tile[2 * pair][j] | ((uint32_t)tile[2 * pair + 1][j] << 16);
+}
+
 // gates[b, m, t] = 1 - alpha[b, t, m] * update_scale[b, t], read[b, m, t] = alpha[b, t, m] *
 // output_scale[b, t] (reference fm_scan.py:116,118-119,130: two products, two transposed
 // copies and a subtraction). 64 x 64 tiles of (t, m) through LDS; float32 arithmetic, one
