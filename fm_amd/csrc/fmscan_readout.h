@@ -361,16 +361,14 @@ __global__ __launch_bounds__(256) void layer_finish_kernel(
             float dg = 0.0f, dr = 0.0f;
             if (m < M && t < L) {
                 const float* __restrict__ p = gate_grad_partial + ((b * M + m) * G) * L + t;
-                float d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;  // four loads in flight per lane
+                float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};  // eight loads in flight per lane
                 int32_t g = 0;
-                for (; g + 4 <= G; g += 4) {
-                    dg += p[(int64_t)g * L];
-                    d1 += p[(int64_t)(g + 1) * L];
-                    d2 += p[(int64_t)(g + 2) * L];
-                    d3 += p[(int64_t)(g + 3) * L];
+                for (; g + 8 <= G; g += 8) {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc[u] += p[(int64_t)(g + u) * L];
                 }
-                for (; g < G; ++g) dg += p[(int64_t)g * L];
-                dg = (dg + d1) + (d2 + d3);
+                for (; g < G; ++g) acc[0] += p[(int64_t)g * L];
+                dg = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
                 dr = read_grad[(b * M + m) * L + t];
             }
             const float a = ta[lane][i];
