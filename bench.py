@@ -46,6 +46,7 @@ WORKLOADS = {
     "cfg3": (16, 2048, 16384, "bfloat16"),
     "cfg4": (4, 1024, 65536, "bfloat16"),
     "cfg5": (32, 4096, 2048, "bfloat16"),
+    "cfg5f16": (32, 4096, 2048, "float16"),  # configuration 5 in its other 16-bit type
 }
 
 # HBM bytes per backward launch read from rocprofv3 counters (FETCH_SIZE and
@@ -64,6 +65,8 @@ def make_inputs(torch, name, device):
     gen = torch.Generator(device=device).manual_seed(0)
     rn = lambda *s: torch.randn(*s, device=device, generator=gen)
     ru = lambda *s: torch.rand(*s, device=device, generator=gen)
+    if name == "cfg5f16":
+        name = "cfg5"
     if name == "cfg1":
         g = torch.sigmoid(rn(rows, 1, T) + 2.0)
         x = rn(rows, 1, T)
