@@ -23,14 +23,48 @@ FLAG_SEGMENTS_SHIFT = 20
 _lib = None
 
 
+def _open_current() -> ctypes.CDLL:
+    """The built library, rebuilt first when it is missing or older than its sources (its
+    build id is a hash of them). Without a compiler an outdated library is an error."""
+    try:
+        want = _build.source_id()
+    except OSError:
+        want = None  # the sources are not there (a deployed library): nothing to compare with
+    for attempt in (0, 1):
+        if _build.LIB.exists():
+            lib = ctypes.CDLL(str(_build.LIB))
+            try:
+                lib.fmscan_build_id.restype = c_char_p
+                lib.fmscan_build_id.argtypes = []
+                have = lib.fmscan_build_id().decode()
+            except AttributeError:
+                have = "none"
+            if want is None or have == want:
+                return lib
+            import _ctypes
+
+            _ctypes.dlclose(lib._handle)  # or loading the same path again would return this one
+            del lib
+            why = f"libfmscan_hip.so was built from other sources (build id {have}, sources {want})"
+        else:
+            why = "libfmscan_hip.so has not been built"
+        if attempt:
+            break
+        try:
+            _build.hipcc_path()
+        except RuntimeError:
+            raise RuntimeError(why + " and hipcc is not available; build it with `python -m fm_amd.build`")
+        # dlopen keeps a loaded file by path: build to the same path, then load it afresh
+        _build.build(verbose=False)
+    raise RuntimeError(why + " after a rebuild; run `python -m fm_amd.build` and check its output")
+
+
 def load() -> ctypes.CDLL:
-    """Loads the built library; builds it first only when no build exists."""
+    """Loads the built library (see _open_current) and declares its entry points."""
     global _lib
     if _lib is not None:
         return _lib
-    if not _build.LIB.exists():
-        _build.build(verbose=False)
-    lib = ctypes.CDLL(str(_build.LIB))
+    lib = _open_current()
     lib.fmscan_abi_version.restype = c_int
     lib.fmscan_abi_version.argtypes = []
     lib.fmscan_last_error.restype = c_char_p

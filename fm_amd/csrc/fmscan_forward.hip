@@ -1,0 +1,80 @@
+// fmscan_forward: argument checks, choice of kernel variant, launch.
+// Contract: include/fmscan.h.
+#include "fmscan_host.h"
+#include "fmscan_kernels.h"
+
+using namespace fmscan::host;
+
+namespace {
+
+template <typename T, int W, int R, int P, bool PLAIN, bool VEC, bool FOLD>
+int launch_fwd(const Problem& pb, const Tuning& t, const void* g, const void* x, const void* h0,
+               void* out, const float2* pairs, hipStream_t s) {
+    auto kern = fmscan::scan_forward_kernel<T, W, R, P, PLAIN, VEC, FOLD>;
+    static std::atomic<uint64_t> armed{0};
+    if (int rc = raise_lds_limit((const void*)kern, armed, "fmscan_forward")) return rc;
+    const unsigned blocks = (unsigned)((pb.rows * t.nseg + R - 1) / R);
+    kern<<<blocks, 64 * W * R, lds_share(t.blocks_per_cu), s>>>((const T*)g, (const T*)x, (const T*)h0, (T*)out,
+                                                                pb.rows, (int32_t)pb.M, (int32_t)pb.D, pb.L,
+                                                                t.nseg, t.seg_tiles, pairs);
+    return 0;
+}
+
+// Pass one of a segmented scan: one wave per segment, four segments per block.
+void launch_aggregate(int dtype, const Problem& pb, const Tuning& t, bool vec, const void* g,
+                      const void* other, float2* pairs, hipStream_t s) {
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        with_bool(pb.plain, [&](auto pt) {
+            with_bool(vec, [&](auto vt) {
+                constexpr int R = 4, P = 3;
+                auto kern = fmscan::scan_aggregate_kernel<T, R, P, decltype(pt)::value, decltype(vt)::value, false>;
+                const unsigned blocks = (unsigned)((pb.rows * t.nseg + R - 1) / R);
+                kern<<<blocks, 64 * R, 0, s>>>((const T*)g, (const T*)other, pairs, pb.rows, (int32_t)pb.M,
+                                              (int32_t)pb.D, pb.L, t.nseg, t.seg_tiles);
+            });
+        });
+    });
+}
+
+}  // namespace
+
+extern "C" {
+
+int fmscan_forward(const void* gates, const void* tokens, const void* initial_state, void* out,
+                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+    Problem pb;
+    if (int rc = parse(B, M, D, L, dtype, flags, &pb)) return rc;
+    if (!gates || !tokens || !out)
+        return fail(FMSCAN_E_NULL, "fmscan_forward: gates, tokens and out must not be NULL");
+    const Range o{"out", out, pb.rows * L * pb.esize};
+    const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
+                         {"tokens", tokens, B * D * L * pb.esize},
+                         {"initial_state", initial_state, pb.rows * pb.esize},
+                         {"workspace", workspace, (int64_t)workspace_bytes}};
+    for (const Range& in : ins)
+        if (overlap(o, in))
+            return fail(FMSCAN_E_ALIAS, "fmscan_forward: out overlaps %s", in.name);
+
+    const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(tokens) && aligned16(out);
+    Tuning tune;
+    if (int rc = settle(pb, false, workspace, workspace_bytes, "fmscan_forward", &tune)) return rc;
+    float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
+    if (pairs) {
+        launch_aggregate(dtype, pb, tune, vec, gates, tokens, pairs, (hipStream_t)stream);
+        if (int rc = launched("forward (segment pass)")) return rc;
+    }
+    const bool fold = M == 1 && D == 1;
+    int rc = 0;
+    dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
+        using T = typename decltype(tt)::type;
+        rc = launch_fwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
+                   decltype(vt)::value, decltype(ft)::value>(pb, tune, gates, tokens, initial_state, out,
+                                                             pairs, (hipStream_t)stream);
+    });
+    if (rc) return rc;
+    return launched("forward");
+}
+
+}  // extern "C"

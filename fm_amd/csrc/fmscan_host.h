@@ -1,0 +1,285 @@
+// Host-side pieces shared by the translation units of libfmscan_hip.so: error text,
+// argument checks, the choice of kernel variant, and the tags that turn run-time choices
+// into template arguments. Declarations and the contract of every entry point:
+// include/fmscan.h.
+#pragma once
+
+#include "../../include/fmscan.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <initializer_list>
+
+namespace fmscan {
+namespace host {
+
+// Text of the last rejected call on this thread (fmscan_last_error); defined in fmscan_core.hip.
+extern thread_local char g_err[512];
+
+inline int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+struct Range {
+    const char* name;
+    const void* p;
+    int64_t bytes;
+};
+inline bool overlap(const Range& a, const Range& b) {
+    if (!a.p || !b.p) return false;
+    const uintptr_t a0 = (uintptr_t)a.p, b0 = (uintptr_t)b.p;
+    return a0 < b0 + (uintptr_t)b.bytes && b0 < a0 + (uintptr_t)a.bytes;
+}
+
+struct Problem {
+    int64_t B, M, D, L, rows;
+    int esize;
+    unsigned waves;          // requested waves per row, 0 = auto
+    unsigned blocks_per_cu;  // requested cap on resident blocks per CU, 0 = auto
+    unsigned depth;          // requested prefetch depth in tiles, 0 = auto
+    unsigned segments;       // requested segments per row, 0 = auto
+    bool plain;
+};
+
+constexpr unsigned kKnownFlags = FMSCAN_FLAG_PLAIN | FMSCAN_FLAG_WAVES_MASK | FMSCAN_FLAG_BLOCKS_MASK |
+                                 FMSCAN_FLAG_DEPTH_MASK | FMSCAN_FLAG_SEGMENTS_MASK;
+
+inline int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, Problem* pb) {
+    if (B < 1 || M < 1 || D < 1 || L < 1)
+        return fail(FMSCAN_E_SHAPE, "fmscan: B, M, D, L must be >= 1 (got %lld, %lld, %lld, %lld)",
+                    (long long)B, (long long)M, (long long)D, (long long)L);
+    if (M > INT32_MAX || D > INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "fmscan: M and D must fit 32 bits");
+    if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16)
+        return fail(FMSCAN_E_DTYPE, "fmscan: dtype %d is not float32 (0), float16 (1) or bfloat16 (2)",
+                    dtype);
+    if (flags & ~kKnownFlags)
+        return fail(FMSCAN_E_FLAGS, "fmscan: unknown flag bits 0x%x", flags & ~kKnownFlags);
+    const unsigned waves = (flags & FMSCAN_FLAG_WAVES_MASK) >> FMSCAN_FLAG_WAVES_SHIFT;
+    if (waves != 0 && waves != 1 && waves != 2 && waves != 4 && waves != 8)
+        return fail(FMSCAN_E_FLAGS, "fmscan: waves per row must be 0 (auto), 1, 2, 4 or 8 (got %u)",
+                    waves);
+    const unsigned depth = (flags & FMSCAN_FLAG_DEPTH_MASK) >> FMSCAN_FLAG_DEPTH_SHIFT;
+    if (depth != 0 && (depth < 2 || depth > 4))
+        return fail(FMSCAN_E_FLAGS, "fmscan: prefetch depth must be 0 (auto), 2, 3 or 4 (got %u)", depth);
+    // rows*L elements must be addressable and the grid must fit 31 bits
+    const __int128 rows = (__int128)B * M * D;
+    if (rows > (__int128)INT32_MAX || rows * L > ((__int128)1 << 46))
+        return fail(FMSCAN_E_SHAPE, "fmscan: B*M*D = rows must be < 2^31 and rows*L <= 2^46");
+    pb->B = B; pb->M = M; pb->D = D; pb->L = L;
+    pb->rows = (int64_t)rows;
+    pb->esize = dtype == FMSCAN_DTYPE_F32 ? 4 : 2;
+    pb->waves = waves;
+    pb->blocks_per_cu = (flags & FMSCAN_FLAG_BLOCKS_MASK) >> FMSCAN_FLAG_BLOCKS_SHIFT;
+    pb->depth = depth;
+    pb->segments = (flags & FMSCAN_FLAG_SEGMENTS_MASK) >> FMSCAN_FLAG_SEGMENTS_SHIFT;
+    pb->plain = (flags & FMSCAN_FLAG_PLAIN) != 0;
+    return 0;
+}
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+inline int launched(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail((int)e, "fmscan: %s launch failed: %s", what, hipGetErrorString(e));
+    return 0;
+}
+
+// A kernel may ask for more dynamic LDS than the default limit only after the limit has been
+// raised for it. The limit is an upper bound, so it is raised once per (kernel, device) to
+// (nearly) all the LDS a compute unit has and never lowered: whatever a launch then asks for is within
+// it, and calls from several threads cannot undercut each other. `armed` belongs to one
+// kernel instantiation: bit d is set once the limit has been raised on device d (devices
+// beyond 63 raise it on every call). Returns 0 or a positive hipError_t with the text set.
+constexpr unsigned kLdsPerCU = 160u * 1024u;
+constexpr unsigned kMaxDynamicLds = kLdsPerCU - 2048u;  // 2 KiB stay free for the kernels' static LDS
+inline int raise_lds_limit(const void* kern, std::atomic<uint64_t>& armed, const char* who) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "%s: hipGetDevice failed: %s", who, hipGetErrorString(e));
+    const uint64_t bit = dev < 64 ? (1ull << dev) : 0ull;
+    if (bit && (armed.load(std::memory_order_acquire) & bit)) return 0;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynamicLds);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail((int)e, "%s: cannot raise the kernel's dynamic LDS limit to %u bytes: %s", who, kMaxDynamicLds,
+                    hipGetErrorString(e));
+    }
+    if (bit) armed.fetch_or(bit, std::memory_order_release);
+    return 0;
+}
+
+// Each block of the streaming kernels asks for a share of the 160 KiB of LDS of a compute
+// unit that it never touches: at most `blocks_per_cu` blocks then fit a unit at a time,
+// which bounds the number of rows that stream concurrently.
+inline unsigned lds_share(unsigned blocks_per_cu) {
+    return (kMaxDynamicLds / blocks_per_cu) & ~1023u;
+}
+
+// Waves per row, resident blocks per compute unit, prefetch depth and segments per row
+// when the caller leaves the choice to the library. The table comes from sweeps on an
+// MI355X over the benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536
+// in 16-bit types and 8192 x 4096 in float32, forward and backward separately. What it
+// encodes: one or two waves per row stream best when there are many rows of moderate
+// length; long rows want eight waves side by side so that fewer rows are open at a
+// time; with few rows a block per row keeps every compute unit busy. One to two waves
+// per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few rows
+// that even eight waves per row leave compute units idle (fewer than 32 rows), and a
+// workspace to hold the segment pairs, rows are cut into segments (two passes).
+struct Tuning {
+    unsigned waves, blocks_per_cu, depth;
+    int32_t nseg;       // segments per row (1 = the row is scanned in one piece)
+    int64_t seg_tiles;  // tiles per segment
+};
+constexpr int64_t kSplitBelowRows = 32;     // rows below which cutting rows pays (measured)
+constexpr int64_t kSplitTargetSlots = 2048;  // segments in flight the cut aims for
+constexpr int64_t kSplitMinTiles = 4;       // a segment is at least this many tiles
+constexpr int64_t kMaxSegments = 255;
+
+inline void plan_segments(const Problem& pb, Tuning& t, bool may_split) {
+    const int64_t tile1 = (16 / pb.esize) * 64;
+    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;
+    t.nseg = 1;
+    t.seg_tiles = tiles1;
+    if (!may_split) return;
+    int64_t want = pb.segments;
+    if (!want) {
+        if (pb.rows >= kSplitBelowRows || pb.waves) return;
+        want = (kSplitTargetSlots + pb.rows - 1) / pb.rows;
+        const int64_t most = tiles1 / kSplitMinTiles;
+        if (want > most) want = most;
+    }
+    if (want > tiles1) want = tiles1;
+    if (want > kMaxSegments) want = kMaxSegments;
+    if (want < 2) return;
+    const int64_t seg_tiles = (tiles1 + want - 1) / want;
+    const int64_t nseg = (tiles1 + seg_tiles - 1) / seg_tiles;
+    if (nseg < 2) return;
+    // a cut row is scanned by single waves: enough slots exist without sharing a row
+    t.waves = 1;
+    t.seg_tiles = seg_tiles;
+    t.nseg = (int32_t)nseg;
+}
+
+inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
+    Tuning t;
+    const int64_t tile1 = (16 / pb.esize) * 64;          // elements one wave covers per tile
+    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;   // tiles per row for one wave
+    // Gates shared by D rows and tokens shared by M rows come from the caches: the kernel
+    // then mostly writes (forward) and the limit on concurrent rows no longer applies.
+    // Measured on (B, M, D, L) = (32,32,128,2048), (1,32,2048,8192), (2,32,512,16384).
+    const bool shared_inputs = pb.M > 1 || pb.D > 1;
+    const bool long_rows = tiles1 >= 64, few_rows = pb.rows < 16384 && tiles1 >= 8;
+    unsigned w = pb.waves;
+    if (!w) {
+        if (shared_inputs && pb.rows >= 16384) w = 1;
+        else if (long_rows) w = 8;
+        else if (few_rows) w = 4;
+        else if (tiles1 >= 16) w = backward ? 1 : 2;
+        else if (tiles1 >= 8) w = backward ? 2 : 1;
+        else w = 1;
+        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
+        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
+    }
+    t.waves = w;
+    plan_segments(pb, t, may_split);
+    w = t.waves;
+    const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
+    unsigned bpc, depth;
+    if (shared_inputs) { bpc = 8; depth = 2; }
+    else if (w == 8) { bpc = backward ? 2 : 1; depth = 4; }
+    else if (w == 4) { bpc = 4; depth = backward ? 4 : 2; }
+    else if (w == 2) { bpc = 4; depth = 2; }
+    else if (tiles_per_slot >= 16) { bpc = backward ? 1 : 2; depth = 2; }
+    else if (tiles_per_slot >= 8) { bpc = 2; depth = 2; }
+    else { bpc = 4; depth = 2; }
+    t.blocks_per_cu = pb.blocks_per_cu ? pb.blocks_per_cu : bpc;
+    t.depth = pb.depth ? pb.depth : depth;
+    return t;
+}
+
+inline size_t pairs_bytes(const Problem& pb, const Tuning& t) {
+    return t.nseg > 1 ? (size_t)pb.rows * (size_t)t.nseg * sizeof(float2) : 0;
+}
+
+// Settles the plan for one call: rows are cut only when the workspace can hold the pairs.
+// Returns 0, FMSCAN_E_WORKSPACE when the caller asked for a cut that does not fit, or
+// FMSCAN_E_SHAPE when rows * segments does not fit a grid.
+inline int settle(const Problem& pb, bool backward, const void* workspace, size_t workspace_bytes, const char* who,
+                  Tuning* t) {
+    *t = choose(pb, backward, workspace != nullptr);
+    if (t->nseg > 1 && (pairs_bytes(pb, *t) > workspace_bytes || ((uintptr_t)workspace & 7u))) {
+        if (pb.segments > 1)
+            return fail(FMSCAN_E_WORKSPACE, "%s: %u segments per row need an 8-byte aligned workspace of "
+                        "%zu bytes (got %zu)", who, pb.segments, pairs_bytes(pb, *t), workspace_bytes);
+        *t = choose(pb, backward, false);
+    } else if (pb.segments > 1 && !workspace) {
+        return fail(FMSCAN_E_WORKSPACE, "%s: %u segments per row need a workspace", who, pb.segments);
+    }
+    // one block per slot at most (one per four slots with a wave per row): the grid is 31 bits
+    if ((__int128)pb.rows * t->nseg > (__int128)INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: rows * segments = %lld * %d must be < 2^31", who, (long long)pb.rows,
+                    (int)t->nseg);
+    return 0;
+}
+
+// Expands run-time choices into template arguments: F is a generic lambda called with tags.
+template <typename T> struct TypeTag { using type = T; };
+template <int V> struct IntTag { static constexpr int value = V; };
+template <bool V> struct BoolTag { static constexpr bool value = V; };
+
+template <typename F>
+void with_dtype(int dtype, F&& f) {
+    if (dtype == FMSCAN_DTYPE_F32) f(TypeTag<float>{});
+    else if (dtype == FMSCAN_DTYPE_F16) f(TypeTag<_Float16>{});
+    else f(TypeTag<__bf16>{});
+}
+
+template <typename F>
+void with_bool(bool v, F&& f) {
+    if (v) f(BoolTag<true>{});
+    else f(BoolTag<false>{});
+}
+
+// dtype, waves per row (with the rows per block that go with it), prefetch depth, plain,
+// vector access, fold -> f(tt, wt, rt, dt, pt, vt, ft)
+template <typename F>
+void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f) {
+    with_dtype(dtype, [&](auto tt) {
+        auto with_waves = [&](auto wt, auto rt) {
+            auto with_depth = [&](auto dt, auto vt, auto ft) {
+                if (plain) f(tt, wt, rt, dt, BoolTag<true>{}, vt, ft);
+                else f(tt, wt, rt, dt, BoolTag<false>{}, vt, ft);
+            };
+            if (!vec) {  // element access: the slow path gets one variant
+                with_depth(IntTag<2>{}, BoolTag<false>{}, BoolTag<false>{});
+                return;
+            }
+            auto with_fold = [&](auto dt) {
+                if (fold) with_depth(dt, BoolTag<true>{}, BoolTag<true>{});
+                else with_depth(dt, BoolTag<true>{}, BoolTag<false>{});
+            };
+            switch (t.depth) {
+                case 2: with_fold(IntTag<2>{}); break;
+                case 3: with_fold(IntTag<3>{}); break;
+                default: with_fold(IntTag<4>{}); break;
+            }
+        };
+        switch (t.waves) {
+            case 1: with_waves(IntTag<1>{}, IntTag<4>{}); break;  // 4 independent rows per block
+            case 2: with_waves(IntTag<2>{}, IntTag<1>{}); break;
+            case 4: with_waves(IntTag<4>{}, IntTag<1>{}); break;
+            default: with_waves(IntTag<8>{}, IntTag<1>{}); break;
+        }
+    });
+}
+
+}  // namespace host
+}  // namespace fmscan

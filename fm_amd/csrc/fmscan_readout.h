@@ -122,8 +122,8 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
 // once per slot and reused for the J rows.
 template <typename T, int J, bool NORM, bool VEC>
 __global__ __launch_bounds__(256) void readout_forward_kernel(
-    const T* __restrict__ states /* (B, M, D, L) */, const float* __restrict__ inv_rms /* (B, M, L) */,
-    const T* __restrict__ read /* (B, M, L) */, T* __restrict__ states_out /* (B, M, D, L) */,
+    const T* states /* (B, M, D, L) */, const float* __restrict__ inv_rms /* (B, M, L) */,
+    const T* __restrict__ read /* (B, M, L) */, T* states_out /* (B, M, D, L); may be `states` itself */,
     T* __restrict__ output /* (B, D, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
@@ -174,8 +174,8 @@ template <typename T, int J, bool NORM, bool EXT, bool VEC>
 __global__ __launch_bounds__(256) void readout_backward_kernel(
     const T* __restrict__ states_n /* (B, M, D, L), normalised; unused without the norm */,
     const float* __restrict__ inv_rms, const T* __restrict__ read, const T* __restrict__ out_grad /* (B, D, L) */,
-    const T* __restrict__ ext_grad /* (B, M, D, L) */, const float* __restrict__ q, const float* __restrict__ qe,
-    T* __restrict__ state_grad /* (B, M, D, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles) {
+    const T* ext_grad /* (B, M, D, L) */, const float* __restrict__ q, const float* __restrict__ qe,
+    T* state_grad /* (B, M, D, L); may be `ext_grad` itself */, int32_t M, int32_t D, int64_t L, int32_t tiles) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     const int lane = threadIdx.x & 63;

@@ -1,0 +1,132 @@
+// fmscan_backward_reduced and fmscan_backward_layer: the backward scan with the sums over
+// D and M inside. Contract: include/fmscan.h.
+#include "fmscan_host.h"
+#include "fmscan_reduced.h"
+
+using namespace fmscan::host;
+
+namespace {
+
+constexpr int kReducedGroup = 8;  // consecutive d one block of the reduced backward kernel sums over
+constexpr int kReducedChunk = 4;  // tiles of a row visited before moving to the next m
+constexpr int kLayerChunk = 2;    // ... in the form that makes the states' gradient on the spot
+constexpr int kReducedDepth = 1;  // visits whose loads are in flight ahead of the one worked on
+
+}  // namespace
+
+extern "C" {
+
+int64_t fmscan_reduced_groups(int64_t D) { return D < 1 ? 0 : (D + kReducedGroup - 1) / kReducedGroup; }
+
+// Shared by fmscan_backward_reduced and fmscan_backward_layer (coef_out != NULL): in the second
+// form `out_grad` carries the normalised states and the gradient of the states is made in the kernel.
+static int backward_reduced(const char* who, const void* gates, const void* out_grad, const void* first_prop_grad,
+                            void* token_grad, const void* cached_output, const void* input_tokens,
+                            float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                            const void* coef_out, const void* coef_self, const void* layer_out_grad,
+                            const void* rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                            unsigned flags, void* stream) {
+    Problem pb;
+    if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
+    if (flags & ~FMSCAN_FLAG_PLAIN)
+        return fail(FMSCAN_E_FLAGS, "%s: only FMSCAN_FLAG_PLAIN is understood here", who);
+    const bool layer = coef_out != nullptr;
+    const bool recover = layer && !cached_output;  // the states come back from states_n * rms
+    if (!gates || !out_grad || !token_grad || (!cached_output && !recover) || !gate_grad_partial)
+        return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
+                    "be NULL", who, coef_out ? "states_n" : "out_grad");
+    if (recover && !rms)
+        return fail(FMSCAN_E_NULL, "%s: without cached_output the states are states_n * rms: rms must "
+                    "not be NULL", who);
+    if (layer && (!coef_self || !layer_out_grad))
+        return fail(FMSCAN_E_NULL, "%s: coef_self and out_grad must not be NULL", who);
+    if (!pb.plain && !input_tokens)
+        return fail(FMSCAN_E_NULL, "%s: input_tokens must not be NULL without FMSCAN_FLAG_PLAIN", who);
+    if (B > INT32_MAX / fmscan_reduced_groups(D))
+        return fail(FMSCAN_E_SHAPE, "%s: B * ceil(D/%d) must be < 2^31", who, kReducedGroup);
+    const int64_t full = pb.rows * L * pb.esize;
+    const int64_t groups = fmscan_reduced_groups(D);
+    const Range outs[] = {{"token_grad", token_grad, B * D * L * pb.esize},
+                          {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
+                          {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
+    const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
+                         {layer ? "states_n" : "out_grad", out_grad, full},
+                         {"first_prop_grad", first_prop_grad, pb.rows * pb.esize},
+                         {"cached_output", cached_output, full},
+                         {"input_tokens", pb.plain ? nullptr : input_tokens, B * D * L * pb.esize},
+                         {"initial_state", initial_state, pb.rows * pb.esize},
+                         {"coef_out", coef_out, B * M * L * pb.esize},
+                         {"coef_self", layer ? coef_self : nullptr, B * M * L * pb.esize},
+                         {"out_grad", layer ? layer_out_grad : nullptr, B * D * L * pb.esize},
+                         {"rms", recover ? rms : nullptr, B * M * L * pb.esize}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
+    for (int i = 0; i < 3; ++i)
+        for (int j = i + 1; j < 3; ++j)
+            if (overlap(outs[i], outs[j]))
+                return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, outs[i].name, outs[j].name);
+    const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
+                     aligned16(token_grad) && aligned16(cached_output) && (!recover || aligned16(rms)) &&
+                     (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial) &&
+                     (!layer || (aligned16(coef_out) && aligned16(coef_self) && aligned16(layer_out_grad)));
+    if (!vec)
+        return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
+    const size_t tile = (size_t)(16 / pb.esize) * 64;
+    const size_t lds = (2 * kReducedGroup * tile + (size_t)kReducedGroup * (size_t)M) * sizeof(float);
+    if (lds > kMaxDynamicLds)
+        return fail(FMSCAN_E_SHAPE, "%s: M = %lld needs %zu bytes of LDS (limit %u)", who, (long long)M, lds,
+                    kMaxDynamicLds);
+    if ((L + (int64_t)tile - 1) / (int64_t)tile + kReducedChunk > INT32_MAX / M)
+        return fail(FMSCAN_E_SHAPE, "%s: M * ceil(L / %zu) must be < 2^31", who, tile);
+    const void* h_init = initial_state ? initial_state : first_prop_grad;
+    const unsigned grid = (unsigned)(B * groups);
+    int rc = 0;
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        auto go = [&](auto pt, auto lt, auto ct) {
+            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, decltype(ct)::value, kReducedDepth,
+                                                             decltype(pt)::value, decltype(lt)::value>;  // lt: 0 plain call, 1 layer, 2 layer + recovered states
+            static std::atomic<uint64_t> armed{0};
+            if ((rc = raise_lds_limit((const void*)kern, armed, who)) != 0) return;
+            kern<<<grid, 64 * kReducedGroup, lds, (hipStream_t)stream>>>(
+                (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
+                (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
+                (T*)initial_state_grad, (const T*)coef_out, (const T*)coef_self, (const T*)layer_out_grad,
+                (const T*)(recover ? rms : nullptr), (int32_t)M, (int32_t)D, L);
+        };
+        auto with_plain = [&](auto lt, auto ct) {
+            if (pb.plain) go(BoolTag<true>{}, lt, ct);
+            else go(BoolTag<false>{}, lt, ct);
+        };
+        // the layer forms hold three more loads per ring entry: two tiles per visit instead of four
+        if (recover) with_plain(IntTag<2>{}, IntTag<kLayerChunk>{});
+        else if (layer) with_plain(IntTag<1>{}, IntTag<kLayerChunk>{});
+        else with_plain(IntTag<0>{}, IntTag<kReducedChunk>{});
+    });
+    if (rc) return rc;
+    return launched(who);
+}
+
+int fmscan_backward_reduced(const void* gates, const void* out_grad, const void* first_prop_grad,
+                            void* token_grad, const void* cached_output, const void* input_tokens,
+                            float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                            int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                            void* stream) {
+    return backward_reduced("fmscan_backward_reduced", gates, out_grad, first_prop_grad, token_grad, cached_output,
+                            input_tokens, gate_grad_partial, initial_state, initial_state_grad, nullptr, nullptr,
+                            nullptr, nullptr, B, M, D, L, dtype, flags, stream);
+}
+
+int fmscan_backward_layer(const void* gates, const void* states_n, const void* coef_out, const void* coef_self,
+                          const void* out_grad, const void* first_prop_grad, void* token_grad,
+                          const void* cached_output, const void* rms, const void* input_tokens,
+                          float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                          int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, void* stream) {
+    if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer: coef_out must not be NULL");
+    return backward_reduced("fmscan_backward_layer", gates, states_n, first_prop_grad, token_grad, cached_output,
+                            input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
+                            out_grad, rms, B, M, D, L, dtype, flags, stream);
+}
+
+}  // extern "C"

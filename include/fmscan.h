@@ -81,6 +81,11 @@ extern "C" {
  * JIT-built from source at import, fm/scan/fm_scan.py:18-33). */
 int fmscan_abi_version(void);
 
+/* Hash of the sources and compiler flags the library was built from (16 hex digits), so
+ * that a loader can tell a library older than its sources. No counterpart in the
+ * reference, which compiles its source at every import (fm/scan/fm_scan.py:18-33). */
+const char* fmscan_build_id(void);
+
 /* Text of the last error raised on the calling thread ("" if none).
  * Replaces the c10::Error text of the reference's TORCH_CHECKs
  * (fm/scan/fm_scan.cuh:329,341,346-354,367-378). */

@@ -9,7 +9,7 @@
  * (fm/scan/fm_pytorch.py:35-38):
  *
  *   fmscan_oracle_*_f64   double in, double out: the checker.
- *   fmscan_cpu_*          storage dtype in/out (float32 or bfloat16), float32
+ *   fmscan_cpu_*          storage dtype in/out (float32, float16 or bfloat16), float32
  *                         arithmetic, OpenMP over rows: the timed CPU baseline.
  *
  * Formulas (the same for both):
@@ -92,6 +92,7 @@ void fmscan_oracle_backward_f64(const double* g, const double* G, const double* 
 /* ------------------------------------------------ storage-dtype port (timed baseline) */
 
 #define FMSCAN_CPU_F32 0
+#define FMSCAN_CPU_F16 1
 #define FMSCAN_CPU_BF16 2
 
 static inline float bf16_to_f32(uint16_t v) {
@@ -108,12 +109,58 @@ static inline uint16_t f32_to_bf16(float f) { /* round to nearest even; NaN kept
     return (uint16_t)(u >> 16);
 }
 
-#define LD(T, p, i) (sizeof(T) == 4 ? ((const float*)(p))[i] : bf16_to_f32(((const uint16_t*)(p))[i]))
-#define ST(T, p, i, v)                                        \
-    do {                                                      \
-        if (sizeof(T) == 4) ((float*)(p))[i] = (v);           \
-        else ((uint16_t*)(p))[i] = f32_to_bf16(v);            \
-    } while (0)
+/* IEEE binary16 <-> binary32 in integer arithmetic (the host compiler has no _Float16) */
+static inline float f16_to_f32(uint16_t v) {
+    const uint32_t sign = (uint32_t)(v & 0x8000u) << 16;
+    uint32_t exp = (v >> 10) & 0x1fu, man = v & 0x3ffu, u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+        } else { /* subnormal: normalise */
+            int sh = 0;
+            while (!(man & 0x400u)) { man <<= 1; ++sh; }
+            u = sign | ((uint32_t)(113 - sh) << 23) | ((man & 0x3ffu) << 13);
+        }
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | (man << 13);
+    } else {
+        u = sign | ((exp + 112) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static inline uint16_t f32_to_f16(float f) { /* round to nearest even */
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (a > 0x7f800000u ? 0x200u : 0u));
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* rounds to infinity */
+    if (a < 0x38800000u) {                                    /* subnormal or zero in binary16 */
+        if (a < 0x33000000u) return sign;                     /* below half the smallest subnormal */
+        const int e = (int)(a >> 23);
+        const uint32_t m = (a & 0x7fffffu) | 0x800000u;
+        const int shift = 126 - e; /* 14..24 */
+        uint32_t r = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (r & 1u))) ++r;
+        return (uint16_t)(sign | r);
+    }
+    uint32_t r = a - 0x38000000u; /* rebias */
+    r += 0xfffu + ((r >> 13) & 1u);
+    return (uint16_t)(sign | (r >> 13));
+}
+
+static inline float ld_f32(const float* p, int64_t i) { return p[i]; }
+static inline void st_f32(float* p, int64_t i, float v) { p[i] = v; }
+static inline float ld_bf16(const uint16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+static inline void st_bf16(uint16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+static inline float ld_f16(const uint16_t* p, int64_t i) { return f16_to_f32(p[i]); }
+static inline void st_f16(uint16_t* p, int64_t i, float v) { p[i] = f32_to_f16(v); }
+
+#define LD(T, p, i) LOAD((const T*)(p), i)
+#define ST(T, p, i, v) STORE((T*)(p), i, v)
 
 #define DEFINE_PORT(T, SUF)                                                                        \
     static void forward_##SUF(const T* g, const T* x, const T* h0, T* out, int64_t M, int64_t D,   \
@@ -167,8 +214,26 @@ static inline uint16_t f32_to_bf16(float f) { /* round to nearest even; NaN kept
         }                                                                                          \
     }
 
+#define LOAD ld_f32
+#define STORE st_f32
 DEFINE_PORT(float, f32)
+#undef LOAD
+#undef STORE
+#define LOAD ld_bf16
+#define STORE st_bf16
 DEFINE_PORT(uint16_t, bf16)
+#undef LOAD
+#undef STORE
+#define LOAD ld_f16
+#define STORE st_f16
+DEFINE_PORT(uint16_t, f16)
+#undef LOAD
+#undef STORE
+
+/* float32 -> binary16 bit patterns with the port's own rounding (for its conversion test) */
+void fmscan_cpu_round_f16(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = f32_to_f16(in[i]);
+}
 
 static void set_threads(int nthreads) {
 #ifdef _OPENMP
@@ -186,7 +251,7 @@ int fmscan_cpu_max_threads(void) {
 #endif
 }
 
-/* returns 0, or -3 for a dtype other than float32 (0) / bfloat16 (2) */
+/* returns 0, or -3 for a dtype other than float32 (0) / float16 (1) / bfloat16 (2) */
 int fmscan_cpu_forward(const void* g, const void* x, const void* h0, void* out, int64_t B, int64_t M,
                        int64_t D, int64_t L, int dtype, int plain, int nthreads) {
     set_threads(nthreads);
@@ -195,6 +260,9 @@ int fmscan_cpu_forward(const void* g, const void* x, const void* h0, void* out, 
     else if (dtype == FMSCAN_CPU_BF16)
         forward_bf16((const uint16_t*)g, (const uint16_t*)x, (const uint16_t*)h0, (uint16_t*)out, M, D, L,
                      B * M * D, plain);
+    else if (dtype == FMSCAN_CPU_F16)
+        forward_f16((const uint16_t*)g, (const uint16_t*)x, (const uint16_t*)h0, (uint16_t*)out, M, D, L,
+                    B * M * D, plain);
     else
         return -3;
     return 0;
@@ -211,6 +279,10 @@ int fmscan_cpu_backward(const void* g, const void* G, const void* fpg, void* dto
         backward_bf16((const uint16_t*)g, (const uint16_t*)G, (const uint16_t*)fpg, (uint16_t*)dtok,
                       (const uint16_t*)h, (const uint16_t*)x, (uint16_t*)dgate, (const uint16_t*)h0, M, D, L,
                       B * M * D, plain);
+    else if (dtype == FMSCAN_CPU_F16)
+        backward_f16((const uint16_t*)g, (const uint16_t*)G, (const uint16_t*)fpg, (uint16_t*)dtok,
+                     (const uint16_t*)h, (const uint16_t*)x, (uint16_t*)dgate, (const uint16_t*)h0, M, D, L,
+                     B * M * D, plain);
     else
         return -3;
     return 0;

@@ -3,7 +3,7 @@
 `forward_f64` / `backward_f64` are the compiled float64 checker (same results as
 oracle/fm_scan_oracle.py, fast enough for millions of elements);
 `port_forward` / `port_backward` run the storage-dtype float32-arithmetic port
-on torch CPU tensors (float32 or bfloat16): the timed CPU baseline.
+on torch CPU tensors (float32, float16 or bfloat16): the timed CPU baseline.
 Reference lines each C function follows: see the header of fmscan_cpu.c.
 """
 from __future__ import annotations
@@ -91,7 +91,7 @@ def backward_f64(gates, out_grad, states, tokens, first_prop_grad=None, initial_
 def _dtype_code(t):
     import torch
 
-    return {torch.float32: 0, torch.bfloat16: 2}[t.dtype]
+    return {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[t.dtype]
 
 
 def max_threads() -> int:

@@ -24,7 +24,7 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
-                                    "fmscan_backward_reduced",
+                                    "fmscan_backward_reduced", "fmscan_build_id",
                                     "fmscan_forward", "fmscan_last_error", "fmscan_layer_finish",
                                     "fmscan_layer_prepare", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
@@ -118,6 +118,52 @@ def test_rejected_arguments(lib):
     assert bwd(lib, dx=4 * P) == E_ALIAS              # token_grad_out on top of cached_output
     assert bwd(lib, dg=3 * P) == E_ALIAS              # the two outputs on top of each other
     assert b"overlaps" in lib.fmscan_last_error()
+
+
+def test_rows_times_segments_must_fit_a_grid(lib):
+    """A requested cut that would need 2^31 or more blocks is rejected, not truncated."""
+    rows, L, seg = 1 << 24, 1 << 16, 255
+    need = rows * seg * 8
+    Q = 1 << 44  # each tensor spans 2^41 bytes here
+    assert fwd(lib, g=Q, x=2 * Q, out=3 * Q, B=rows, L=L, dtype=2, flags=seg << 20, ws=7 * Q,
+               ws_bytes=need) == _const("FMSCAN_E_SHAPE")
+    assert b"segments" in lib.fmscan_last_error()
+    assert bwd(lib, g=Q, G=2 * Q, dx=3 * Q, h=4 * Q, x=5 * Q, dg=6 * Q, B=rows, L=L, dtype=2, flags=seg << 20,
+               ws=7 * Q, ws_bytes=need) == _const("FMSCAN_E_SHAPE")
+    assert lib.fmscan_workspace_bytes(rows, 1, 1, L, 2, seg << 20) == 0
+
+
+def test_error_text_is_per_thread(lib):
+    """Two threads issue rejected calls at the same time; each reads its own message afterwards
+    (the calls are stateless apart from this per-thread text)."""
+    import threading
+
+    barrier = threading.Barrier(2)
+    seen = {}
+
+    def worker(name, kwargs, word):
+        for _ in range(200):
+            barrier.wait()
+            rc = fwd(lib, **kwargs)
+            barrier.wait()  # the other thread's call has failed too by now
+            text = lib.fmscan_last_error()
+            if rc >= 0 or word not in text:
+                seen[name] = (rc, text)
+                break
+        else:
+            seen[name] = "ok"
+
+    a = threading.Thread(target=worker, args=("a", {"dtype": 7}, b"dtype"))
+    b = threading.Thread(target=worker, args=("b", {"g": None}, b"NULL"))
+    a.start(); b.start(); a.join(); b.join()
+    assert seen == {"a": "ok", "b": "ok"}, seen
+
+
+def test_build_id_matches_the_sources(lib):
+    from fm_amd import build
+
+    lib.fmscan_build_id.restype = ctypes.c_char_p
+    assert lib.fmscan_build_id().decode() == build.source_id()
 
 
 def test_rejected_readout_arguments(lib):

@@ -334,7 +334,7 @@ def test_c_oracle_equals_numpy_oracle(plain):
         np.testing.assert_allclose(gc, gg, rtol=1e-14, atol=1e-14)
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2), (torch.float16, 1e-2)])
 def test_cpu_port_within_tolerance_of_f64(dtype, tol):
     gen = torch.Generator().manual_seed(16)
     B, M, D, L = 2, 2, 3, 1000
@@ -351,3 +351,34 @@ def test_cpu_port_within_tolerance_of_f64(dtype, tol):
     C.port_backward(g, G, None, dx, out, x, dg, initial_state=h0)
     tr, gr = C.backward_f64(g, G, out, x, None, h0)
     assert nerr(dx, tr) <= tol and nerr(dg, gr) <= tol
+
+
+def test_cpu_port_float16_conversions_equal_numpy():
+    """The port's own binary16 conversions (the host compiler has no half type) against numpy's:
+    the scan with gate 0 stores exactly the token (a load, a multiply by one, a store), so every
+    binary16 value must come back unchanged; and the store's float32 -> binary16 rounding must be
+    numpy's (nearest even, subnormals, overflow to infinity)."""
+    bits = np.arange(65536, dtype=np.uint16)
+    vals = bits.view(np.float16)
+    # (an infinite state times a zero gate is NaN for the step after; 0 * h + (-0) is +0)
+    keep = np.isfinite(vals) & (bits != 0x8000)
+    x = torch.from_numpy(vals[keep].copy()).view(1, 1, -1)
+    g = torch.zeros_like(x)
+    out = torch.empty(1, 1, 1, x.shape[-1], dtype=torch.float16)
+    C.port_forward(g, x, None, out)
+    assert np.array_equal(out.view(-1).numpy().view(np.uint16), vals[keep].view(np.uint16))
+    # rounding on store
+    rng = np.random.default_rng(3)
+    cases = np.concatenate([rng.standard_normal(4096).astype(np.float32) * np.float32(s)
+                            for s in (1e-8, 1e-6, 1e-4, 1.0, 300.0, 70000.0)])
+    ties = (np.arange(1, 2049, dtype=np.float32) * 2 + 1) * np.float32(2.0 ** -11)  # halfway between neighbours
+    cases = np.concatenate([cases, ties, ties * np.float32(2.0 ** -14), [65504.0, 65519.9, 65520.0, 1e9]]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = cases.astype(np.float16)
+    lib = C.load()
+    got = np.empty(cases.shape, np.uint16)
+    import ctypes
+    lib.fmscan_cpu_round_f16.restype = None
+    lib.fmscan_cpu_round_f16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    lib.fmscan_cpu_round_f16(cases.ctypes.data, got.ctypes.data, cases.size)
+    assert np.array_equal(got, want.view(np.uint16))
