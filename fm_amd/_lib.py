@@ -75,6 +75,9 @@ def load() -> ctypes.CDLL:
     lib.fmscan_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_int64, c_int64, c_int64, c_int, c_uint,
                                    c_void_p, c_size_t, c_void_p]
+    lib.fmscan_forward_static.restype = c_int
+    lib.fmscan_forward_static.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_int64, c_int64, c_int64, c_int64, c_int, c_uint, c_void_p]
     lib.fmscan_backward.restype = c_int
     lib.fmscan_backward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_void_p, c_void_p,

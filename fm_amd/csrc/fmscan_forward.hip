@@ -1,9 +1,16 @@
-// fmscan_forward: argument checks, choice of kernel variant, launch.
+// fmscan_forward and fmscan_forward_static: argument checks, choice of kernel variant, launch.
 // Contract: include/fmscan.h.
 #include "fmscan_host.h"
 #include "fmscan_kernels.h"
 
 using namespace fmscan::host;
+
+// The segment pairs of fmscan_forward_static.
+// Device memory that belongs to the library: every GPU the library runs on holds its own
+// copy of this array (64 KiB) from the first call on it until the process ends. Host code
+// must not use the array's name as an address; it asks the runtime for the array's address
+// on the current device and hands that to the kernels like any other workspace.
+static __device__ __align__(256) float2 scratch[FMSCAN_STATIC_PAIRS];
 
 namespace {
 
@@ -37,17 +44,42 @@ void launch_aggregate(int dtype, const Problem& pb, const Tuning& t, bool vec, c
     });
 }
 
-}  // namespace
+// ---- the segment pairs of fmscan_forward_static (the array itself is at the top of the file)
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-extern "C" {
+// Address of `scratch` on the device that is current, looked up once per device.
+int static_pairs(void** ptr) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return fail((int)e, "fmscan_forward_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(FMSCAN_E_SHAPE, "fmscan_forward_static: device %d is beyond the %d this call keeps a "
+                    "workspace for", dev, kMaxDevices);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return fail(e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol,
+                        "fmscan_forward_static: cannot locate the library's workspace on device %d: %s", dev,
+                        hipGetErrorString(e));
+        }
+        g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+    }
+    *ptr = p;
+    return 0;
+}
 
-int fmscan_forward(const void* gates, const void* tokens, const void* initial_state, void* out,
-                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
-                   void* workspace, size_t workspace_bytes, void* stream) {
+// Both forward entry points: `who` names the one that was called.
+int forward(const char* who, const void* gates, const void* tokens, const void* initial_state, void* out,
+            int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+            void* workspace, size_t workspace_bytes, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags, &pb)) return rc;
     if (!gates || !tokens || !out)
-        return fail(FMSCAN_E_NULL, "fmscan_forward: gates, tokens and out must not be NULL");
+        return fail(FMSCAN_E_NULL, "%s: gates, tokens and out must not be NULL", who);
     const Range o{"out", out, pb.rows * L * pb.esize};
     const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
                          {"tokens", tokens, B * D * L * pb.esize},
@@ -55,11 +87,11 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
                          {"workspace", workspace, (int64_t)workspace_bytes}};
     for (const Range& in : ins)
         if (overlap(o, in))
-            return fail(FMSCAN_E_ALIAS, "fmscan_forward: out overlaps %s", in.name);
+            return fail(FMSCAN_E_ALIAS, "%s: out overlaps %s", who, in.name);
 
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(tokens) && aligned16(out);
     Tuning tune;
-    if (int rc = settle(pb, false, workspace, workspace_bytes, "fmscan_forward", &tune)) return rc;
+    if (int rc = settle(pb, false, workspace, workspace_bytes, who, &tune)) return rc;
     float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
     if (pairs) {
         launch_aggregate(dtype, pb, tune, vec, gates, tokens, pairs, (hipStream_t)stream);
@@ -75,6 +107,26 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
     });
     if (rc) return rc;
     return launched("forward");
+}
+
+}  // namespace
+
+extern "C" {
+
+int fmscan_forward(const void* gates, const void* tokens, const void* initial_state, void* out,
+                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+    return forward("fmscan_forward", gates, tokens, initial_state, out, B, M, D, L, dtype, flags, workspace,
+                   workspace_bytes, stream);
+}
+
+int fmscan_forward_static(const void* gates, const void* tokens, const void* initial_state, void* out,
+                          int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                          void* stream) {
+    void* ws = nullptr;
+    if (int rc = static_pairs(&ws)) return rc;
+    return forward("fmscan_forward_static", gates, tokens, initial_state, out, B, M, D, L, dtype, flags, ws,
+                   sizeof(float2) * FMSCAN_STATIC_PAIRS, stream);
 }
 
 }  // extern "C"

@@ -115,6 +115,28 @@ int fmscan_forward(const void* gates, const void* tokens, const void* initial_st
                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * fmscan_forward for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it) and so cannot bring the workspace
+ * that cut rows need: same arguments and results as fmscan_forward, with the segment pairs
+ * in device memory that the library itself holds, a static array of FMSCAN_STATIC_PAIRS
+ * pairs (64 KiB) on every GPU the call has been used on, kept until the process ends. It
+ * has no counterpart in the reference (whose kernel gives a whole row to one block and
+ * needs no workspace, fm/scan/fm_scan.cuh:62-64,84). The call allocates nothing. Every
+ * automatic cut fits (fewer than 32 rows, at most 255 segments each); a requested cut
+ * (FMSCAN_FLAG_SEGMENTS) of more than FMSCAN_STATIC_PAIRS segments in total is rejected
+ * with FMSCAN_E_WORKSPACE. All calls on one GPU share the array: calls whose rows are cut
+ * must not overlap in time on the same GPU (different streams, different threads), or
+ * they overwrite each other's pairs. Nothing in the array needs clearing between calls:
+ * every pair a call reads, that call has written first. The first call on a GPU looks up
+ * the array's address; make that call before capturing a graph.
+ */
+#define FMSCAN_STATIC_PAIRS 8192
+int fmscan_forward_static(const void* gates, const void* tokens, const void* initial_state,
+                          void* out,
+                          int64_t B, int64_t M, int64_t D, int64_t L,
+                          int dtype, unsigned flags, void* stream);
+
+/*
  * Backward scan. Replaces fm_scan_backward (reference fm/scan/fm_scan.cuh:361-381)
  * and the backward instantiation of its kernel (:42-218 with reverse=true,
  * backward=true; gate shift :103-108, epilogues :184-185 and :188-208).
