@@ -211,6 +211,51 @@ __device__ __forceinline__ void wave_scan_inclusive(float& a, float& b) {
         : "+v"(a), "+v"(b));
 }
 
+// The same scan in the other lane direction, for step pairs whose time order runs from lane
+// 63 down to lane 0 (the backward kernels lay a tile out that way and still need states that
+// run forward in time). DPP has no row broadcast towards lower lanes, so this comes in two
+// parts. First every row of 16 lanes scans itself: on exit lane l holds the composition of
+// the chunks of lanes (l | 15) down to l.
+__device__ __forceinline__ void row_scan_inclusive_down(float& a, float& b) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shl:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shl:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_fmac_f32_dpp %1, %1, %0 row_shl:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "+v"(b));
+}
+
+constexpr int kRowShl1 = 0x101;  // lane i <- lane i+1 inside its row of 16
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(v), lane));
+}
+
+// Second part: the state that enters every lane's chunk when `entry` (the same in all lanes)
+// enters lane 63's. (a, b) are the row-scanned pairs of row_scan_inclusive_down. The totals of
+// rows 3, 2, 1 sit in lanes 48, 32, 16; three chained steps on wave-uniform values carry the
+// state from row to row, and inside a row a lane applies the pairs of the lanes above it.
+__device__ __forceinline__ float state_entering_lane_down(float a, float b, float entry, int lane) {
+    const float e3 = entry;
+    const float e2 = __builtin_fmaf(lane_value(a, 48), e3, lane_value(b, 48));
+    const float e1 = __builtin_fmaf(lane_value(a, 32), e2, lane_value(b, 32));
+    const float e0 = __builtin_fmaf(lane_value(a, 16), e1, lane_value(b, 16));
+    const int row = lane >> 4;
+    const float e = row == 3 ? e3 : (row == 2 ? e2 : (row == 1 ? e1 : e0));
+    const float xa = dpp<kRowShl1>(1.0f, a);  // the lanes above, inside the row
+    const float xb = dpp<kRowShl1>(0.0f, b);
+    return __builtin_fmaf(xa, e, xb);
+}
+
 __device__ __forceinline__ float lane63(float v) {
     return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(v), 63));
 }

@@ -182,7 +182,7 @@ inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
         if (shared_inputs && pb.rows >= 16384) w = 1;
         else if (long_rows) w = 8;
         else if (few_rows) w = 4;
-        else if (tiles1 >= 16) w = backward ? 1 : 2;
+        else if (tiles1 >= 16) w = 1;
         else if (tiles1 >= 8) w = backward ? 2 : 1;
         else w = 1;
         while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
@@ -194,10 +194,10 @@ inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
     const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
     unsigned bpc, depth;
     if (shared_inputs) { bpc = 8; depth = 2; }
-    else if (w == 8) { bpc = backward ? 2 : 1; depth = 4; }
+    else if (w == 8) { bpc = 1; depth = backward ? 2 : 4; }
     else if (w == 4) { bpc = 4; depth = backward ? 4 : 2; }
     else if (w == 2) { bpc = 4; depth = 2; }
-    else if (tiles_per_slot >= 16) { bpc = backward ? 1 : 2; depth = 2; }
+    else if (tiles_per_slot >= 16) { bpc = 2; depth = 2; }
     else if (tiles_per_slot >= 8) { bpc = 2; depth = 2; }
     else { bpc = 4; depth = 2; }
     t.blocks_per_cu = pb.blocks_per_cu ? pb.blocks_per_cu : bpc;

@@ -273,9 +273,16 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
 
     const int64_t lane_off = (int64_t)(64 * W - 1 - (w * 64 + lane)) * E;
 
+    // PLAIN reads the saved states (its gate gradient needs nothing else). Otherwise the
+    // states of a tile are not read but made again, in float32, from the tile's gates and
+    // tokens (already in registers) and the one saved state just before this wave's part of
+    // the tile: a second wave scan, forward in time, in place of a fourth 16-byte stream.
     struct Entry {
-        u32x4 g, G, h, x;
-        float hb;  // lane 63 only: h just before this wave's part of the tile (h[-1] at t = 0)
+        u32x4 g, G;
+        u32x4 hx;  // PLAIN: saved states; otherwise tokens
+        float hb;  // h just before this wave's part of the tile (h[-1] at t = 0)
+        float h_first;  // checked tiles only, when this wave's part begins the row (`first`): the saved h[0]
+        bool first;
     };
     // tiles in [k_lo, k_whole) lie wholly inside the row
     const int64_t k_whole = VEC ? L / TILE : 0;
@@ -286,17 +293,19 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
         const int64_t t0 = k * TILE + lane_off;
         q.g = load16<T, FOLD>(grow + t0);
         q.G = load16<T, true>(Grow + t0);
-        q.h = load16<T, true>(hrow + t0);
-        if constexpr (!PLAIN) q.x = load16<T, FOLD>(xrow + t0);
+        if constexpr (PLAIN) q.hx = load16<T, true>(hrow + t0);
+        else q.hx = load16<T, FOLD>(xrow + t0);
         q.hb = Elem<T>::widen(hrow[k * TILE + wave_off - 1]);
+        q.h_first = 0.0f;  // never looked at: whole tiles are not the first of a row
+        q.first = false;
     };
     auto fetch = [&](Entry& q, int64_t k) {
         // k < k_lo (before the segment): t0 = L, which every bound check rejects
         const int64_t t0 = k >= seg.k_lo ? k * TILE + lane_off : L;
         q.g = load_chunk<T, VEC, FOLD>(grow, t0, L, Elem<T>::kOnes);
         q.G = load_chunk<T, VEC, true>(Grow, t0, L, 0u);
-        q.h = load_chunk<T, VEC, true>(hrow, t0, L, 0u);
-        if constexpr (!PLAIN) q.x = load_chunk<T, VEC, FOLD>(xrow, t0, L, 0u);
+        if constexpr (PLAIN) q.hx = load_chunk<T, VEC, true>(hrow, t0, L, 0u);
+        else q.hx = load_chunk<T, VEC, FOLD>(xrow, t0, L, 0u);
         // h just before this wave's part of the tile: one address for the whole wave,
         // always loaded (position 0 stands in where there is nothing before) and replaced by
         // h[-1] at the start of the row
@@ -304,16 +313,21 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
         const bool before = k >= seg.k_lo && tw > 0 && tw < L;
         const float loaded = Elem<T>::widen(hrow[before ? tw - 1 : 0]);
         q.hb = before ? loaded : hinit;
+        // Where the part begins the row, `hinit` is what the gate gradient at t = 0 is to see,
+        // which need not be the state the forward call started from (a caller that passes no
+        // initial state gets the reference's first_prop_grad there). The states after it are
+        // therefore made from the saved h[0], which `loaded` then holds.
+        q.h_first = loaded;
+        q.first = k >= seg.k_lo && tw == 0;
     };
 
     // One tile: fold, wave scan, meet the other waves, replay with both epilogues, store.
     // `whole` tiles store without a bound check.
     auto scan_tile = [&](const Entry& cur, int64_t k, auto whole) {
         const int64_t t0 = k * TILE + lane_off;
-        float g[E], G[E], h[E], p[E];
+        float g[E], G[E], p[E];
         Elem<T>::unpack(cur.g, g);
         Elem<T>::unpack(cur.G, G);
-        Elem<T>::unpack(cur.h, h);
 #pragma unroll
         for (int i = 0; i < E; ++i) p[i] = g[i] * G[i];
 
@@ -324,13 +338,46 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
             b = __builtin_fmaf(g[i], b, p[i]);
             a *= g[i];
         }
+        float fa = a;  // the product of the chunk's gates serves the forward step pair too
         wave_scan_inclusive(a, b);
         const float ea = dpp<kWaveShr1>(1.0f, a);
         const float eb = dpp<kWaveShr1>(0.0f, b);
         const float ta = lane63(a), tb = lane63(b);
-        // h at the position before this chunk: last element of the chunk before it
-        // in memory, which the next lane holds; lane 63 takes the look-behind value.
-        const float hprev0 = dpp<kWaveShl1>(cur.hb, h[E - 1]);
+
+        // hp[i] = h at the position before element i of the chunk; x[] the tokens
+        float hp[E], x[E];
+        if constexpr (PLAIN) {
+            float h[E];
+            Elem<T>::unpack(cur.hx, h);
+            // the last element of the chunk before this one in memory, which the next lane
+            // holds; lane 63 takes the look-behind value
+            hp[0] = dpp<kWaveShl1>(cur.hb, h[E - 1]);
+#pragma unroll
+            for (int i = 1; i < E; ++i) hp[i] = h[i - 1];
+        } else {
+            float u[E];
+            Elem<T>::unpack(cur.hx, x);
+#pragma unroll
+            for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], x[i], x[i]);  // as the forward kernel forms it
+            float g0 = g[0];
+            if constexpr (!decltype(whole)::value) {
+                // first step of the row: whatever enters, the saved h[0] leaves
+                if (lane == 63 && cur.first) {
+                    g0 = 0.0f;
+                    u[0] = cur.h_first;
+                    fa = 0.0f;
+                }
+            }
+            float fb = u[0];
+#pragma unroll
+            for (int i = 1; i < E; ++i) fb = __builtin_fmaf(g[i], fb, u[i]);
+            // positions past the end of the row carry g = 1, x = 0: identity steps
+            row_scan_inclusive_down(fa, fb);
+            hp[0] = state_entering_lane_down(fa, fb, cur.hb, lane);
+            hp[1] = __builtin_fmaf(g0, hp[0], u[0]);
+#pragma unroll
+            for (int i = 2; i < E; ++i) hp[i] = __builtin_fmaf(g[i - 1], hp[i - 1], u[i - 1]);
+        }
 
         float cin = carry;
         if constexpr (W > 1) {
@@ -341,18 +388,16 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
 
         float c = __builtin_fmaf(ea, cin, eb);
         float dx[E], dg[E];
-        if constexpr (!PLAIN) Elem<T>::unpack(cur.x, dg);  // dg[] starts as x_t
 #pragma unroll
         for (int i = E - 1; i >= 0; --i) {
             const float delta = G[i] + c;
             c = __builtin_fmaf(g[i], c, p[i]);
-            const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
             if constexpr (PLAIN) {
                 dx[i] = delta;
-                dg[i] = hp * delta;
+                dg[i] = hp[i] * delta;
             } else {
                 dx[i] = __builtin_fmaf(-g[i], delta, delta);
-                dg[i] = (hp - dg[i]) * delta;
+                dg[i] = (hp[i] - x[i]) * delta;
             }
         }
         if constexpr (decltype(whole)::value) {
