@@ -29,6 +29,10 @@ What each function follows in the reference:
                        differences and against autograd through the same PyTorch
                        operations the reference lines name (tests/test_oracle.py).
 * `memory_forward`     fm/scan/fm_scan.py:115-133, the whole layer.
+* `memory_backward`    the gradients of the whole layer (left to autograd by the reference):
+                       the chain rule through :116-119,130 on top of `readout_backward` and
+                       `backward`; pinned against autograd through the operations those lines
+                       name and against finite differences (tests/test_oracle.py).
 
 How it is pinned (tests/test_oracle.py): exact rational arithmetic on small
 inputs with forward-mode derivatives (tests/golden/), closed forms (constant
@@ -46,7 +50,7 @@ from __future__ import annotations
 import numpy as np
 
 __all__ = ["forward", "backward_per_row", "backward", "to_f64", "readout_forward", "readout_backward",
-           "memory_forward"]
+           "memory_forward", "memory_backward"]
 
 
 def to_f64(a):
@@ -193,13 +197,59 @@ def readout_backward(out_grad, ext_grad, read, states, mem_norm=True, eps=1e-6):
     return inv_rms[:, :, None, :] * (dn - normed * inner), read_grad
 
 
-def memory_forward(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True, eps=1e-6):
+def _layer_operands(alpha, update_scale, output_scale, inputs, storage):
+    """gates (B, M, L), tokens (B, D, L), read (B, M, L) as the layer hands them to the scan and
+    the read-out. `storage`, when given, rounds an array to the layer's storage dtype: the
+    reference materialises the gates and the read weights in that dtype before the scan sees
+    them (fm_scan.py:116-119,130 are PyTorch operations on bfloat16 tensors), and a gate near
+    one moves by up to 2^-9 when stored in bfloat16, which changes the decay it stands for.
+    A comparison with a storage-dtype implementation therefore starts from the stored gates."""
+    storage = storage or (lambda a: a)
+    write = np.ascontiguousarray(np.transpose(alpha * update_scale, (0, 2, 1)))        # :116,118
+    tokens = np.ascontiguousarray(np.transpose(inputs, (0, 2, 1)))                    # :117
+    gates = storage(1.0 - write)                                                       # :119
+    read = storage(np.ascontiguousarray(np.transpose(alpha * output_scale, (0, 2, 1))))  # :130
+    return gates, tokens, read
+
+
+def memory_forward(alpha, update_scale, output_scale, inputs, initial_state=None, mem_norm=True, eps=1e-6,
+                   storage=None):
     """fm_memory (fm_scan.py:102-133): alpha (B, L, M), scales (B, L, 1), inputs (B, L, D)
-    -> (output (B, L, D), memory states (B, M, D, L))."""
+    -> (output (B, L, D), memory states (B, M, D, L)). `storage`: see _layer_operands."""
     alpha, update_scale, output_scale, inputs = (to_f64(a) for a in (alpha, update_scale, output_scale, inputs))
-    write = np.ascontiguousarray(np.transpose(alpha * update_scale, (0, 2, 1)))  # :116,118
-    tokens = np.ascontiguousarray(np.transpose(inputs, (0, 2, 1)))              # :117
-    states = forward(1.0 - write, tokens, initial_state)                         # :119,121
-    read = np.ascontiguousarray(np.transpose(alpha * output_scale, (0, 2, 1)))   # :130
+    gates, tokens, read = _layer_operands(alpha, update_scale, output_scale, inputs, storage)
+    states = forward(gates, tokens, initial_state)                                     # :121
     output, states, _ = readout_forward(states, read, mem_norm, eps)
     return np.ascontiguousarray(np.transpose(output, (0, 2, 1))), states
+
+
+def memory_backward(alpha, update_scale, output_scale, inputs, out_grad, mem_grad=None, initial_state=None,
+                    mem_norm=True, eps=1e-6, storage=None):
+    """Gradients of sum(out_grad * output) + sum(mem_grad * memory_states) for memory_forward.
+
+    out_grad (B, L, D) or None, mem_grad (B, M, D, L) or None. Returns a dict with d_alpha (B, L, M),
+    d_update_scale (B, L, 1), d_output_scale (B, L, 1), d_inputs (B, L, D), d_initial_state (B, M, D).
+    `storage` (see _layer_operands) rounds the gates and read weights the gradients are taken at; the
+    rounding itself passes gradients through unchanged, as autograd does for a cast.
+    """
+    alpha, update_scale, output_scale, inputs = (to_f64(a) for a in (alpha, update_scale, output_scale, inputs))
+    B, L, M = alpha.shape
+    D = inputs.shape[2]
+    gates, tokens, read = _layer_operands(alpha, update_scale, output_scale, inputs, storage)
+    states = forward(gates, tokens, initial_state)
+    og = np.zeros((B, D, L)) if out_grad is None else np.ascontiguousarray(np.transpose(to_f64(out_grad), (0, 2, 1)))
+    ext = None if mem_grad is None else to_f64(mem_grad)
+    if mem_norm:
+        d_states, d_read = readout_backward(og, ext, read, states, True, eps)
+    else:  # the states are returned as they are: mem_grad reaches them unchanged
+        d_states, d_read = readout_backward(og, None, read, states, False, eps)
+        if ext is not None:
+            d_states = d_states + ext
+    d_gates, d_tokens, d_h0 = backward(gates, tokens, d_states, initial_state, states=states)
+    dg = np.transpose(d_gates, (0, 2, 1))   # (B, L, M): gates = 1 - alpha * update_scale
+    dr = np.transpose(d_read, (0, 2, 1))    # (B, L, M): read = alpha * output_scale
+    return {"d_alpha": dr * output_scale - dg * update_scale,
+            "d_update_scale": -(dg * alpha).sum(axis=2, keepdims=True),
+            "d_output_scale": (dr * alpha).sum(axis=2, keepdims=True),
+            "d_inputs": np.ascontiguousarray(np.transpose(d_tokens, (0, 2, 1))),
+            "d_initial_state": d_h0}

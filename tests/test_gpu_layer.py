@@ -1,0 +1,197 @@
+"""Parity of the Factorization-Memory layer around the scan (fm_memory, fm_layer: scan, RMS norm
+over D, read-out over M, and every gradient) with the float64 CPU oracle of the same layer
+(reference fm/scan/fm_scan.py:102-133, gradients by the chain rule), on an MI355X.
+
+Both sides start from the same, already quantised inputs, and the oracle takes the gates
+1 - alpha * update_scale and the read weights alpha * output_scale rounded to the storage dtype,
+as the layer (the reference's as well as this one) hands them to the scan: stored in bfloat16 a
+gate near one moves by up to 2^-9, which is a different decay and not an error of the scan.
+Errors are normwise,
+    max|y - ref| / max|ref|   and   ||y - ref||_2 / ||ref||_2,
+per returned quantity. Tolerances, with what they pay for:
+
+  float32            1e-5 for every quantity (the benchmark's bar); measured below 1e-6.
+  bfloat16/float16   1e-2 for every quantity (the benchmark's bar). The results of the forward
+                     pass are one to three roundings of the storage type away from float32
+                     arithmetic (states -> normalised states -> output); the gradients are made
+                     from the stored normalised states, pass through the cancellation
+                     dn - n * mean(dn * n) of the norm's gradient and through
+                     (h[t-1] - x[t]) * delta of the scan's, and are rounded once on store.
+                     Measured: up to 7e-3 in bfloat16, 1e-3 in float16. Values are printed.
+
+The shapes take every branch of the layer's backward: both sums inside one kernel (M > 1, D > 1,
+16-byte rows), M = 1, D = 1, D not a multiple of the 8 rows a block sums over, rows that are not
+16-byte multiples (element access), rows shorter than a tile, a loss on the output alone and on
+both results, with and without an initial state. D = 1 with the norm is run with eps of the order
+of the squared states: for eps << h^2 that gradient is pure cancellation and no implementation
+that stores the normalised states can deliver it (tests/test_oracle.py::
+test_norm_gradient_with_one_channel_is_all_cancellation).
+"""
+import numpy as np
+import pytest
+import torch
+
+import fm_scan_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+FWD_TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+GRAD_TOL = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 1e-2}
+
+
+@pytest.fixture(scope="module")
+def scan():
+    import fm.scan.fm_scan as m
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return m
+
+
+def storage(dtype):
+    """Rounds a float64 array to `dtype` and back."""
+    return lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dtype).to(torch.float64).numpy()
+
+
+def errs(y, ref):
+    y = y.detach().double().cpu().numpy().reshape(ref.shape)
+    d = y - ref
+    return (float(np.abs(d).max() / max(np.abs(ref).max(), 1e-300)),
+            float(np.linalg.norm(d.ravel()) / max(np.linalg.norm(ref.ravel()), 1e-300)))
+
+
+def check_all(tag, got, want, tols):
+    worst = []
+    for name in want:
+        e_max, e_l2 = errs(got[name], want[name])
+        print(f"{tag} {name}: max-norm {e_max:.2e} l2 {e_l2:.2e} (tolerance {tols[name]:g})", flush=True)
+        if not (e_max <= tols[name] and e_l2 <= tols[name]):
+            worst.append(f"{name}: max-norm {e_max:.3e}, l2 {e_l2:.3e} > {tols[name]:g}")
+    assert not worst, f"{tag}: " + "; ".join(worst)
+
+
+# (B, L, M, D), norm eps, what the shape is there for
+LAYER_SHAPES = [
+    ((2, 512, 4, 24), 1e-4, "both sums inside one kernel"),
+    ((2, 304, 1, 16), 1e-4, "M = 1"),
+    ((1, 7, 5, 1), 1.0, "D = 1, row shorter than 16 bytes"),
+    ((2, 264, 3, 5), 1e-4, "D below the 8 rows of a block"),
+    ((1, 1001, 3, 12), 1e-4, "rows that are not 16-byte multiples"),
+    ((3, 40, 2, 9), 1e-4, "row shorter than a tile, ragged D"),
+    ((1, 2048, 2, 130), 1e-4, "D beyond one block of the read-out"),
+]
+
+
+def layer_inputs(shape, dtype, with_h0, seed):
+    B, L, M, D = shape
+    gen = torch.Generator().manual_seed(seed)
+    q = lambda t: t.to(dtype).to(torch.float64)  # both sides start from the same quantised values
+    alpha = q(torch.softmax(torch.randn(B, L, M, generator=gen, dtype=torch.float64), dim=-1))
+    us = q(torch.rand(B, L, 1, generator=gen, dtype=torch.float64))
+    osc = q(torch.rand(B, L, 1, generator=gen, dtype=torch.float64) + 0.5)
+    inp = q(torch.randn(B, L, D, generator=gen, dtype=torch.float64))
+    h0 = q(torch.randn(B, M, D, generator=gen, dtype=torch.float64)) if with_h0 else None
+    w_out = q(torch.randn(B, L, D, generator=gen, dtype=torch.float64))
+    w_mem = q(torch.randn(B, M, D, L, generator=gen, dtype=torch.float64) * 0.1)
+    return alpha, us, osc, inp, h0, w_out, w_mem
+
+
+@pytest.mark.parametrize("mem_in_loss", [False, True])
+@pytest.mark.parametrize("mem_norm", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_fm_memory_against_the_oracle(scan, dtype, mem_norm, mem_in_loss):
+    for i, (shape, eps, why) in enumerate(LAYER_SHAPES):
+        B, L, M, D = shape
+        with_h0 = i % 2 == 0
+        alpha, us, osc, inp, h0, w_out, w_mem = layer_inputs(shape, dtype, with_h0, seed=100 + i)
+        leaves = [t.to(dtype).to(DEV).requires_grad_() for t in (alpha, us, osc, inp)]
+        h0_gpu = None if h0 is None else h0.to(dtype).to(DEV).requires_grad_()
+        y, mem = scan.fm_memory(*leaves, h0_gpu, mem_norm=mem_norm, norm_eps=eps)
+        assert y.shape == (B, L, D) and mem.shape == (B, M, D, L) and y.is_contiguous()
+        # a linear loss: its gradients with respect to the two results are w_out and w_mem exactly
+        loss = (y.float() * w_out.to(DEV).float()).sum()
+        if mem_in_loss:
+            loss = loss + (mem.float() * w_mem.to(DEV).float()).sum()
+        loss.backward()
+        o_y, o_mem = O.memory_forward(alpha, us, osc, inp, h0, mem_norm, eps, storage(dtype))
+        want = O.memory_backward(alpha, us, osc, inp, w_out, w_mem if mem_in_loss else None, h0, mem_norm, eps,
+                                 storage(dtype))
+        got = {"output": y, "memory_states": mem, "d_alpha": leaves[0].grad, "d_update_scale": leaves[1].grad,
+               "d_output_scale": leaves[2].grad, "d_inputs": leaves[3].grad}
+        want = dict(output=o_y, memory_states=o_mem, **want)
+        if h0 is None:
+            del want["d_initial_state"]
+        else:
+            got["d_initial_state"] = h0_gpu.grad
+        tols = {k: (FWD_TOL if k in ("output", "memory_states") else GRAD_TOL)[dtype] for k in want}
+        check_all(f"fm_memory {shape} ({why}) {dtype} norm={mem_norm} mem_in_loss={mem_in_loss} h0={with_h0}",
+                  got, want, tols)
+
+
+@pytest.mark.parametrize("mem_in_loss", [False, True])
+@pytest.mark.parametrize("mem_norm", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_fm_layer_against_the_oracle(scan, dtype, mem_norm, mem_in_loss):
+    """fm_layer: the same layer with time last (gates, read (B, M, L), tokens (B, D, L))."""
+    for i, (shape, eps, why) in enumerate(LAYER_SHAPES):
+        B, L, M, D = shape
+        gen = torch.Generator().manual_seed(200 + i)
+        q = lambda t: t.to(dtype).to(torch.float64)
+        g = q(torch.sigmoid(torch.randn(B, M, L, generator=gen, dtype=torch.float64) + 2))
+        x = q(torch.randn(B, D, L, generator=gen, dtype=torch.float64))
+        read = q(torch.randn(B, M, L, generator=gen, dtype=torch.float64))
+        h0 = q(torch.randn(B, M, D, generator=gen, dtype=torch.float64)) if i % 2 else None
+        w_out = q(torch.randn(B, D, L, generator=gen, dtype=torch.float64))
+        w_mem = q(torch.randn(B, M, D, L, generator=gen, dtype=torch.float64) * 0.1)
+        leaves = [t.to(dtype).to(DEV).requires_grad_() for t in (g, x, read)]
+        h0_gpu = None if h0 is None else h0.to(dtype).to(DEV).requires_grad_()
+        y, mem = scan.fm_layer(leaves[0], leaves[1], h0_gpu, leaves[2], mem_norm, eps)
+        loss = (y.float() * w_out.to(DEV).float()).sum()
+        if mem_in_loss:
+            loss = loss + (mem.float() * w_mem.to(DEV).float()).sum()
+        loss.backward()
+        states = O.forward(g, x, h0)
+        o_y, o_mem, _ = O.readout_forward(states, read, mem_norm, eps)
+        ext = w_mem.numpy() if mem_in_loss else None
+        if mem_norm:
+            d_states, d_read = O.readout_backward(w_out, ext, read, states, True, eps)
+        else:
+            d_states, d_read = O.readout_backward(w_out, None, read, states, False, eps)
+            if ext is not None:
+                d_states = d_states + ext
+        d_g, d_x, d_h0 = O.backward(g, x, d_states, h0, states=states)
+        got = {"output": y, "memory_states": mem, "d_gates": leaves[0].grad, "d_tokens": leaves[1].grad,
+               "d_read": leaves[2].grad}
+        want = {"output": o_y, "memory_states": o_mem, "d_gates": d_g, "d_tokens": d_x, "d_read": d_read}
+        if h0 is not None:
+            got["d_initial_state"], want["d_initial_state"] = h0_gpu.grad, d_h0
+        tols = {k: (FWD_TOL if k in ("output", "memory_states") else GRAD_TOL)[dtype] for k in want}
+        check_all(f"fm_layer {shape} ({why}) {dtype} norm={mem_norm} mem_in_loss={mem_in_loss}", got, want, tols)
+
+
+def test_layer_at_the_benchmark_shape(scan):
+    """fm_memory at the shape bench.py --workload layer times, (B, L, M, D) = (32, 2048, 32, 128)
+    bfloat16 with the norm and a loss on the output: forward results and all four input gradients
+    against the float64 oracle on batch elements 0 and B - 1 (the batch elements are independent)."""
+    B, L, M, D, dt = 32, 2048, 32, 128, torch.bfloat16
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    alpha = torch.softmax(rn(B, L, M), -1).to(dt).requires_grad_()
+    us = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt).requires_grad_()
+    osc = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt).requires_grad_()
+    inp = rn(B, L, D).to(dt).requires_grad_()
+    w_out = rn(B, L, D).to(dt)
+    y, mem = scan.fm_memory(alpha, us, osc, inp)
+    (y.float() * w_out.float()).sum().backward()
+    torch.cuda.synchronize()
+    for b in (0, B - 1):
+        sel = lambda t: t.detach()[b:b + 1].double().cpu()
+        a, u, o, x, w = (sel(t) for t in (alpha, us, osc, inp, w_out))
+        o_y, o_mem = O.memory_forward(a, u, o, x, None, True, 1e-6, storage(dt))
+        want = O.memory_backward(a, u, o, x, w, None, None, True, 1e-6, storage(dt))
+        del want["d_initial_state"]
+        want = dict(output=o_y, memory_states=o_mem, **want)
+        got = {"output": y[b:b + 1], "memory_states": mem[b:b + 1], "d_alpha": alpha.grad[b:b + 1],
+               "d_update_scale": us.grad[b:b + 1], "d_output_scale": osc.grad[b:b + 1], "d_inputs": inp.grad[b:b + 1]}
+        tols = {k: (FWD_TOL if k in ("output", "memory_states") else GRAD_TOL)[dt] for k in want}
+        check_all(f"fm_memory bench shape, batch element {b}", got, want, tols)

@@ -295,6 +295,8 @@ def test_segment_chaining(scan):
     delta_k = dx2[..., 0] / (1 - g[:, :, k].view(rows, 1, 1))
     cross = (g[:, :, k].view(rows, 1, 1) * delta_k).contiguous()
     _, dx1, dg1 = run_fwd_bwd(scan, cut(g, 0, k), cut(x, 0, k), cut(G, 0, k), fpg=cross)
+    # 1e-4: the gradient that crosses the cut was rebuilt above by a division by 1 - g >= 0.01, which
+    # magnifies the float32 rounding of dx2 a hundredfold before it enters the first part
     check("chained token grad", torch.cat([dx1, dx2], dim=3), dx.double().cpu().numpy(), 1e-4)
     check("chained gate grad", torch.cat([dg1, dg2], dim=3), dg.double().cpu().numpy(), 1e-4)
 
@@ -378,7 +380,8 @@ def test_backward_with_sums_inside(scan, dtype, plain):
         check(tag + " d_gates", d_g, gg.sum(axis=2), TOL[dtype])
         check(tag + " d_tokens", d_x, tg.sum(axis=1), TOL[dtype])
         check(tag + " d_initial_state", dh0, O.to_f64(g)[:, :, 0][:, :, None] * delta[..., 0], TOL[dtype])
-        # the reference's route: two full tensors, then torch.sum
+        # the reference's route: two full tensors, then torch.sum (2 * TOL: two rounded results
+        # against each other, each within TOL of the exact one)
         dx, dg = torch.empty_like(out), torch.empty_like(out)
         scan.fm_scan_backward(g, G, fpg, dx, out, x, dg, initial_state=h0, plain=plain)
         check(tag + " vs two-tensor route (gates)", d_g, dg.sum(dim=2).double().cpu().numpy(), 2 * TOL[dtype])
@@ -418,6 +421,8 @@ def test_notebook_design(scan):
         states = fn(g, x)
         states.sum().backward()
         res[name] = (states.detach().float().clone(), x.grad.float().clone(), g.grad.float().clone())
+    # 2e-2 where bfloat16 is involved: as in the notebook the inputs themselves differ there (the same
+    # rand() values rounded to bfloat16 on one side, kept in float32 on the other)
     for a, b, tol in (("fp32", "loop", 1e-5), ("bf16", "loop", 2e-2), ("bf16", "fp32", 2e-2)):
         for ta, tb, what in zip(res[a], res[b], ("states", "token grad", "gate grad")):
             scale = tb.abs().max().item()
@@ -502,8 +507,8 @@ def test_readout_kernels(scan, dtype, mem_norm):
         states_n = normed if mem_norm else states
         d_states, d_read = scan.fm_readout_backward(out_grad, ext, read, states_n, inv_rms)
         o_ds, o_dr = O.readout_backward(out_grad, ext, read, states, mem_norm, eps)
-        check(tag + " d_states", d_states, o_ds, 2 * TOL[dtype])
-        check(tag + " d_read", d_read, o_dr, 2 * TOL[dtype])
+        check(tag + " d_states", d_states, o_ds, TOL[dtype])
+        check(tag + " d_read", d_read, o_dr, TOL[dtype])
 
 
 def test_readout_in_place_and_determinism(scan):
@@ -552,11 +557,12 @@ def test_layer_backward_kernel_equals_the_two_step_route(scan, dtype, mem_norm):
         assert torch.equal(out_b, out)
         out_b.backward(og)
         tag = f"{(B, M, D, L)} {dtype} norm={mem_norm}"
-        tol = 4 * TOL[dtype]
+        tol = 2 * TOL[dtype]  # two rounded results against each other, each within TOL of the exact one
         check(tag + " d_gates vs two steps", leaves[0].grad, dg_a.double().cpu().numpy(), tol)
         check(tag + " d_tokens vs two steps", leaves[1].grad, dx_a.double().cpu().numpy(), tol)
         check(tag + " d_initial_state vs two steps", leaves[2].grad, dh0_a.double().cpu().numpy(), tol)
         check(tag + " d_read vs two steps", leaves[3].grad, d_read.double().cpu().numpy(), tol)
+        tol = TOL[dtype]
         # oracle: read-out gradient, then the scan's
         o_sg, o_dr = O.readout_backward(og, None, read, states, mem_norm, 1e-5)
         tg, gg, delta = O.backward_per_row(g, o_sg, states, x, None, h0, False)
@@ -618,7 +624,7 @@ def test_scan_then_readout_equals_the_one_node_layer(scan):
         grads.append([out.detach(), mem.detach(), g.grad, x.grad, h.grad, r.grad])
     assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
     for a, b, name in zip(grads[0][2:], grads[1][2:], ("d_gates", "d_tokens", "d_initial_state", "d_read")):
-        check(name, b, a.double().cpu().numpy(), 2e-2)
+        check(name, b, a.double().cpu().numpy(), 2e-2)  # two bfloat16 results against each other
 
 
 def test_layer_keeps_no_second_copy_of_the_states(scan):
@@ -650,53 +656,6 @@ def test_swap_last_two_is_exact(scan):
                       ((2, 300, 258), torch.bfloat16)]:
         t = torch.randn(*shape, device=DEV).to(dt)
         assert torch.equal(_swap_last_two(t), t.transpose(1, 2).contiguous()), (shape, dt)
-
-
-@pytest.mark.parametrize("mem_in_loss", [True, False])
-@pytest.mark.parametrize("dtype,mem_norm", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, True)])
-def test_fm_memory_layer(scan, dtype, mem_norm, mem_in_loss):
-    """The layer on top of the scan, forward and backward, against the float64 oracle layer /
-    the same layer written with the PyTorch operations the reference names, in float64 on the
-    CPU. With the returned memory states in the loss the states' gradient is a tensor between
-    the read-out's and the scan's backward kernels; with the output alone it is made inside
-    the scan's backward kernel."""
-    from fm.scan.fm_pytorch import fm_scan_pytorch
-
-    B, L, M, D = 2, 512, 4, 24
-    gen = torch.Generator().manual_seed(13)
-    mk = lambda *s: torch.randn(*s, generator=gen, dtype=torch.float64)
-    q = lambda t: t.to(dtype).to(torch.float64)  # both sides start from the same quantised values
-    alpha64 = q(torch.softmax(mk(B, L, M), dim=-1))
-    us64, os64, inp64 = q(torch.rand(B, L, 1, generator=gen, dtype=torch.float64)), \
-        q(torch.rand(B, L, 1, generator=gen, dtype=torch.float64)), q(mk(B, L, D))
-    h064 = q(mk(B, M, D))
-    w_mem = q(mk(B, M, D, L)) * 0.1
-    outs = {}
-    for name, dt, dev in (("gpu", dtype, DEV), ("ref", torch.float64, "cpu")):
-        a, u, o, i, h0 = (t.to(dt).to(dev).requires_grad_() for t in (alpha64, us64, os64, inp64, h064))
-        if name == "gpu":
-            y, mem = scan.fm_memory(a, u, o, i, h0, mem_norm=mem_norm, norm_eps=1e-4)
-            assert y.shape == (B, L, D) and mem.shape == (B, M, D, L) and y.is_contiguous()
-        else:
-            tok = i.transpose(1, 2).contiguous()
-            gate = 1.0 - (a * u).transpose(1, 2).contiguous()
-            mem = fm_scan_pytorch(gate, tok, h0)
-            if mem_norm:
-                mem = mem * torch.rsqrt((mem ** 2).mean(dim=2, keepdim=True) + 1e-4)
-            y = torch.einsum("blm,bmdl->bld", a * o, mem)
-            o_y, o_mem = O.memory_forward(alpha64, us64, os64, inp64, h064, mem_norm, 1e-4)
-            np.testing.assert_allclose(y.detach().numpy(), o_y, rtol=1e-10, atol=1e-10)
-            np.testing.assert_allclose(mem.detach().numpy(), o_mem, rtol=1e-10, atol=1e-10)
-        acc = torch.float64 if name == "ref" else torch.float32
-        loss = y.to(acc).square().sum()
-        if mem_in_loss:
-            loss = loss + (mem.to(acc) * w_mem.to(dev).to(acc)).sum()
-        loss.backward()
-        outs[name] = [y.detach(), mem.detach(), a.grad, u.grad, o.grad, i.grad, h0.grad]
-    tol = 1e-4 if dtype == torch.float32 else 3e-2
-    for t_gpu, t_ref, what in zip(outs["gpu"], outs["ref"], ("output", "memory", "d_alpha", "d_update_scale",
-                                                            "d_output_scale", "d_inputs", "d_initial_state")):
-        check(what, t_gpu, t_ref.numpy(), tol)
 
 
 def test_kernels_follow_the_current_stream(scan):

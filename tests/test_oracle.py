@@ -320,6 +320,80 @@ def test_memory_layer_agrees_with_the_operations_the_reference_names(mem_norm):
     np.testing.assert_allclose(t["osc"].grad.numpy(), d_osc, rtol=1e-11, atol=1e-12)
 
 
+@pytest.mark.parametrize("mem_norm", [True, False])
+@pytest.mark.parametrize("loss_on", ["output", "memory", "both"])
+def test_memory_backward_against_autograd_and_finite_differences(mem_norm, loss_on):
+    """The oracle's gradients of the whole layer against (i) autograd through the PyTorch operations
+    fm_scan.py:115-133 names, in float64, and (ii) central finite differences of the oracle's own
+    forward: every input, with a non-zero initial state, for a loss on either result or both."""
+    from fm_amd.scan.fm_pytorch import fm_scan_pytorch
+
+    rng = np.random.default_rng(31)
+    B, L, M, D = 2, 7, 3, 4
+    alpha = rng.random((B, L, M))
+    us, osc = rng.random((B, L, 1)), rng.standard_normal((B, L, 1))
+    x, h0 = rng.standard_normal((B, L, D)), rng.standard_normal((B, M, D))
+    w_out = rng.standard_normal((B, L, D)) if loss_on != "memory" else None
+    w_mem = rng.standard_normal((B, M, D, L)) if loss_on != "output" else None
+    eps = 1e-2
+    got = O.memory_backward(alpha, us, osc, x, w_out, w_mem, h0, mem_norm, eps)
+
+    t = [torch.tensor(v, requires_grad=True) for v in (alpha, us, osc, x, h0)]
+    write = (t[0] * t[1]).transpose(1, 2).contiguous()
+    states = fm_scan_pytorch(1.0 - write, t[3].transpose(1, 2).contiguous(), t[4])
+    if mem_norm:
+        states = states * torch.rsqrt(torch.mean(states ** 2, dim=2, keepdim=True) + eps)
+    out = torch.einsum("blm,bmdl->bld", t[0] * t[2], states)
+    loss = 0.0
+    if w_out is not None:
+        loss = loss + (out * torch.tensor(w_out)).sum()
+    if w_mem is not None:
+        loss = loss + (states * torch.tensor(w_mem)).sum()
+    loss.backward()
+    names = ("d_alpha", "d_update_scale", "d_output_scale", "d_inputs", "d_initial_state")
+    for name, leaf in zip(names, t):
+        want = np.zeros(leaf.shape) if leaf.grad is None else leaf.grad.numpy()  # output_scale without the output
+        np.testing.assert_allclose(got[name], want, rtol=1e-10, atol=1e-11, err_msg=name)
+
+    def f():
+        o, m = O.memory_forward(alpha, us, osc, x, h0, mem_norm, eps)
+        return float((0.0 if w_out is None else (o * w_out).sum()) + (0.0 if w_mem is None else (m * w_mem).sum()))
+
+    for name, arr in zip(names, (alpha, us, osc, x, h0)):
+        np.testing.assert_allclose(got[name], fd_grad(f, arr), rtol=2e-6, atol=1e-7, err_msg=name)
+
+
+def test_norm_gradient_with_one_channel_is_all_cancellation():
+    """D = 1: the norm maps a state to n = h / sqrt(h^2 + eps), close to its sign, and the
+    gradient that comes back through it is r * dn * (1 - n^2) = r * dn * eps / (h^2 + eps): what
+    is left of dn after a cancellation to one part in (h^2 + eps) / eps. Made from normalised
+    states that were stored in bfloat16 (spacing 2^-8 below one) or float32 (2^-24), the factor
+    1 - n^2 is rounding noise unless eps is of the order of h^2: an implementation that keeps the
+    normalised states (this one does; the reference's autograd keeps the bfloat16 factors of the
+    same product) cannot do better there. With D >= 2 the part of dn across n survives and the
+    same rounding is harmless."""
+    rng = np.random.default_rng(5)
+    B, M, L = 1, 5, 64
+    read, out_grad = rng.standard_normal((B, M, L)), None
+
+    def grad_from_stored(states, eps, quantum):
+        D = states.shape[2]
+        og = rng.standard_normal((B, D, L))
+        exact, _ = O.readout_backward(og, None, read, states, True, eps)
+        _, n, r = O.readout_forward(states, read, True, eps)
+        n_stored = np.round(n / quantum) * quantum            # the stored, rounded normalised states
+        dn = read[:, :, None, :] * og[:, None, :, :]
+        approx = r[:, :, None, :] * (dn - n_stored * np.mean(dn * n_stored, axis=2, keepdims=True))
+        return np.abs(approx - exact).max() / np.abs(exact).max()
+
+    h1 = rng.standard_normal((B, M, 1, L)) + 3.0 * np.sign(rng.standard_normal((B, M, 1, L)))
+    assert grad_from_stored(h1, 1e-6, 2.0 ** -8) > 0.5       # bfloat16, eps << h^2: n rounds to +-1, nothing is left
+    assert grad_from_stored(h1, 1e-6, 2.0 ** -24) > 1e-3     # float32 too, against a 1e-5 bar
+    assert grad_from_stored(h1, 16.0, 2.0 ** -8) < 1e-2      # eps of the order of h^2: fine
+    h4 = rng.standard_normal((B, M, 4, L))
+    assert grad_from_stored(h4, 1e-6, 2.0 ** -8) < 1e-2      # D = 4: fine with the same rounding
+
+
 # ------------------------------------------------------------------ compiled oracle and port
 
 @pytest.mark.parametrize("plain", [False, True])
