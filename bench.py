@@ -185,10 +185,10 @@ def run_layer(torch, args) -> int:
     lib, st = S.module, torch.cuda.current_stream().cuda_stream
     inv = torch.empty(B, M, L, device=dev)
     q = torch.empty_like(inv)
-    rms = torch.full_like(read, 1.5)  # 1 / inv_rms: takes the scanned states back from the normalised ones
+    rms = torch.full_like(inv, 1.5)  # 1 / inv_rms (float32): takes the scanned states back from the normalised ones
     normed, sg = torch.empty_like(states), torch.empty_like(states)
     out = torch.empty(B, D, L, dtype=dt, device=dev)
-    coef, dtok = rn(B, M, L).to(dt), torch.empty(B, D, L, dtype=dt, device=dev)
+    coef, dtok = rn(B, M, L), torch.empty(B, D, L, dtype=dt, device=dev)  # coefficient vectors are float32
     partial = torch.empty(B, M, lib.fmscan_reduced_groups(D), L, device=dev)
     code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
     P = lambda t: t.data_ptr()
@@ -206,7 +206,7 @@ def run_layer(torch, args) -> int:
         # the form that makes the states' gradient itself (no readout_backward_kernel, no G) and
         # takes the scanned states back from the normalised ones (reads one (B,M,D,L) tensor)
         "scan_backward_reduced_kernel (layer form)": (s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
-            P(gates), P(normed), P(read), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
+            P(gates), P(normed), P(coef), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
             None, None, B, M, D, L, code, 0, st)),
     }
     if args.probe:  # for rocprofv3 --pmc: a copy of known size, then every kernel a few times

@@ -51,8 +51,8 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
     const T* __restrict__ states /* (B, M, D, L) */, const T* __restrict__ out_grad /* (B, D, L) */,
     const T* __restrict__ ext_grad /* (B, M, D, L) */, float* __restrict__ result /* (B, M, L) */,
     float* __restrict__ result_ext /* (B, M, L) */, const float* __restrict__ inv_rms /* (B, M, L) */,
-    const T* __restrict__ read /* (B, M, L) */, T* __restrict__ coef_out, T* __restrict__ coef_self,
-    T* __restrict__ rms_out /* (B, M, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles, float eps) {
+    const T* __restrict__ read /* (B, M, L) */, float* __restrict__ coef_out, float* __restrict__ coef_self,
+    float* __restrict__ rms_out /* (B, M, L) */, int32_t M, int32_t D, int64_t L, int32_t tiles, float eps) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     __shared__ float part[EXT ? 2 : 1][WV][TILE];
@@ -108,11 +108,11 @@ __global__ __launch_bounds__(64 * WV) void rowdot_kernel(
             // coef_out * out_grad - coef_self * normalised state
             if (coef_out != nullptr) {
                 const float c = (inv_rms ? inv_rms[bm * L + t] : 1.0f) * (float)read[bm * L + t];
-                coef_out[bm * L + t] = (T)c;
-                coef_self[bm * L + t] = (T)(inv_rms ? c * s / (float)D : 0.0f);
+                coef_out[bm * L + t] = c;
+                coef_self[bm * L + t] = inv_rms ? c * s / (float)D : 0.0f;
             }
             // ... and what takes the scanned states back from the normalised ones
-            if (rms_out != nullptr) rms_out[bm * L + t] = (T)(1.0f / inv_rms[bm * L + t]);
+            if (rms_out != nullptr) rms_out[bm * L + t] = 1.0f / inv_rms[bm * L + t];
         }
     }
 }

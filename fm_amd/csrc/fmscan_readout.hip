@@ -108,7 +108,7 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
 }
 
 int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad, float* q, float* qe,
-                       const float* inv_rms, const void* read, void* coef_out, void* coef_self, void* rms_out,
+                       const float* inv_rms, const void* read, float* coef_out, float* coef_self, float* rms_out,
                        int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream) {
     ReadoutShape rs;
     if (int rc = parse_readout("fmscan_readout_dot", B, M, D, L, dtype, &rs)) return rc;
@@ -120,8 +120,8 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
     if (rms_out && !inv_rms) return fail(FMSCAN_E_NULL, "fmscan_readout_dot: rms_out needs inv_rms");
     const int64_t full = B * M * D * L * rs.esize, slot = B * M * L;
     const Range outs[] = {{"q", q, slot * 4}, {"qe", ext_grad ? qe : nullptr, slot * 4},
-                          {"coef_out", coef_out, slot * rs.esize}, {"coef_self", coef_self, slot * rs.esize},
-                          {"rms_out", rms_out, slot * rs.esize}};
+                          {"coef_out", coef_out, slot * 4}, {"coef_self", coef_self, slot * 4},
+                          {"rms_out", rms_out, slot * 4}};
     const Range ins[] = {{"states_n", states_n, full}, {"out_grad", out_grad, B * D * L * rs.esize},
                          {"ext_grad", ext_grad, full}, {"inv_rms", (coef_out || rms_out) ? inv_rms : nullptr, slot * 4},
                          {"read", coef_out ? read : nullptr, slot * rs.esize}};
@@ -141,7 +141,7 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
                 fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kDot, decltype(et)::value, decltype(vt)::value>
                     <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>(
                         (const T*)states_n, (const T*)out_grad, (const T*)ext_grad, q, qe, inv_rms, (const T*)read,
-                        (T*)coef_out, (T*)coef_self, (T*)rms_out, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
+                        coef_out, coef_self, rms_out, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
             });
         });
     });

@@ -1,36 +1,120 @@
 // The backward scan of Factorization-Memory shapes (M > 1 and D > 1) with the sums over D
-// and M inside, and its forms for the layer around the scan. Building blocks (rows,
-// lanes, the wave scan): fmscan_kernels.h, fmscan_device.h.
+// and M inside, and its forms for the layer around the scan. Building blocks (lanes, the
+// wave scan): fmscan_kernels.h, fmscan_device.h.
 #pragma once
 
 #include "fmscan_kernels.h"
 
 namespace fmscan {
 
+// ---- wave scan with the gates' part done once ------------------------------------------
+// The J rows a wave visits for one memory slot m share their gates, hence the `a` halves of
+// all their step pairs and everything the wave scan does to them. scan_gates runs that half
+// once per slot and keeps what each of the six levels needs (the value of `a` before the
+// level); scan_values then scans the `b` half of a row with one instruction per level.
+struct GateLevels {
+    float before[6];  // a in this lane before level 1..6
+    float ea;         // product of the gates of all chunks before this lane's (1 in lane 0)
+    float ta;         // product over the whole tile
+};
+
+__device__ __forceinline__ GateLevels scan_gates(float a) {
+    GateLevels g;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mov_b32 %1, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %2, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %3, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %4, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %5, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %6, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "=&v"(g.before[0]), "=&v"(g.before[1]), "=&v"(g.before[2]), "=&v"(g.before[3]),
+          "=&v"(g.before[4]), "=&v"(g.before[5]));
+    g.ea = dpp<kWaveShr1>(1.0f, a);
+    g.ta = lane63(a);
+    return g;
+}
+
+__device__ __forceinline__ void scan_values(float& b, const GateLevels& g) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %1 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %2 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %3 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %4 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %5 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %6 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(b)
+        : "v"(g.before[0]), "v"(g.before[1]), "v"(g.before[2]), "v"(g.before[3]), "v"(g.before[4]),
+          "v"(g.before[5]));
+}
+
+// E consecutive floats at p (16-byte aligned)
+template <int E>
+struct FloatChunk {
+    float4 v[E / 4];
+};
+template <int E>
+__device__ __forceinline__ FloatChunk<E> load_float_chunk(const float* __restrict__ p) {
+    FloatChunk<E> c;
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) c.v[i] = reinterpret_cast<const float4*>(p)[i];
+    return c;
+}
+template <int E>
+__device__ __forceinline__ void spread(const FloatChunk<E>& c, float (&f)[E]) {
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) {
+        f[4 * i] = c.v[i].x; f[4 * i + 1] = c.v[i].y; f[4 * i + 2] = c.v[i].z; f[4 * i + 3] = c.v[i].w;
+    }
+}
+
 // ---- backward with the D and M sums inside -------------------------------------------
 // For M > 1 and D > 1 the per-pair gradients are only ever summed: d_gates = sum over d,
 // d_tokens = sum over m (reference fm/scan/fm_scan.py:76-78; its kernel writes both
 // (B, M, D, L) tensors "to avoid atomicAdd", fm_scan.cuh:200-207, and torch.sum reads them
-// back). This kernel never writes them. A block is one batch element b and DG
-// consecutive d (one wave each). Its waves walk their rows from the end in chunks of C
-// tiles; for a chunk they visit the M rows (b, m, d) one after the other and, in each, the
-// C tiles of the chunk from the last to the first, all waves on the same step:
-//   * token gradient: summed over m in registers (C tiles of accumulators), stored once
-//     per chunk as d_tokens[b, d, :]
-//   * gate gradient: the DG waves add their tiles up in LDS (one barrier per step) and
-//     store the sum for this group of d, gate_partial[b, m, group, :] in float32; the
-//     caller adds the ceil(D / DG) groups.
-// Each wave keeps the running state of its M rows in LDS (one float per row). The visits
-// (chunk, m) form one linear sequence; a ring holds the loads of the next R visits, and
-// every step issues the same loads whatever its position (addresses are clamped into
-// the row), so the number of loads in flight is known at compile time and a step waits
-// for its own entry only. A larger C makes the pieces a wave reads from one row longer
-// (C KiB at a time), which the memory likes, at C tiles of accumulators.
-// HBM traffic: G and h once (2s per element) plus 4/DG bytes per element of partials,
-// against 6s for the unfused kernel plus the two torch.sum passes. This kernel, unlike the two
-// above, does depend on per-entry waits: its 8 waves meet at a barrier every tile, so a wave
-// that waits for its newest loads stalls the block (measured: 0.75 -> 0.50 ms on the
-// (1, 32, 2048, 8192) shape when the waits became per entry).
+// back). This kernel never writes them.
+//
+// A block is one batch element b and J consecutive d; its NW waves split the M memory
+// slots between them (Mw consecutive slots each). A wave walks the tiles of the sequence
+// from the last to the first and, in each tile, its Mw x J rows (b, m, d): slot after slot,
+// and for a slot the J rows one after the other. So
+//   * what depends on the slot only (gates, the layer's coefficient vectors, the gate half
+//     of the wave scan) is prepared once per J rows;
+//   * the gate gradient of a slot, summed over the J rows, builds up in registers and is
+//     stored as float32 partial gate_partial[b, m, group, :]; the caller adds the
+//     ceil(D / J) groups;
+//   * the token gradients of the J rows, summed over the wave's slots, build up in
+//     registers over the whole tile; at its end the waves of the block hand them on from
+//     wave to wave through LDS (each adds its own; fixed order, hence deterministic) and the
+//     last stores d_tokens[b, d, tile].
+// No wave waits for another except in that hand-over, once per tile. The running state of
+// every row lives in LDS (one float per row, private to its wave). Loads run one slot
+// ahead: while the J rows of a slot are worked on, the J tiles of the next slot (or of the
+// first slot of the tile before) are in flight, as are its per-slot vectors; every step
+// issues the same loads whatever its position (addresses are clamped into the tensors), so
+// the count of loads in flight is a compile-time number.
+// HBM traffic per element of (B, M, D, L): G and h (2s), or the normalised states alone in
+// the layer form (s), plus 4/J bytes of partials, against 6s for the unfused kernel plus the
+// two torch.sum passes.
 //
 // LAYER: the gradient that arrives at the states is not read but made on the spot from what
 // the layer around the scan holds (reference fm/scan/fm_scan.py:124-131 differentiated):
@@ -39,275 +123,330 @@ namespace fmscan {
 // never written or read. LAYER == 2: the scanned states themselves are not read either
 // (h_saved is NULL) but taken back from the normalised ones, h = out_grad * rms, so that
 // the layer has to keep nothing of size (B, M, D, L) besides the states it returns.
-template <typename T, int DG, int C, int R, bool PLAIN, int LAYER>
-__global__ __launch_bounds__(64 * DG) void scan_backward_reduced_kernel(
+// coef_out, coef_self and rms are float32.
+template <typename T, int J, int NW, bool PLAIN, int LAYER>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) void scan_backward_reduced_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved,
     const T* __restrict__ tokens, float* __restrict__ gate_partial /* (B, M, NG, L) */,
-    const T* __restrict__ h0, T* __restrict__ h0_grad, const T* __restrict__ coef_out /* (B, M, L) */,
-    const T* __restrict__ coef_self /* (B, M, L) */, const T* __restrict__ layer_out_grad /* (B, D, L) */,
-    const T* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L) {
+    const T* __restrict__ h0, T* __restrict__ h0_grad, const float* __restrict__ coef_out /* (B, M, L) */,
+    const float* __restrict__ coef_self /* (B, M, L) */, const T* __restrict__ layer_out_grad /* (B, D, L) */,
+    const float* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L, int32_t Mw) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
-    constexpr int SLICE = TILE / DG;  // elements of a summed tile each wave adds up and stores
-    constexpr bool HOIST = C <= 2;    // keep the chunk's tokens widened across its M rows
-    static_assert(TILE % DG == 0, "a tile must split evenly over the waves");
     extern __shared__ float lds[];
-    float* red = lds;                            // [2][DG][TILE]
-    float* carries = lds + 2 * DG * TILE;        // [DG][M]
+    static_assert(J % NW == 0, "the waves share the loads of the J token rows evenly");
+    float* handover = lds;                    // [2][J][E / 4][64][4]: token gradients on their way down the waves
+    u32x4* shared_xy = reinterpret_cast<u32x4*>(lds + 2 * J * TILE);  // [2][J][2][64]: tokens and layer_out_grad of a tile
+    float* carries = lds + 2 * J * TILE + 2 * J * 2 * 64 * 4;         // [NW][Mw * J]
 
     const int lane = threadIdx.x & 63;
     const int w = uniform((int)(threadIdx.x >> 6));
-    const int32_t NG = (D + DG - 1) / DG;
-    // (the division runs on the vector unit; everything derived from b is an address, so
-    // bring it back to a scalar register)
+    const int32_t NG = (D + J - 1) / J;
     // Blocks go to the 8 XCDs (each with its own L2) round robin. The blocks of one b read the
-    // same gates (and coefficient vectors), so they are renumbered to share an XCD: XCD x takes
-    // the x-th eighth of the (b, group) pairs.
+    // same gates, tokens and coefficient vectors, so they are renumbered to share an XCD: XCD x
+    // takes the x-th eighth of the (b, group) pairs.
     uint32_t id = blockIdx.x;
     if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
-    const int32_t b32 = uniform((int)(id / (uint32_t)NG));
-    const int64_t b = b32;
-    const int32_t grp = uniform((int)id - b32 * NG);
-    const bool active = grp * DG + w < D;        // a wave past the last d still joins every barrier
-    const int64_t d = active ? grp * DG + w : D - 1;
+    const int64_t b = uniform((int)(id / (uint32_t)NG));
+    const int32_t grp = uniform((int)id - (int32_t)b * NG);
+    const int32_t d0 = grp * J;
+    const int32_t m0 = w * Mw;
+    const int32_t mcount = uniform(M - m0 < 0 ? 0 : (M - m0 < Mw ? M - m0 : Mw));  // slots of this wave
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
-    const int32_t nchunks = (ntiles + C - 1) / C;
-    const int64_t lane_off = (int64_t)(63 - lane) * E;
-    float* mycarry = carries + w * M;
+    const int32_t lane_off = (63 - lane) * E;  // lane l owns the chunk l chunks before the end of the tile
+    float* mycarry = carries + w * Mw * J;
 
-    for (int32_t m = lane; m < M; m += 64)
-        mycarry[m] = first_prop_grad ? Elem<T>::widen(first_prop_grad[(b * M + m) * D + d]) : 0.0f;
+    // (the trip count is the same for all lanes and only the access is predicated: a loop that
+    // some lanes skip would leave the values it shares with the code below in vector registers,
+    // and every address would then be computed there)
+    for (int32_t base = 0; base < mcount * J; base += 64) {
+        const int32_t idx = base + lane;
+        const int32_t mi = idx / J, j = idx - mi * J;
+        const int32_t d = d0 + j < D ? d0 + j : D - 1;
+        if (idx < mcount * J)
+            mycarry[idx] = first_prop_grad ? Elem<T>::widen(first_prop_grad[((b * M + m0 + mi) * D + d)]) : 0.0f;
+    }
+    // Row j of the block's group of d, clamped: a d beyond D (last group) is loaded like any
+    // other (as D - 1), never accumulated or stored. Everything here is wave-uniform.
+    auto d_of = [&](int j) { return d0 + j < D ? d0 + j : D - 1; };
+    auto slot_of = [&](int32_t mi) {  // clamped: a wave without slots still issues (unused) loads
+        const int32_t m = m0 + mi;
+        return m < M ? m : M - 1;
+    };
 
-    const T* __restrict__ xrow = tokens + (b * D + d) * L;  // never read when PLAIN
-    const T* __restrict__ yrow = layer_out_grad + (b * D + d) * L;  // never read unless LAYER
-    T* __restrict__ dxrow = token_grad + (b * D + d) * L;
 
     // What a step loads, exactly as it arrives: anything computed from a loaded value at
     // the time of the load would have to be finished before the loop comes round, which
-    // means waiting for every load in flight. Fill values for chunks beyond L and the
-    // choice of h[-1] are therefore applied when the entry is used.
-    struct Entry {
-        u32x4 g, G, h, x;
-        u32x4 co, cs, y;  // LAYER only
-        u32x4 rr;         // LAYER == 2: rms of the chunk's steps
-        T hb;
-        T hbr;            // LAYER == 2: rms at the step hb belongs to
+    // means waiting for every load in flight.
+    struct Row {
+        u32x4 a;   // out_grad, or the normalised states (LAYER)
+        u32x4 h;   // saved states (LAYER != 2)
+        T hb;      // what stands before the tile in the row that `h` comes from
     };
-    // Where a visit is: chunk `chunk` of row (b, m, d), with the offsets that go with it
-    // kept as running sums in scalar registers (a 64-bit product per step would run on the
-    // vector unit, at a quarter of the rate).
-    struct Cursor {
-        int32_t chunk, m;
-        int64_t row;   // (b * M + m) * D + d
-        int64_t hoff;  // row * L: where the row starts in out_grad and h
-        int64_t goff;  // (b * M + m) * L: in gates
-        int64_t poff;  // ((b * M + m) * NG + grp) * L: in gate_partial
+    struct Slot {
+        u32x4 g;
+        FloatChunk<E> co, cs, rr;  // LAYER; rr: LAYER == 2
+        float hbr;                 // LAYER == 2: rms at the step hb belongs to
     };
-    const int64_t row_step = D, hoff_step = (int64_t)D * L, goff_step = L, poff_step = (int64_t)NG * L;
-    // the visit after: the next row at the same chunk, then row 0 of the chunk before
-    auto advance = [&](Cursor& c) {
-        const bool wrap = c.m + 1 == M;
-        c.chunk = wrap ? c.chunk - 1 : c.chunk;
-        c.m = wrap ? 0 : c.m + 1;
-        c.row = uniform64(wrap ? c.row - (M - 1) * row_step : c.row + row_step);
-        c.hoff = uniform64(wrap ? c.hoff - (M - 1) * hoff_step : c.hoff + hoff_step);
-        c.goff = uniform64(wrap ? c.goff - (M - 1) * goff_step : c.goff + goff_step);
-        c.poff = uniform64(wrap ? c.poff - (M - 1) * poff_step : c.poff + poff_step);
-    };
-    const int32_t lane_off32 = (63 - lane) * E;
-    // tile i of the chunk; addresses are clamped into the row (a chunk before the first, or
-    // a tile past the last, reads the nearest tile of the row)
-    auto fetch = [&](Entry& e, const Cursor& c, int i) {
-        int32_t k = c.chunk * C + i;
-        k = k < 0 ? 0 : (k > ntiles - 1 ? ntiles - 1 : k);
-        const int64_t tw = (int64_t)k * TILE;
-        const int64_t left = L - tw;
+    // lane offset (elements) inside tile k, clamped into the row (a chunk past the end reads the last one)
+    auto lane_elems = [&](int32_t k) {
+        const int64_t left = L - (int64_t)k * TILE;
         const int32_t rem = left < TILE ? (int32_t)left : TILE;
-        const uint32_t loff = (uint32_t)(lane_off32 < rem ? lane_off32 : rem - E) * (uint32_t)sizeof(T);
-        auto at = [&](const T* base) {  // scalar base + 32-bit lane offset
-            return reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + loff);
-        };
-        // where h comes from: the saved states, or the normalised ones (LAYER == 2)
-        const T* __restrict__ hrow = (LAYER == 2 ? out_grad : h_saved) + c.hoff;
-        e.g = load16<T, false>(at(gates + c.goff + tw));
-        e.G = load16<T, true>(at(out_grad + c.hoff + tw));
-        e.h = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (LAYER != 2) e.h = load16<T, true>(at(hrow + tw));
-        e.x = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (!PLAIN) e.x = load16<T, false>(at(xrow + tw));
-        e.co = e.cs = e.y = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (LAYER != 0) {
-            e.co = load16<T, false>(at(coef_out + c.goff + tw));
-            e.cs = load16<T, false>(at(coef_self + c.goff + tw));
-            e.y = load16<T, false>(at(yrow + tw));
-        }
-        e.rr = u32x4{0u, 0u, 0u, 0u};
-        e.hbr = T(0);
-        if constexpr (LAYER == 2) {
-            e.rr = load16<T, false>(at(rms + c.goff + tw));
-            e.hbr = rms[c.goff + (tw > 0 ? tw - 1 : 0)];
-        }
+        return (uint32_t)(lane_off < rem ? lane_off : rem - E);
+    };
+    auto fetch_row = [&](Row& r, int32_t k, int32_t mi, int j) {
+        const int64_t tw = (int64_t)k * TILE;
+        const uint32_t lo = lane_elems(k);
+        const int64_t row = (b * M + slot_of(mi)) * D + d_of(j);
+        const int64_t base = row * L + tw;
+        r.a = load16<T, true>(out_grad + base + lo);
+        r.h = u32x4{0u, 0u, 0u, 0u};
+        if constexpr (LAYER != 2) r.h = load16<T, true>(h_saved + base + lo);
+        const T* __restrict__ hsrc = LAYER == 2 ? out_grad : h_saved;
         // h just before the tile (h[-1] at the start of the row): one address for the whole wave
-        const T* src = tw > 0 ? hrow + (tw - 1) : (h0 != nullptr ? h0 + c.row : hrow);
-        e.hb = *src;
+        const T* src = tw > 0 ? hsrc + (base - 1) : (h0 != nullptr ? h0 + row : hsrc + base);
+        r.hb = *src;
+    };
+    auto fetch_slot = [&](Slot& s, int32_t k, int32_t mi) {
+        const int64_t tw = (int64_t)k * TILE;
+        const uint32_t lo = lane_elems(k);
+        const int64_t base = (b * M + slot_of(mi)) * L + tw;
+        s.g = load16<T, false>(gates + base + lo);
+        if constexpr (LAYER != 0) {
+            s.co = load_float_chunk<E>(coef_out + base + lo);
+            s.cs = load_float_chunk<E>(coef_self + base + lo);
+        }
+        s.hbr = 0.0f;
+        if constexpr (LAYER == 2) {
+            s.rr = load_float_chunk<E>(rms + base + lo);
+            s.hbr = rms[base - (tw > 0 ? 1 : 0)];
+        }
+    };
+    // the position one slot ahead of (k, mi): the next slot of the tile, else the first slot of
+    // the tile before; before the first tile there is nothing: stay (the loads are not used)
+    auto ahead = [&](int32_t& k, int32_t& mi) {
+        if (mi + 1 < mcount) {
+            ++mi;
+        } else if (k > 0) {
+            --k;
+            mi = 0;
+        }
     };
 
-    Entry q[R][C];
-    Cursor ahead = {nchunks - 1, 0, uniform64(b * M * D + d), uniform64((b * M * D + d) * L),
-                    uniform64(b * M * L), uniform64((b * M * NG + grp) * L)};
-    Cursor at = ahead;
+    // The J token rows of the block (and the J rows of the layer's output gradient) are the same
+    // for every slot and every wave: each tile of them is loaded once per block, J / NW rows
+    // per wave, and passed through LDS, a tile ahead of its use.
+    constexpr bool kSharedX = !PLAIN, kSharedY = LAYER != 0;
+    struct TokenShare {
+        u32x4 x[J / NW], y[J / NW];
+    };
+    auto fetch_share = [&](TokenShare& ts, int32_t k) {
+        const int64_t tw = (int64_t)k * TILE;
+        const uint32_t lo = lane_elems(k);
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-#pragma unroll
-        for (int i = C - 1; i >= 0; --i) fetch(q[r][i], ahead, i);
-        advance(ahead);
-    }
-
-    __syncthreads();  // carries are in place
-
-    float dtok[C][E], xf[HOIST ? C : 1][E], yf[HOIST ? C : 1][E];
-#pragma unroll
-    for (int i = 0; i < C; ++i) {
-#pragma unroll
-        for (int j = 0; j < E; ++j) dtok[i][j] = 0.0f;
-    }
-#pragma unroll
-    for (int i = 0; i < (HOIST ? C : 1); ++i) {
-#pragma unroll
-        for (int j = 0; j < E; ++j) xf[i][j] = yf[i][j] = 0.0f;
-    }
-    int parity = 0;
-    const int32_t visits = nchunks * M;  // the host checks that this fits
-    for (int32_t n = 0; n < visits; n += R) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if (n + r >= visits) break;  // same for every wave of the block
-            const int32_t m = at.m;
-            float carry = mycarry[m];
-#pragma unroll
-            for (int i = C - 1; i >= 0; --i) {
-                Entry cur = q[r][i];
-                fetch(q[r][i], ahead, i);
-
-                const int32_t k = at.chunk * C + i;  // may be past the last tile in the last chunk
-                const int64_t tw = (int64_t)k * TILE;
-                if (tw + TILE > L && tw + lane_off >= L) {  // short or absent tile: nothing there
-                    cur.g = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
-                    cur.G = cur.h = cur.x = cur.co = cur.cs = cur.y = u32x4{0u, 0u, 0u, 0u};
-                    cur.rr = u32x4{0u, 0u, 0u, 0u};
-                }
-                float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(cur.hb) : 0.0f;
-                if constexpr (LAYER == 2) {
-                    if (k > 0) hb *= Elem<T>::widen(cur.hbr);  // at k == 0 it is the initial state itself
-                }
-                float g[E], G[E], h[E], p[E], xs[E];
-                Elem<T>::unpack(cur.g, g);
-                Elem<T>::unpack(cur.G, G);
-                Elem<T>::unpack(cur.h, h);
-                if constexpr (!PLAIN) {
-                    if constexpr (HOIST) {
-                        if (m == 0) Elem<T>::unpack(cur.x, xf[i]);  // the M rows share their tokens
-                    } else {
-                        Elem<T>::unpack(cur.x, xs);
-                    }
-                }
-                if constexpr (LAYER == 2) {  // h = normalised state * rms (G[] holds the normalised state)
-                    float r[E];
-                    Elem<T>::unpack(cur.rr, r);
-#pragma unroll
-                    for (int j = 0; j < E; ++j) h[j] = G[j] * r[j];
-                }
-                if constexpr (LAYER != 0) {
-                    float co[E], cs[E], ys[E];
-                    Elem<T>::unpack(cur.co, co);
-                    Elem<T>::unpack(cur.cs, cs);
-                    if constexpr (HOIST) {
-                        if (m == 0) Elem<T>::unpack(cur.y, yf[i]);  // shared by the M rows, like the tokens
-                    } else {
-                        Elem<T>::unpack(cur.y, ys);
-                    }
-#pragma unroll
-                    for (int j = 0; j < E; ++j) {
-                        const float y = HOIST ? yf[HOIST ? i : 0][j] : ys[j];
-                        G[j] = __builtin_fmaf(-cs[j], G[j], co[j] * y);  // G[] held the normalised state
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < E; ++j) p[j] = g[j] * G[j];
-                float a = g[E - 1], bb = p[E - 1];
-#pragma unroll
-                for (int j = E - 2; j >= 0; --j) {
-                    bb = __builtin_fmaf(g[j], bb, p[j]);
-                    a *= g[j];
-                }
-                wave_scan_inclusive(a, bb);
-                const float ea = dpp<kWaveShr1>(1.0f, a);
-                const float eb = dpp<kWaveShr1>(0.0f, bb);
-                const float ta = lane63(a), tb = lane63(bb);
-                const float hprev0 = dpp<kWaveShl1>(hb, h[E - 1]);
-
-                float c = __builtin_fmaf(ea, carry, eb);
-                carry = __builtin_fmaf(ta, carry, tb);
-                float dg[E];
-#pragma unroll
-                for (int j = E - 1; j >= 0; --j) {
-                    const float delta = G[j] + c;
-                    c = __builtin_fmaf(g[j], c, p[j]);
-                    const float hp = (j > 0) ? h[j > 0 ? j - 1 : 0] : hprev0;
-                    if constexpr (PLAIN) {
-                        dtok[i][j] += delta;
-                        dg[j] = hp * delta;
-                    } else {
-                        dtok[i][j] += __builtin_fmaf(-g[j], delta, delta);
-                        const float x = HOIST ? xf[HOIST ? i : 0][j] : xs[j];
-                        dg[j] = (hp - x) * delta;
-                    }
-                }
-                if (!active) {  // whole wave: a wave past the last d adds nothing
-#pragma unroll
-                    for (int j = 0; j < E; ++j) dg[j] = 0.0f;
-                }
-
-                // add the gate gradient tiles of the DG waves: each wave lays its tile out in
-                // memory order, then sums one slice of the tile over all waves and stores it
-                float* mine = red + (parity * DG + w) * TILE + lane_off;
-#pragma unroll
-                for (int j = 0; j < E; j += 4)
-                    *reinterpret_cast<float4*>(mine + j) = make_float4(dg[j], dg[j + 1], dg[j + 2], dg[j + 3]);
-                __syncthreads();
-                const float* all = red + parity * DG * TILE + w * SLICE;
-                float* __restrict__ prow = gate_partial + at.poff + tw + w * SLICE;
-                for (int e = lane; e < SLICE; e += 64) {
-                    float sum = 0.0f;
-#pragma unroll
-                    for (int v = 0; v < DG; ++v) sum += all[v * TILE + e];
-                    if (tw + w * SLICE + e < L) __builtin_nontemporal_store(sum, prow + e);
-                }
-                parity ^= 1;
-            }
-            if (lane == 0) mycarry[m] = carry;
-
-            if (m + 1 == M) {  // the chunk's token gradient is complete
-#pragma unroll
-                for (int i = 0; i < C; ++i) {
-                    const int64_t t0 = (int64_t)(at.chunk * C + i) * TILE + lane_off;
-                    if (active) store_chunk<T, true>(dxrow, t0, L, Elem<T>::pack(dtok[i]));
-#pragma unroll
-                    for (int j = 0; j < E; ++j) dtok[i][j] = 0.0f;
-                }
-            }
-            advance(at);
-            advance(ahead);
+        for (int s = 0; s < J / NW; ++s) {
+            const int32_t jj = w * (J / NW) + s;
+            const int32_t d = d0 + jj < D ? d0 + jj : D - 1;
+            const int64_t off = (b * D + d) * L + tw + lo;
+            ts.x[s] = ts.y[s] = u32x4{0u, 0u, 0u, 0u};
+            if constexpr (kSharedX) ts.x[s] = load16<T, false>(tokens + off);
+            if constexpr (kSharedY) ts.y[s] = load16<T, false>(layer_out_grad + off);
         }
+    };
+    auto publish_share = [&](const TokenShare& ts, int par) {
+#pragma unroll
+        for (int s = 0; s < J / NW; ++s) {
+            const int32_t jj = w * (J / NW) + s;
+            if constexpr (kSharedX) shared_xy[((par * J + jj) * 2 + 0) * 64 + lane] = ts.x[s];
+            if constexpr (kSharedY) shared_xy[((par * J + jj) * 2 + 1) * 64 + lane] = ts.y[s];
+        }
+    };
+
+    Row rows[J];
+    Slot next_slot;
+    int32_t kf = ntiles - 1, mf = 0;  // where the loads are: one step (a slot's J rows) ahead of the work
+    fetch_slot(next_slot, kf, mf);
+#pragma unroll
+    for (int j = 0; j < J; ++j) fetch_row(rows[j], kf, mf, j);
+
+    int parity = 0;
+    if constexpr (kSharedX || kSharedY) {
+        TokenShare first;
+        fetch_share(first, ntiles - 1);
+        publish_share(first, parity);
+    }
+    __syncthreads();  // carries and the first tile of the shared rows are in place
+
+    for (int32_t k = ntiles - 1; k >= 0; --k) {
+        const int64_t tw = (int64_t)k * TILE;
+        TokenShare upcoming;  // the tile before this one, on its way to LDS
+        if constexpr (kSharedX || kSharedY) fetch_share(upcoming, k > 0 ? k - 1 : 0);
+        const bool inside = tw + lane_off < L;  // this lane's chunk lies in the row (tiles are whole chunks)
+        float dtok[J][E];
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+#pragma unroll
+            for (int i = 0; i < E; ++i) dtok[j][i] = 0.0f;
+        }
+        for (int32_t mi = 0; mi < mcount; ++mi) {
+            const Slot cur = next_slot;
+            ahead(kf, mf);
+            fetch_slot(next_slot, kf, mf);
+
+            // per slot: gates (1 where there is no step: identity), coefficients (0 there: no gradient)
+            float g[E], co[E], cs[E];
+            Elem<T>::unpack(cur.g, g);
+            if constexpr (LAYER != 0) {
+                spread<E>(cur.co, co);
+                spread<E>(cur.cs, cs);
+            }
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+                g[i] = inside ? g[i] : 1.0f;
+                if constexpr (LAYER != 0) {
+                    co[i] = inside ? co[i] : 0.0f;
+                    cs[i] = inside ? cs[i] : 0.0f;
+                }
+            }
+            float a = g[E - 1];
+#pragma unroll
+            for (int i = E - 2; i >= 0; --i) a *= g[i];
+            const GateLevels levels = scan_gates(a);
+
+            // The slot's gate gradient over this group of d is sum_d (h[t-1] - x[t]) * delta[t]. With
+            // the states taken back from the normalised ones, h[t-1] = rms[t-1] * n[t-1] and rms
+            // belongs to the slot: sum_d n[t-1] * delta[t] is built up (`with_state`), the factor
+            // applied once, after the rows; sum_d x[t] * delta[t] separately (`with_token`).
+            float with_state[E], with_token[E];
+#pragma unroll
+            for (int i = 0; i < E; ++i) with_state[i] = with_token[i] = 0.0f;
+            float* carry_of = mycarry + mi * J;
+
+            {
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const Row r = rows[j];
+                    fetch_row(rows[j], kf, mf, j);
+
+                    float carry = carry_of[j];
+                    float G[E], h[E], x[E];
+                    Elem<T>::unpack(r.a, G);
+                    // what stands before the tile in the row: a state, or a normalised one (the factor
+                    // follows with the slot); at k == 0 the initial state itself, or nothing
+                    const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(r.hb) : 0.0f;
+                    if constexpr (LAYER == 2) {
+#pragma unroll
+                        for (int i = 0; i < E; ++i) h[i] = G[i];  // G[] holds the normalised state
+                    } else {
+                        Elem<T>::unpack(r.h, h);
+                    }
+                    if constexpr (LAYER != 0) {
+                        float y[E];
+                        Elem<T>::unpack(shared_xy[((parity * J + j) * 2 + 1) * 64 + lane], y);
+#pragma unroll
+                        for (int i = 0; i < E; ++i) G[i] = __builtin_fmaf(-cs[i], G[i], co[i] * y[i]);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < E; ++i) G[i] = inside ? G[i] : 0.0f;
+                    }
+                    if constexpr (!PLAIN) Elem<T>::unpack(shared_xy[((parity * J + j) * 2 + 0) * 64 + lane], x);
+
+                    // the chunk as one step on what arrives from later steps: c_out = a * c_in + bb
+                    float bb = g[E - 1] * G[E - 1];
+#pragma unroll
+                    for (int i = E - 2; i >= 0; --i) bb = g[i] * (bb + G[i]);
+                    scan_values(bb, levels);
+                    const float eb = dpp<kWaveShr1>(0.0f, bb);
+                    const float tb = lane63(bb);
+                    const float hprev0 = dpp<kWaveShl1>(hb, h[E - 1]);
+
+                    float c = __builtin_fmaf(levels.ea, carry, eb);
+                    carry = __builtin_fmaf(levels.ta, carry, tb);
+                    if (lane == 0) carry_of[j] = carry;
+                    const bool counted = d0 + j < D;  // the whole wave: a row past the last d adds nothing
+#pragma unroll
+                    for (int i = E - 1; i >= 0; --i) {
+                        const float delta = G[i] + c;
+                        c = g[i] * delta;
+                        const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
+                        // token gradient (1 - g) * delta = delta - g * delta
+                        dtok[j][i] += PLAIN ? delta : delta - c;
+                        if (counted) {
+                            with_state[i] = __builtin_fmaf(hp, delta, with_state[i]);
+                            if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
+                        }
+                    }
+                }
+            }
+
+            // the slot's gate gradient, summed over this group of d
+            float dgate[E];
+            if constexpr (LAYER == 2) {
+                // rms at the step before each element: the chunk's own values moved up by one, the
+                // first from the lane that owns the chunk before (lane 63: from before the tile; at
+                // k == 0 what stands there is the initial state itself: factor 1)
+                float rr[E];
+                spread<E>(cur.rr, rr);
+                const float before = dpp<kWaveShl1>(k > 0 ? cur.hbr : 1.0f, rr[E - 1]);
+#pragma unroll
+                for (int i = 0; i < E; ++i)
+                    dgate[i] = __builtin_fmaf(i > 0 ? rr[i > 0 ? i - 1 : 0] : before, with_state[i], -with_token[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < E; ++i) dgate[i] = with_state[i] - with_token[i];
+            }
+            if (inside) {
+                float* __restrict__ prow = gate_partial + ((b * M + m0 + mi) * NG + grp) * L + tw + lane_off;
+#pragma unroll
+                for (int i = 0; i < E; i += 4) {
+                    const u32x4 v = {f2u(dgate[i]), f2u(dgate[i + 1]), f2u(dgate[i + 2]), f2u(dgate[i + 3])};
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(prow + i));
+                }
+            }
+        }
+
+        // the shared rows of the tile before: in place once the barriers below have been passed
+        // (its buffer was last read two tiles ago)
+        if constexpr (kSharedX || kSharedY) publish_share(upcoming, parity ^ 1);
+
+        // the token gradients of the tile go down the waves; the last wave stores the sums
+        float* buf = handover + parity * (J * TILE);
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) {
+            if (w == ww) {
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+#pragma unroll
+                    for (int q4 = 0; q4 < E / 4; ++q4) {
+                        float4* cell = reinterpret_cast<float4*>(buf + ((j * (E / 4) + q4) * 64 + lane) * 4);
+                        if (ww > 0) {
+                            const float4 v = *cell;
+                            dtok[j][4 * q4] += v.x; dtok[j][4 * q4 + 1] += v.y;
+                            dtok[j][4 * q4 + 2] += v.z; dtok[j][4 * q4 + 3] += v.w;
+                        }
+                        if (ww < NW - 1)
+                            *cell = make_float4(dtok[j][4 * q4], dtok[j][4 * q4 + 1], dtok[j][4 * q4 + 2],
+                                                dtok[j][4 * q4 + 3]);
+                    }
+                    if (ww == NW - 1 && d0 + j < D)
+                        store_chunk<T, true>(token_grad + (b * D + d0 + j) * L, tw + lane_off, L, Elem<T>::pack(dtok[j]));
+                }
+            }
+            if (ww < NW - 1) __syncthreads();
+        }
+        parity ^= 1;
     }
 
-    if (h0_grad && active) {
+    if (h0_grad) {
         __builtin_amdgcn_wave_barrier();  // lane 0's carry writes precede the reads below
-        for (int32_t mm = lane; mm < M; mm += 64) {
-            float v[E] = {mycarry[mm]};
+        for (int32_t base = 0; base < mcount * J; base += 64) {
+            const int32_t idx = base + lane;
+            const int32_t mi = idx / J, j = idx - mi * J;
+            if (idx >= mcount * J || d0 + j >= D) continue;
+            float v[E] = {mycarry[idx]};
             const u32x4 packed = Elem<T>::pack(v);
-            const int64_t row = (b * M + mm) * D + d;
+            const int64_t row = (b * M + m0 + mi) * D + d0 + j;
             if constexpr (sizeof(T) == 4) reinterpret_cast<uint32_t*>(h0_grad)[row] = packed.x;
             else reinterpret_cast<uint16_t*>(h0_grad)[row] = (uint16_t)(packed.x & 0xffffu);
         }

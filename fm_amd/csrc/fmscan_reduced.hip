@@ -7,10 +7,8 @@ using namespace fmscan::host;
 
 namespace {
 
-constexpr int kReducedGroup = 8;  // consecutive d one block of the reduced backward kernel sums over
-constexpr int kReducedChunk = 4;  // tiles of a row visited before moving to the next m
-constexpr int kLayerChunk = 2;    // ... in the form that makes the states' gradient on the spot
-constexpr int kReducedDepth = 1;  // visits whose loads are in flight ahead of the one worked on
+constexpr int kReducedGroup = 4;  // consecutive d one block of the reduced backward kernel sums over
+constexpr int kReducedWaves = 4;  // waves of a block: they split the M memory slots between them
 
 }  // namespace
 
@@ -23,8 +21,8 @@ int64_t fmscan_reduced_groups(int64_t D) { return D < 1 ? 0 : (D + kReducedGroup
 static int backward_reduced(const char* who, const void* gates, const void* out_grad, const void* first_prop_grad,
                             void* token_grad, const void* cached_output, const void* input_tokens,
                             float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
-                            const void* coef_out, const void* coef_self, const void* layer_out_grad,
-                            const void* rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                            const float* coef_out, const float* coef_self, const void* layer_out_grad,
+                            const float* rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
                             unsigned flags, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
@@ -55,10 +53,10 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                          {"cached_output", cached_output, full},
                          {"input_tokens", pb.plain ? nullptr : input_tokens, B * D * L * pb.esize},
                          {"initial_state", initial_state, pb.rows * pb.esize},
-                         {"coef_out", coef_out, B * M * L * pb.esize},
-                         {"coef_self", layer ? coef_self : nullptr, B * M * L * pb.esize},
+                         {"coef_out", coef_out, B * M * L * 4},
+                         {"coef_self", layer ? coef_self : nullptr, B * M * L * 4},
                          {"out_grad", layer ? layer_out_grad : nullptr, B * D * L * pb.esize},
-                         {"rms", recover ? rms : nullptr, B * M * L * pb.esize}};
+                         {"rms", recover ? rms : nullptr, B * M * L * 4}};
     for (const Range& o : outs)
         for (const Range& in : ins)
             if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
@@ -73,36 +71,37 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     if (!vec)
         return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
     const size_t tile = (size_t)(16 / pb.esize) * 64;
-    const size_t lds = (2 * kReducedGroup * tile + (size_t)kReducedGroup * (size_t)M) * sizeof(float);
+    const int64_t Mw = (M + kReducedWaves - 1) / kReducedWaves;  // slots per wave
+    const size_t lds = (2 * kReducedGroup * tile + 2 * kReducedGroup * 2 * 64 * 4 +
+                        (size_t)kReducedWaves * (size_t)Mw * kReducedGroup) * sizeof(float);
     if (lds > kMaxDynamicLds)
         return fail(FMSCAN_E_SHAPE, "%s: M = %lld needs %zu bytes of LDS (limit %u)", who, (long long)M, lds,
                     kMaxDynamicLds);
-    if ((L + (int64_t)tile - 1) / (int64_t)tile + kReducedChunk > INT32_MAX / M)
-        return fail(FMSCAN_E_SHAPE, "%s: M * ceil(L / %zu) must be < 2^31", who, tile);
+    if ((L + (int64_t)tile - 1) / (int64_t)tile > INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: ceil(L / %zu) must be < 2^31", who, tile);
     const void* h_init = initial_state ? initial_state : first_prop_grad;
     const unsigned grid = (unsigned)(B * groups);
     int rc = 0;
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
-        auto go = [&](auto pt, auto lt, auto ct) {
-            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, decltype(ct)::value, kReducedDepth,
-                                                             decltype(pt)::value, decltype(lt)::value>;  // lt: 0 plain call, 1 layer, 2 layer + recovered states
+        auto go = [&](auto pt, auto lt) {
+            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, kReducedWaves, decltype(pt)::value,
+                                                             decltype(lt)::value>;  // lt: 0 plain call, 1 layer, 2 layer + recovered states
             static std::atomic<uint64_t> armed{0};
             if ((rc = raise_lds_limit((const void*)kern, armed, who)) != 0) return;
-            kern<<<grid, 64 * kReducedGroup, lds, (hipStream_t)stream>>>(
+            kern<<<grid, 64 * kReducedWaves, lds, (hipStream_t)stream>>>(
                 (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
                 (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
-                (T*)initial_state_grad, (const T*)coef_out, (const T*)coef_self, (const T*)layer_out_grad,
-                (const T*)(recover ? rms : nullptr), (int32_t)M, (int32_t)D, L);
+                (T*)initial_state_grad, coef_out, coef_self, (const T*)layer_out_grad,
+                recover ? rms : nullptr, (int32_t)M, (int32_t)D, L, (int32_t)Mw);
         };
-        auto with_plain = [&](auto lt, auto ct) {
-            if (pb.plain) go(BoolTag<true>{}, lt, ct);
-            else go(BoolTag<false>{}, lt, ct);
+        auto with_plain = [&](auto lt) {
+            if (pb.plain) go(BoolTag<true>{}, lt);
+            else go(BoolTag<false>{}, lt);
         };
-        // the layer forms hold three more loads per ring entry: two tiles per visit instead of four
-        if (recover) with_plain(IntTag<2>{}, IntTag<kLayerChunk>{});
-        else if (layer) with_plain(IntTag<1>{}, IntTag<kLayerChunk>{});
-        else with_plain(IntTag<0>{}, IntTag<kReducedChunk>{});
+        if (recover) with_plain(IntTag<2>{});
+        else if (layer) with_plain(IntTag<1>{});
+        else with_plain(IntTag<0>{});
     });
     if (rc) return rc;
     return launched(who);
@@ -118,9 +117,9 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
                             nullptr, nullptr, B, M, D, L, dtype, flags, stream);
 }
 
-int fmscan_backward_layer(const void* gates, const void* states_n, const void* coef_out, const void* coef_self,
+int fmscan_backward_layer(const void* gates, const void* states_n, const float* coef_out, const float* coef_self,
                           const void* out_grad, const void* first_prop_grad, void* token_grad,
-                          const void* cached_output, const void* rms, const void* input_tokens,
+                          const void* cached_output, const float* rms, const void* input_tokens,
                           float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
                           int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags, void* stream) {
     if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer: coef_out must not be NULL");

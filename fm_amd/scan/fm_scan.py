@@ -484,8 +484,8 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
     if ext_grad is None and _reduced_ok(gates, tokens, states_n, states_n) and _aligned(read, out_grad):
         code = _dtype_code(states_n)
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
-        coef_out, coef_self = torch.empty_like(read), torch.empty_like(read)
-        rms = torch.empty_like(read) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
+        coef_out, coef_self = torch.empty_like(q), torch.empty_like(q)  # float32, like q
+        rms = torch.empty_like(q) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
         groups = _raw.fmscan_reduced_groups(D)
         d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
@@ -595,7 +595,7 @@ class FM_Memory(torch.autograd.Function):
         dev = alpha.device
         d_alpha = torch.empty_like(alpha)
         d_update_scale, d_output_scale = torch.empty_like(update_scale), torch.empty_like(output_scale)
-        if partial.shape[2] > 16:
+        if partial.shape[2] > 64:
             # many groups of d: the finishing kernel walks them one by one, a reduction does better
             partial = partial.sum(dim=2, keepdim=True)
         partial = partial.contiguous()

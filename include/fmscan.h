@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FMSCAN_ABI_VERSION 3
+#define FMSCAN_ABI_VERSION 4
 
 /* element type of every tensor in one call (reference fm_scan.cuh:333-342) */
 #define FMSCAN_DTYPE_F32  0
@@ -177,7 +177,7 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
  * M > 1 and D > 1; the per-pair tensors are never written.
  *   token_grad         (B, D, L)     out, element dtype: sum over m of (1 - g) * delta
  *   gate_grad_partial  (B, M, G, L)  out, float32, G = fmscan_reduced_groups(D): the sum of
- *                      (h[t-1] - x[t]) * delta over each group of 8 consecutive d;
+ *                      (h[t-1] - x[t]) * delta over each group of 4 consecutive d;
  *                      d_gates[b,m,t] is the sum of the G partials (one more small pass
  *                      for the caller; sums are accumulated in float32 throughout)
  * Other arguments as fmscan_backward. Needs 16-byte aligned pointers and
@@ -201,18 +201,19 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
  * which is the gradient of the RMS norm and read-out (fmscan_readout_backward without
  * ext_grad) when coef_out = inv_rms * read and coef_self = inv_rms * read * q / D, and of
  * the read-out alone when coef_out = read, coef_self = 0 and states_n = cached_output.
- *   states_n   (B, M, D, L)  the normalised states      coef_out, coef_self  (B, M, L)
+ *   states_n   (B, M, D, L)  the normalised states      coef_out, coef_self  (B, M, L) float32
  *   out_grad   (B, D, L)     gradient of the layer's output, time last
- * all of the call's dtype. cached_output may be NULL when rms ((B, M, L), 1 / inv_rms:
+ * states_n and out_grad of the call's dtype. cached_output may be NULL when rms ((B, M, L)
+ * float32, 1 / inv_rms:
  * fmscan_readout_dot writes it) is given: the scanned states are then taken back from the
  * normalised ones, states_n * rms, and the layer need not keep them (the reference keeps
  * them for autograd, fm/scan/fm_scan.py:53-55). Everything else, and the limits, as
  * fmscan_backward_reduced.
  */
 int fmscan_backward_layer(const void* gates, const void* states_n,
-                          const void* coef_out, const void* coef_self, const void* out_grad,
+                          const float* coef_out, const float* coef_self, const void* out_grad,
                           const void* first_prop_grad, void* token_grad,
-                          const void* cached_output, const void* rms,
+                          const void* cached_output, const float* rms,
                           const void* input_tokens, float* gate_grad_partial,
                           const void* initial_state, void* initial_state_grad,
                           int64_t B, int64_t M, int64_t D, int64_t L,
@@ -244,11 +245,11 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
  *                           (float32; it is the gradient of `read`) and, when ext_grad
  *                           (a gradient arriving at the returned memory states,
  *                           (B, M, D, L)) is not NULL, qe = sum_d ext_grad * states_n.
- *                           With coef_out and coef_self ((B, M, L), the call's dtype)
+ *                           With coef_out and coef_self ((B, M, L), float32)
  *                           not NULL it also writes what fmscan_backward_layer takes:
  *                           coef_out = inv_rms * read, coef_self = coef_out * q / D
  *                           (inv_rms NULL: coef_out = read, coef_self = 0), and with rms_out
- *                           ((B, M, L), the call's dtype) not NULL, rms_out = 1 / inv_rms.
+ *                           ((B, M, L), float32) not NULL, rms_out = 1 / inv_rms.
  * fmscan_readout_backward:  state_grad (B, M, D, L) = gradient of the scanned states:
  *                           dn = read * out_grad (+ ext_grad);
  *                           with the norm  inv_rms * (dn - states_n * (read*q + qe) / D),
@@ -263,8 +264,8 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
                            int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* ext_grad,
                        float* q, float* qe,
-                       const float* inv_rms, const void* read, void* coef_out, void* coef_self,
-                       void* rms_out,
+                       const float* inv_rms, const void* read, float* coef_out, float* coef_self,
+                       float* rms_out,
                        int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 int fmscan_readout_backward(const void* states_n, const float* inv_rms, const void* read,
                             const void* out_grad, const void* ext_grad,
