@@ -92,6 +92,10 @@ def load() -> ctypes.CDLL:
     dims = [c_int64] * 4
     lib.fmscan_readout_inv_rms.restype = c_int
     lib.fmscan_readout_inv_rms.argtypes = [c_void_p] * 2 + dims + [c_int, c_float, c_void_p]
+    lib.fmscan_forward_normed_max_d.restype = c_int64
+    lib.fmscan_forward_normed_max_d.argtypes = []
+    lib.fmscan_forward_normed.restype = c_int
+    lib.fmscan_forward_normed.argtypes = [c_void_p] * 5 + dims + [c_int, c_float, c_void_p]
     lib.fmscan_readout_forward.restype = c_int
     lib.fmscan_readout_forward.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
     lib.fmscan_readout_dot.restype = c_int

@@ -260,4 +260,84 @@ __device__ __forceinline__ float lane63(float v) {
     return u2f((uint32_t)__builtin_amdgcn_readlane((int)f2u(v), 63));
 }
 
+// ---- wave scan with the gates' part done once ------------------------------------------
+// Rows that share their gates (the rows of one memory slot m) share the `a` halves of
+// all their step pairs and everything the wave scan does to them. scan_gates runs that half
+// once per slot and keeps what each of the six levels needs (the value of `a` before the
+// level); scan_values then scans the `b` half of a row with one instruction per level.
+struct GateLevels {
+    float before[6];  // a in this lane before level 1..6
+    float ea;         // product of the gates of all chunks before this lane's (1 in lane 0)
+    float ta;         // product over the whole tile
+};
+
+__device__ __forceinline__ GateLevels scan_gates(float a) {
+    GateLevels g;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mov_b32 %1, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %2, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %3, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %4, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %5, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %6, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "=&v"(g.before[0]), "=&v"(g.before[1]), "=&v"(g.before[2]), "=&v"(g.before[3]),
+          "=&v"(g.before[4]), "=&v"(g.before[5]));
+    g.ea = dpp<kWaveShr1>(1.0f, a);
+    g.ta = lane63(a);
+    return g;
+}
+
+__device__ __forceinline__ void scan_values(float& b, const GateLevels& g) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %1 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %2 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %3 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %4 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %5 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %6 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(b)
+        : "v"(g.before[0]), "v"(g.before[1]), "v"(g.before[2]), "v"(g.before[3]), "v"(g.before[4]),
+          "v"(g.before[5]));
+}
+
+// E consecutive floats at p (16-byte aligned)
+template <int E>
+struct FloatChunk {
+    float4 v[E / 4];
+};
+template <int E>
+__device__ __forceinline__ FloatChunk<E> load_float_chunk(const float* __restrict__ p) {
+    FloatChunk<E> c;
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) c.v[i] = reinterpret_cast<const float4*>(p)[i];
+    return c;
+}
+template <int E>
+__device__ __forceinline__ void spread(const FloatChunk<E>& c, float (&f)[E]) {
+#pragma unroll
+    for (int i = 0; i < E / 4; ++i) {
+        f[4 * i] = c.v[i].x; f[4 * i + 1] = c.v[i].y; f[4 * i + 2] = c.v[i].z; f[4 * i + 3] = c.v[i].w;
+    }
+}
+
 }  // namespace fmscan

@@ -1,0 +1,157 @@
+// Forward scan and RMS norm of the Factorization-Memory layer in one kernel (reference
+// fm/scan/fm_scan.py:121-127: fm_scan, then states * rsqrt(mean(states^2, dim=2) + eps)):
+// the scanned states never reach memory, only the normalised ones the layer returns.
+#pragma once
+
+#include "fmscan_kernels.h"
+
+namespace fmscan {
+
+// A block is one memory slot (b, m) with all its D rows: wave w owns the J consecutive rows
+// d = w*J .. w*J + J - 1 (NW * J >= D). The block walks the tiles of the sequence from the
+// first to the last. In a tile every wave scans its J rows one after the other (the gate
+// half of the wave scan once for all of them), rounds the states to the storage type as a
+// stored state would be, keeps them packed in registers and adds up their squares; the
+// waves' sums meet in LDS, where each wave adds one slice of the tile over all waves and
+// turns it into inv_rms[b, m, t] = rsqrt(mean_d h^2 + eps) (stored as float32: the
+// read-out's gradient takes it); then every wave scales the states it holds and stores
+// them. Two barriers per tile. Only the gates and tokens are read (from the caches
+// mostly: the tokens serve all M slots of a batch element) and one (B, M, D, L) tensor is
+// written, against one written and read twice plus one more written when the scan, the sum
+// of squares and the scaling are separate kernels.
+// Needs 16-byte aligned rows (vector access only).
+template <typename T, int J, int NW>
+__global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
+    const T* __restrict__ gates, const T* __restrict__ tokens, const T* __restrict__ h0,
+    T* __restrict__ states_n /* (B, M, D, L) */, float* __restrict__ inv_rms /* (B, M, L) */, int32_t M,
+    int32_t D, int64_t L, float eps) {
+    constexpr int E = Elem<T>::E;
+    constexpr int TILE = E * 64;
+    constexpr int SLICE = TILE / NW;  // elements of a tile's sum of squares each wave finishes
+    static_assert(TILE % NW == 0 && SLICE <= 64, "a wave finishes at most one element per lane");
+    __shared__ float part[2][NW][TILE];  // every wave's sum of squares over its rows
+    __shared__ float scale[2][TILE];     // inv_rms of the tile
+
+    const int lane = threadIdx.x & 63;
+    const int w = uniform((int)(threadIdx.x >> 6));
+    // Blocks go to the 8 XCDs (each with its own L2) round robin. The M blocks of one b read
+    // the same tokens, so they are renumbered to share an XCD.
+    uint32_t id = blockIdx.x;
+    if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+    const int64_t bm = (int64_t)uniform((int)id);  // b * M + m
+    const int64_t b = uniform((int)(id / (uint32_t)M));
+    const int32_t d0 = w * J;
+    const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
+    const int32_t lane_off = lane * E;
+    auto d_of = [&](int j) { return d0 + j < D ? d0 + j : D - 1; };  // a row past D is loaded as D - 1 and dropped
+
+    float carry[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) carry[j] = h0 ? Elem<T>::widen(h0[bm * D + d_of(j)]) : 0.0f;
+
+    // lane offset (elements) inside tile k, clamped into the row (a chunk past the end reads the last one)
+    auto lane_elems = [&](int32_t k) {
+        const int64_t left = L - (int64_t)k * TILE;
+        const int32_t rem = left < TILE ? (int32_t)left : TILE;
+        return (uint32_t)(lane_off < rem ? lane_off : rem - E);
+    };
+    struct Loads {
+        u32x4 g;
+        u32x4 x[J];
+    };
+    auto fetch = [&](Loads& q, int32_t k) {  // k beyond the last tile: the last tile again (not used)
+        k = k < ntiles ? k : ntiles - 1;
+        const int64_t tw = (int64_t)k * TILE;
+        const uint32_t lo = lane_elems(k);
+        q.g = load16<T, false>(gates + bm * L + tw + lo);
+#pragma unroll
+        for (int j = 0; j < J; ++j) q.x[j] = load16<T, false>(tokens + (b * D + d_of(j)) * L + tw + lo);
+    };
+
+    Loads next;
+    fetch(next, 0);
+    int parity = 0;
+    for (int32_t k = 0; k < ntiles; ++k) {
+        const Loads cur = next;
+        fetch(next, k + 1);
+        const int64_t tw = (int64_t)k * TILE;
+        const bool inside = tw + lane_off < L;  // this lane's chunk lies in the row (tiles are whole chunks)
+
+        float g[E];
+        Elem<T>::unpack(cur.g, g);
+#pragma unroll
+        for (int i = 0; i < E; ++i) g[i] = inside ? g[i] : 1.0f;
+        float a = g[0];
+#pragma unroll
+        for (int i = 1; i < E; ++i) a *= g[i];
+        const GateLevels levels = scan_gates(a);
+
+        u32x4 held[J];
+        float sumsq[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) sumsq[i] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            float u[E];
+            Elem<T>::unpack(cur.x[j], u);
+#pragma unroll
+            for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], u[i], u[i]);  // (1 - g) x, one rounding
+            float bb = u[0];
+#pragma unroll
+            for (int i = 1; i < E; ++i) bb = __builtin_fmaf(g[i], bb, u[i]);
+            scan_values(bb, levels);
+            const float eb = dpp<kWaveShr1>(0.0f, bb);
+            const float tb = lane63(bb);
+            float h = __builtin_fmaf(levels.ea, carry[j], eb);
+            carry[j] = __builtin_fmaf(levels.ta, carry[j], tb);
+            float o[E];
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+                h = __builtin_fmaf(g[i], h, u[i]);
+                o[i] = h;
+            }
+            held[j] = Elem<T>::pack(o);
+            if (d0 + j < D) {              // the whole wave
+                Elem<T>::unpack(held[j], o);  // the norm sees the states as they would be stored
+#pragma unroll
+                for (int i = 0; i < E; ++i) sumsq[i] = __builtin_fmaf(o[i], o[i], sumsq[i]);
+            }
+        }
+
+        // the waves' sums meet: every wave lays its own out in time order, then finishes a slice
+        float* mine = &part[parity][w][lane_off];
+#pragma unroll
+        for (int i = 0; i < E; i += 4)
+            *reinterpret_cast<float4*>(mine + i) = make_float4(sumsq[i], sumsq[i + 1], sumsq[i + 2], sumsq[i + 3]);
+        __syncthreads();
+        if (lane < SLICE) {
+            const int e = w * SLICE + lane;
+            float s = 0.0f;
+#pragma unroll
+            for (int v = 0; v < NW; ++v) s += part[parity][v][e];  // fixed order: run-to-run identical
+            s = 1.0f / __builtin_sqrtf(s / (float)D + eps);
+            scale[parity][e] = s;
+            if (tw + e < L) inv_rms[bm * L + tw + e] = s;
+        }
+        __syncthreads();
+        float r[E];
+#pragma unroll
+        for (int i = 0; i < E; i += 4) {
+            const float4 v = *reinterpret_cast<const float4*>(&scale[parity][lane_off + i]);
+            r[i] = v.x; r[i + 1] = v.y; r[i + 2] = v.z; r[i + 3] = v.w;
+        }
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            if (d0 + j < D) {
+                float o[E];
+                Elem<T>::unpack(held[j], o);
+#pragma unroll
+                for (int i = 0; i < E; ++i) o[i] *= r[i];
+                store_chunk<T, true>(states_n + (bm * D + d0 + j) * L, tw + lane_off, L, Elem<T>::pack(o));
+            }
+        }
+        parity ^= 1;
+    }
+}
+
+}  // namespace fmscan

@@ -1,0 +1,58 @@
+// fmscan_forward_normed: the layer's forward scan and RMS norm as one kernel.
+// Contract: include/fmscan.h.
+#include "fmscan_host.h"
+#include "fmscan_normed.h"
+
+using namespace fmscan::host;
+
+namespace {
+
+constexpr int64_t kNormedMaxD = 128;  // rows of one slot a block can hold in registers (16 waves x 8 rows)
+
+template <typename T, int J, int NW>
+void launch_normed(const void* g, const void* x, const void* h0, void* out, float* inv_rms, int64_t B, int64_t M,
+                   int64_t D, int64_t L, float eps, hipStream_t s) {
+    fmscan::scan_forward_normed_kernel<T, J, NW><<<(unsigned)(B * M), 64 * NW, 0, s>>>(
+        (const T*)g, (const T*)x, (const T*)h0, (T*)out, inv_rms, (int32_t)M, (int32_t)D, L, eps);
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t fmscan_forward_normed_max_d(void) { return kNormedMaxD; }
+
+int fmscan_forward_normed(const void* gates, const void* tokens, const void* initial_state, void* states_n,
+                          float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, float eps,
+                          void* stream) {
+    const char* who = "fmscan_forward_normed";
+    Problem pb;
+    if (int rc = parse(B, M, D, L, dtype, 0, &pb)) return rc;
+    if (!gates || !tokens || !states_n || !inv_rms)
+        return fail(FMSCAN_E_NULL, "%s: gates, tokens, states_n and inv_rms must not be NULL", who);
+    if (!(eps >= 0.0f)) return fail(FMSCAN_E_SHAPE, "%s: eps must be >= 0", who);
+    if (D > kNormedMaxD)
+        return fail(FMSCAN_E_SHAPE, "%s: D = %lld is beyond the %lld rows a block holds; use fmscan_forward, "
+                    "fmscan_readout_inv_rms and fmscan_readout_forward", who, (long long)D, (long long)kNormedMaxD);
+    if ((__int128)B * M > (__int128)INT32_MAX) return fail(FMSCAN_E_SHAPE, "%s: B * M must be < 2^31", who);
+    const Range outs[] = {{"states_n", states_n, pb.rows * L * pb.esize}, {"inv_rms", inv_rms, B * M * L * 4}};
+    const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
+                         {"tokens", tokens, B * D * L * pb.esize},
+                         {"initial_state", initial_state, pb.rows * pb.esize}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
+    if (overlap(outs[0], outs[1])) return fail(FMSCAN_E_ALIAS, "%s: states_n overlaps inv_rms", who);
+    if ((L * pb.esize) % 16 != 0 || !aligned16(gates) || !aligned16(tokens) || !aligned16(states_n))
+        return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        hipStream_t s = (hipStream_t)stream;
+        if (D <= 32) launch_normed<T, 4, 8>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, s);
+        else if (D <= 64) launch_normed<T, 4, 16>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, s);
+        else launch_normed<T, 8, 16>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, s);
+    });
+    return launched(who);
+}
+
+}  // extern "C"

@@ -457,11 +457,27 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
     else:
         initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
     states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
+    kept_state = initial_state if given_state else None
+    if (mem_norm and states.numel() and D <= _raw.fmscan_forward_normed_max_d() and (L * states.element_size()) % 16 == 0
+            and _aligned(gates, tokens, states)):
+        # scan and norm in one kernel: the scanned states never reach memory
+        dev = gates.device
+        _on_gpu("tokens", tokens, dev)
+        _on_gpu("read", read, dev)
+        _require(tokens.dtype == gates.dtype, f"tokens has dtype {tokens.dtype}, gates has {gates.dtype}")
+        inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev)
+        with _on_device(dev):
+            _lib.check(_raw.fmscan_forward_normed(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+                                                    states.data_ptr(), inv_rms.data_ptr(), B, M, D, L,
+                                                    _dtype_code(gates), float(norm_eps),
+                                                    torch.cuda.current_stream(dev).cuda_stream))
+        output, _, _ = fm_readout_forward(states, read, mem_norm=False)  # the read-out alone, of the normalised states
+        return output, None, states, inv_rms, kept_state
     fm_scan_forward(gates, tokens, initial_state, states)
     # with the norm the scanned states are needed no longer (backward takes them back from the
     # normalised ones): normalise in place, one (B, M, D, L) tensor at any time
     output, normed, inv_rms = fm_readout_forward(states, read, mem_norm, norm_eps, in_place=bool(mem_norm))
-    return output, (None if mem_norm else states), normed, inv_rms, (initial_state if given_state else None)
+    return output, (None if mem_norm else states), normed, inv_rms, kept_state
 
 
 def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms, out_grad, ext_grad,

@@ -273,6 +273,26 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
                             int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
 
 /*
+ * Forward scan and RMS norm in one call (reference fm/scan/fm_scan.py:121-127 inside
+ * fm_memory: fm_scan, then states * rsqrt(mean(states^2, dim=2) + eps)): what fmscan_forward,
+ * fmscan_readout_inv_rms and the scaling half of fmscan_readout_forward compute one after the
+ * other, without the scanned states ever reaching memory. A block holds all D rows of a
+ * memory slot in registers, hence D <= fmscan_forward_normed_max_d() (FMSCAN_E_SHAPE beyond:
+ * use the three calls), and it needs 16-byte aligned pointers with
+ * L * sizeof(element) % 16 == 0 (FMSCAN_E_UNALIGNED otherwise).
+ *   gates (B, M, L), tokens (B, D, L), initial_state (B, M, D) or NULL    in
+ *   states_n (B, M, D, L)   out: the normalised states (each state is rounded to the call's
+ *                           dtype before it enters the norm, as a stored state would be)
+ *   inv_rms  (B, M, L)      out, float32
+ * The read-out over the slots is then fmscan_readout_forward(states_n, NULL, read, NULL, output).
+ */
+int64_t fmscan_forward_normed_max_d(void);
+int fmscan_forward_normed(const void* gates, const void* tokens, const void* initial_state,
+                          void* states_n, float* inv_rms,
+                          int64_t B, int64_t M, int64_t D, int64_t L,
+                          int dtype, float eps, void* stream);
+
+/*
  * The layer's small tensors (reference fm/scan/fm_scan.py:116,118-119,130 and their
  * gradients): alpha (B, L, M), update_scale and output_scale (B, L, 1), all of the call's
  * dtype.

@@ -195,3 +195,47 @@ def test_layer_at_the_benchmark_shape(scan):
                "d_update_scale": us.grad[b:b + 1], "d_output_scale": osc.grad[b:b + 1], "d_inputs": inp.grad[b:b + 1]}
         tols = {k: (FWD_TOL if k in ("output", "memory_states") else GRAD_TOL)[dt] for k in want}
         check_all(f"fm_memory bench shape, batch element {b}", got, want, tols)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_forward_scan_and_norm_in_one_kernel(scan, dtype):
+    """fmscan_forward_normed (through the C interface) against the float64 oracle and against the three
+    separate calls it stands for; D up to the limit, ragged D and L, with and without initial state."""
+    lib, st = scan.module, torch.cuda.current_stream().cuda_stream
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    limit = lib.fmscan_forward_normed_max_d()
+    assert limit >= 128
+    for (B, M, D, L), with_h0 in [((2, 3, 5, 512), True), ((1, 2, 33, 1000), False), ((2, 4, 64, 4096), True),
+                                  ((1, 3, 128, 2056), True), ((3, 2, 100, 8), False), ((1, 1, 1, 2048), True)]:
+        gen = torch.Generator().manual_seed(D * 10 + L)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV) if with_h0 else None
+        eps = 1e-5
+        normed = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        inv = torch.empty(B, M, L, device=DEV)
+        rc = lib.fmscan_forward_normed(g.data_ptr(), x.data_ptr(), None if h0 is None else h0.data_ptr(),
+                                       normed.data_ptr(), inv.data_ptr(), B, M, D, L, code, eps, st)
+        assert rc == 0, lib.fmscan_last_error()
+        states = O.forward(g, x, h0)
+        _, o_normed, o_inv = O.readout_forward(states, np.ones((B, M, L)), True, eps)
+        tag = f"{(B, M, D, L)} {dtype}"
+        tol = FWD_TOL[dtype]
+        check_all(tag, {"normalised states": normed, "inv_rms": inv}, {"normalised states": o_normed, "inv_rms": o_inv},
+                  {"normalised states": tol, "inv_rms": tol})
+        # the separate calls: scan, sum of squares, scaling
+        z = torch.zeros(B, M, D, dtype=dtype, device=DEV)
+        out = torch.empty_like(normed)
+        scan.fm_scan_forward(g, x, z if h0 is None else h0, out)
+        _, n3, r3 = scan.fm_readout_forward(out, torch.ones(B, M, L, dtype=dtype, device=DEV), True, eps)
+        check_all(tag + " vs three calls", {"normalised states": normed, "inv_rms": inv},
+                  {"normalised states": n3.double().cpu().numpy(), "inv_rms": r3.double().cpu().numpy()},
+                  {"normalised states": tol, "inv_rms": 1e-5})
+    # beyond the limit and unaligned: rejected, nothing launched
+    D = limit + 1
+    g = torch.rand(1, 1, 64, device=DEV); x = torch.rand(1, D, 64, device=DEV)
+    n = torch.empty(1, 1, D, 64, device=DEV); r = torch.empty(1, 1, 64, device=DEV)
+    assert lib.fmscan_forward_normed(g.data_ptr(), x.data_ptr(), None, n.data_ptr(), r.data_ptr(), 1, 1, D, 64, 0,
+                                     1e-6, st) == -2
+    assert lib.fmscan_forward_normed(g.data_ptr(), x.data_ptr(), None, n.data_ptr(), r.data_ptr(), 1, 1, 4, 63, 0,
+                                     1e-6, st) == -7

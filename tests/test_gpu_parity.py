@@ -554,7 +554,9 @@ def test_layer_backward_kernel_equals_the_two_step_route(scan, dtype, mem_norm):
         # one step, through the autograd node
         leaves = [t.clone().requires_grad_() for t in (g, x, h0, read)]
         out_b, _ = scan.fm_layer(*leaves[:3], leaves[3], mem_norm, 1e-5)
-        assert torch.equal(out_b, out)
+        # (the one node runs scan and norm as one kernel where it can: its sum of squares is
+        # taken in another order, so the outputs agree to rounding, not to the bit)
+        check("output vs separate calls", out_b, out.double().cpu().numpy(), TOL[dtype])
         out_b.backward(og)
         tag = f"{(B, M, D, L)} {dtype} norm={mem_norm}"
         tol = 2 * TOL[dtype]  # two rounded results against each other, each within TOL of the exact one
@@ -606,7 +608,7 @@ def test_layer_prepare_and_finish_kernels(scan, dtype):
 
 def test_scan_then_readout_equals_the_one_node_layer(scan):
     """fm_scan followed by fm_readout (two autograd nodes, a (B, M, D, L) gradient between them) and
-    fm_layer (one node) are the same function: same values, gradients within the storage type's
+    fm_layer (one node) are the same function: values and gradients within the storage type's
     rounding of each other."""
     B, M, D, L, dt = 2, 4, 24, 2048, torch.bfloat16
     gen = gpu_gen(17)
@@ -622,8 +624,8 @@ def test_scan_then_readout_equals_the_one_node_layer(scan):
             out, mem = scan.fm_layer(g, x, h, r, True, 1e-5)
         out.backward(w)
         grads.append([out.detach(), mem.detach(), g.grad, x.grad, h.grad, r.grad])
-    assert torch.equal(grads[0][0], grads[1][0]) and torch.equal(grads[0][1], grads[1][1])
-    for a, b, name in zip(grads[0][2:], grads[1][2:], ("d_gates", "d_tokens", "d_initial_state", "d_read")):
+    for a, b, name in zip(grads[0], grads[1], ("output", "memory states", "d_gates", "d_tokens", "d_initial_state",
+                                               "d_read")):
         check(name, b, a.double().cpu().numpy(), 2e-2)  # two bfloat16 results against each other
 
 
