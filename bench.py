@@ -49,13 +49,35 @@ WORKLOADS = {
     "cfg5f16": (32, 4096, 2048, "float16"),  # configuration 5 in its other 16-bit type
 }
 
-# HBM bytes per backward launch read from rocprofv3 counters (FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads for a copy of known
-# size); the runs are summarised under profiles/. None = not measured.
-MEASURED_BWD_TRAFFIC_BYTES = {
-    # FETCH_SIZE 2106124.4 KiB x 2.0 (copy calibration) + WRITE_SIZE 2097152.1 KiB x 1.0
-    "cfg3": int((2106124.4 * 2.0 + 2097152.1) * 1024),
-}
+STORAGE = {"bfloat16": "bf16", "float32": "f32", "float16": "f16"}
+
+
+def profiled_traffic(stem, kernel, copy_bytes):
+    """HBM bytes per launch of `kernel` (parts of its name, joined by *) from the rocprofv3 counter
+    summaries kept under profiles/:
+    FETCH_SIZE + WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads in the
+    same run for an elementwise copy of known size (torch.neg, `copy_bytes` read and written).
+    Returns (bytes or None, what it was read from)."""
+    total, used = 0.0, []
+    for counter in ("fetch_size", "write_size"):
+        path = ROOT / "profiles" / f"{stem}_pmc_{counter}.txt"
+        if not path.exists():
+            return None, f"profiles/{path.name} is not there"
+        copy_kib, kernel_kib = None, None
+        for line in path.read_text().splitlines():
+            cols = line.split()
+            if len(cols) < 6 or cols[-5].upper() != counter.upper():
+                continue
+            name, avg = " ".join(cols[:-5]), float(cols[-3])
+            if "neg_kernel" in name:  # the probe's copy (the row with four launches)
+                copy_kib = avg if int(cols[-4]) >= 4 else copy_kib
+            elif all(part in name for part in kernel.split("*")):
+                kernel_kib = avg
+        if not copy_kib or kernel_kib is None:
+            return None, f"profiles/{path.name} has no row for {kernel} or for the copy"
+        total += kernel_kib * (copy_bytes / 1024.0 / copy_kib) * 1024.0
+        used.append(f"profiles/{path.name}")
+    return int(total), " + ".join(used)
 
 
 def make_inputs(torch, name, device):
@@ -189,25 +211,32 @@ def run_layer(torch, args) -> int:
     normed, sg = torch.empty_like(states), torch.empty_like(states)
     out = torch.empty(B, D, L, dtype=dt, device=dev)
     coef, dtok = rn(B, M, L), torch.empty(B, D, L, dtype=dt, device=dev)  # coefficient vectors are float32
-    partial = torch.empty(B, M, lib.fmscan_reduced_groups(D), L, device=dev)
+    partial = torch.empty(B, M, lib.fmscan_reduced_groups(D), L, device=dev)  # float32: groups of 4 consecutive d
     code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
     P = lambda t: t.data_ptr()
     calls = {
+        # what fm_memory runs, forward: scan and norm in one kernel, then the read-out of the normalised states
+        "scan_forward_normed_kernel": (s * N, lambda: lib.fmscan_forward_normed(
+            P(gates), P(tokens), None, P(normed), P(inv), B, M, D, L, code, 1e-6, st)),
+        "readout_forward_kernel (read-out alone)": (s * N, lambda: lib.fmscan_readout_forward(
+            P(normed), None, P(read), None, P(out), B, M, D, L, code, st)),
+        # backward, with only the output in the loss: the dot products, then the scan's backward kernel in
+        # the form that makes the states' gradient itself (no readout_backward_kernel, no G) and takes the
+        # scanned states back from the normalised ones (reads one (B,M,D,L) tensor)
+        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, None, None, None, None, None, B, M, D, L, code, st)),
+        "scan_backward_reduced_kernel (layer form)": (s * N + 4 * N // 4, lambda: lib.fmscan_backward_layer(
+            P(gates), P(normed), P(coef), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
+            None, None, B, M, D, L, code, 0, st)),
+        # the same steps as separate kernels (what runs for D beyond one block's rows, or with the
+        # returned memory states in the loss)
         "scan_forward_kernel": (s * N, lambda: S.fm_scan_forward(gates, tokens, zeros, states)),
         "rowdot_kernel (inv_rms)": (s * N, lambda: lib.fmscan_readout_inv_rms(P(states), P(inv), B, M, D, L, code, 1e-6, st)),
         "readout_forward_kernel": (2 * s * N, lambda: lib.fmscan_readout_forward(
             P(states), P(inv), P(read), P(normed), P(out), B, M, D, L, code, st)),
-        "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, None, None, None, None, None, B, M, D, L, code, st)),
         "readout_backward_kernel": (2 * s * N, lambda: lib.fmscan_readout_backward(
             P(normed), P(inv), P(read), P(og), None, P(q), None, P(sg), B, M, D, L, code, st)),
-        "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 8, lambda: S.fm_scan_backward_reduced(
-            gates, G, zeros, states, tokens)),
-        # what the layer's backward runs when only its output feeds the loss: the kernel above in
-        # the form that makes the states' gradient itself (no readout_backward_kernel, no G) and
-        # takes the scanned states back from the normalised ones (reads one (B,M,D,L) tensor)
-        "scan_backward_reduced_kernel (layer form)": (s * N + 4 * N // 8, lambda: lib.fmscan_backward_layer(
-            P(gates), P(normed), P(coef), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
-            None, None, B, M, D, L, code, 0, st)),
+        "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 4, lambda: lib.fmscan_backward_reduced(
+            P(gates), P(G), P(zeros), P(dtok), P(states), P(tokens), P(partial), None, None, B, M, D, L, code, 0, st)),
     }
     if args.probe:  # for rocprofv3 --pmc: a copy of known size, then every kernel a few times
         for _ in range(4):
@@ -233,20 +262,19 @@ def run_layer(torch, args) -> int:
         ms = ev[0].elapsed_time(ev[1]) / 10
         kernels[name] = {"ms": round(ms, 4), "algorithmic_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
     dom = kernels["scan_backward_reduced_kernel (layer form)"]
+    traffic, traffic_from = profiled_traffic(f"layer_kernels_B{B}_L{L}_M{M}_D{D}_{STORAGE[dtn]}",
+                                             "scan_backward_reduced_kernel*, 2>", s * N)
     result = {
         "metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
         "value": round(N / (ms_per_step * 1e-3) / 1e9, 2), "unit": "Gelem/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "storage_dtype": "bf16", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32", "storage_dtype": STORAGE[dtn], "data": "synthetic",
         "config": {"workload": f"layer: fm_memory (B,L,M,D)=({B},{L},{M},{D}) {dtn}, mem_norm, fwd+bwd via autograd",
                    "elements": N},
         "kernels": kernels,
         "roofline": {"kernel": "scan_backward_reduced_kernel (layer form)", "bound": "hbm", "achieved": dom["GBps"],
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(dom["GBps"] / PEAK_HBM_GBPS, 4),
-                     "algorithmic_bytes": dom["algorithmic_bytes"],
-                     # rocprofv3 counters, summarised under profiles/: FETCH_SIZE 297789.3 KiB x 2.0
-                     # (copy calibration) + WRITE_SIZE 147456.0 KiB x 1.0 per launch
-                     "traffic": int((297789.3 * 2.0 + 147456.0) * 1024)},
+                     "algorithmic_bytes": dom["algorithmic_bytes"], "traffic": traffic, "traffic_from": traffic_from},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = layer_cpu_baseline(torch, alpha, us, osc, inp, w_out)
@@ -357,8 +385,11 @@ def main() -> int:
     N = rows * T
     ms_per_step = elapsed * 1e3 / args.steps
     value = 9 * s * N / (ms_per_step * 1e-3) / 1e9
-    bwd_bytes = 6 * s * N
+    bwd_bytes = 6 * s * N   # the byte model of the metric: g, dL/dh, h, x read; two gradients written
+    bwd_moved = 5 * s * N   # what the kernel moves: it makes h again from g and x instead of reading it
     achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    stem = f"scan_kernels_{args.workload.replace('f16', '')}_{STORAGE[dtn]}"
+    traffic, traffic_from = profiled_traffic(stem, "scan_backward_kernel", s * N)
     result = {
         "metric": METRIC,
         "value": round(value, 1),
@@ -371,20 +402,26 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",  # the arithmetic type; tensors are stored as storage_dtype
-        "storage_dtype": {"bfloat16": "bf16", "float32": "f32", "float16": "f16"}[dtn],
+        "storage_dtype": STORAGE[dtn],
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: (B,C,T)=({B},{Cn},{T}) {dtn}, fwd+bwd, passed as "
                                f"{rows} rows with M=D=1, FM form h=g*h+(1-g)*x",
-                   "bytes_per_element": 9 * s, "elements": N},
+                   "bytes_per_element": 9 * s, "elements": N,
+                   "bytes_moved_per_element": 8 * s,
+                   "note": "value prices the step at the metric's 9 element sizes per element (forward 3, backward "
+                           "6); the backward kernel makes the states again from gates and tokens instead of "
+                           "reading them, so 8 are moved"},
         "pct_of_peak": round(100 * value / PEAK_HBM_GBPS, 2),
         "elements_per_s": round(N / (ms_per_step * 1e-3), 1),
         "fwd_ms": round(fwd_ms, 4),
         "bwd_ms": round(bwd_ms, 4),
         "fwd_GBps": round(3 * s * N / (fwd_ms * 1e-3) / 1e9, 1),
+        "moved_GBps": round(8 * s * N / (ms_per_step * 1e-3) / 1e9, 1),
         "roofline": {"kernel": "scan_backward_kernel", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBPS, 4),
-                     "algorithmic_bytes": bwd_bytes,
-                     "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.workload)},
+                     "algorithmic_bytes": bwd_bytes, "moved_bytes": bwd_moved,
+                     "frac_of_moved_bytes": round(bwd_moved / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+                     "traffic": traffic, "traffic_from": traffic_from},
     }
     if args.graph:
         side = torch.cuda.Stream()
