@@ -340,4 +340,60 @@ __device__ __forceinline__ void spread(const FloatChunk<E>& c, float (&f)[E]) {
     }
 }
 
+// The same split for the scan that runs down the lanes (row_scan_inclusive_down,
+// state_entering_lane_down): the gate half once for all rows that share their gates.
+struct GateLevelsDown {
+    float before[4];        // a in this lane before the four levels inside a row of 16 lanes
+    float xa;               // product of the gates of the lanes above, inside the row (1 in its lane 15)
+    float a48, a32, a16;    // products over the whole rows 3, 2, 1
+};
+
+__device__ __forceinline__ GateLevelsDown scan_gates_down(float a) {
+    GateLevelsDown g;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_mov_b32 %1, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %2, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %3, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_mov_b32 %4, %0\n\t"
+        "v_mul_f32_dpp %0, %0, %0 row_shl:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "=&v"(g.before[0]), "=&v"(g.before[1]), "=&v"(g.before[2]), "=&v"(g.before[3]));
+    g.xa = dpp<kRowShl1>(1.0f, a);
+    g.a48 = lane_value(a, 48);
+    g.a32 = lane_value(a, 32);
+    g.a16 = lane_value(a, 16);
+    return g;
+}
+
+// b half of a row's step pairs -> the state that enters every lane's chunk when `entry` (the
+// same in all lanes) enters lane 63's
+__device__ __forceinline__ float state_entering_lane_down(float b, const GateLevelsDown& g, float entry, int lane) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %1 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %2 row_shl:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %3 row_shl:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_fmac_f32_dpp %0, %0, %4 row_shl:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(b)
+        : "v"(g.before[0]), "v"(g.before[1]), "v"(g.before[2]), "v"(g.before[3]));
+    const float e3 = entry;
+    const float e2 = __builtin_fmaf(g.a48, e3, lane_value(b, 48));
+    const float e1 = __builtin_fmaf(g.a32, e2, lane_value(b, 32));
+    const float e0 = __builtin_fmaf(g.a16, e1, lane_value(b, 16));
+    const int row = lane >> 4;
+    const float e = row == 3 ? e3 : (row == 2 ? e2 : (row == 1 ? e1 : e0));
+    return __builtin_fmaf(g.xa, e, dpp<kRowShl1>(0.0f, b));
+}
+
 }  // namespace fmscan

@@ -99,10 +99,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // What a step loads, exactly as it arrives: anything computed from a loaded value at
     // the time of the load would have to be finished before the loop comes round, which
     // means waiting for every load in flight.
+    // Where the saved states are at hand (LAYER != 2) and there are tokens (!PLAIN), the states
+    // of a tile are not read but made again from its gates and tokens and the one saved state
+    // before the tile, as scan_backward_kernel does.
+    constexpr bool REMAKE = LAYER != 2 && !PLAIN;
     struct Row {
         u32x4 a;   // out_grad, or the normalised states (LAYER)
-        u32x4 h;   // saved states (LAYER != 2)
+        u32x4 h;   // saved states (PLAIN only)
         T hb;      // what stands before the tile in the row that `h` comes from
+        T h_first; // REMAKE, first tile: the saved h[0] (elsewhere: hb again)
     };
     struct Slot {
         u32x4 g;
@@ -122,11 +127,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         const int64_t base = row * L + tw;
         r.a = load16<T, true>(out_grad + base + lo);
         r.h = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (LAYER != 2) r.h = load16<T, true>(h_saved + base + lo);
+        if constexpr (LAYER != 2 && !REMAKE) r.h = load16<T, true>(h_saved + base + lo);
         const T* __restrict__ hsrc = LAYER == 2 ? out_grad : h_saved;
         // h just before the tile (h[-1] at the start of the row): one address for the whole wave
         const T* src = tw > 0 ? hsrc + (base - 1) : (h0 != nullptr ? h0 + row : hsrc + base);
         r.hb = *src;
+        r.h_first = T(0);
+        if constexpr (REMAKE) r.h_first = hsrc[tw > 0 ? base - 1 : base];  // no new cache line except in the first tile
     };
     auto fetch_slot = [&](Slot& s, int32_t k, int32_t mi) {
         const int64_t tw = (int64_t)k * TILE;
@@ -233,6 +240,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
             for (int i = E - 2; i >= 0; --i) a *= g[i];
             const GateLevels levels = scan_gates(a);
+            // (first tile: the chain of remade states starts at the saved h[0], whatever enters: the
+            // first step of lane 63, which owns the start of the row, counts as gate 0, token h[0])
+            const bool first_step = k == 0 && lane == 63;
+            GateLevelsDown down;
+            if constexpr (REMAKE) down = scan_gates_down(first_step ? 0.0f : a);
 
             // The slot's gate gradient over this group of d is sum_d (h[t-1] - x[t]) * delta[t]. With
             // the states taken back from the normalised ones, h[t-1] = rms[t-1] * n[t-1] and rms
@@ -258,7 +270,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     if constexpr (LAYER == 2) {
 #pragma unroll
                         for (int i = 0; i < E; ++i) h[i] = G[i];  // G[] holds the normalised state
-                    } else {
+                    } else if constexpr (!REMAKE) {
                         Elem<T>::unpack(r.h, h);
                     }
                     if constexpr (LAYER != 0) {
@@ -271,6 +283,20 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                         for (int i = 0; i < E; ++i) G[i] = inside ? G[i] : 0.0f;
                     }
                     if constexpr (!PLAIN) Elem<T>::unpack(shared_xy[((parity * J + j) * 2 + 0) * 64 + lane], x);
+                    float hprev[E];  // the state before each of the chunk's steps
+                    if constexpr (REMAKE) {
+                        float u[E];
+#pragma unroll
+                        for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], x[i], x[i]);  // as the forward kernel forms it
+                        if (first_step) u[0] = Elem<T>::widen(r.h_first);
+                        float fb = u[0];
+#pragma unroll
+                        for (int i = 1; i < E; ++i) fb = __builtin_fmaf(g[i], fb, u[i]);
+                        hprev[0] = state_entering_lane_down(fb, down, hb, lane);
+                        hprev[1] = first_step ? u[0] : __builtin_fmaf(g[0], hprev[0], u[0]);
+#pragma unroll
+                        for (int i = 2; i < E; ++i) hprev[i] = __builtin_fmaf(g[i - 1], hprev[i - 1], u[i - 1]);
+                    }
 
                     // the chunk as one step on what arrives from later steps: c_out = a * c_in + bb
                     float bb = g[E - 1] * G[E - 1];
@@ -279,7 +305,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     scan_values(bb, levels);
                     const float eb = dpp<kWaveShr1>(0.0f, bb);
                     const float tb = lane63(bb);
-                    const float hprev0 = dpp<kWaveShl1>(hb, h[E - 1]);
+                    if constexpr (!REMAKE) {
+                        hprev[0] = dpp<kWaveShl1>(hb, h[E - 1]);
+#pragma unroll
+                        for (int i = 1; i < E; ++i) hprev[i] = h[i - 1];
+                    }
 
                     float c = __builtin_fmaf(levels.ea, carry, eb);
                     carry = __builtin_fmaf(levels.ta, carry, tb);
@@ -289,7 +319,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     for (int i = E - 1; i >= 0; --i) {
                         const float delta = G[i] + c;
                         c = g[i] * delta;
-                        const float hp = (i > 0) ? h[i > 0 ? i - 1 : 0] : hprev0;
+                        const float hp = hprev[i];
                         // token gradient (1 - g) * delta = delta - g * delta
                         dtok[j][i] += PLAIN ? delta : delta - c;
                         if (counted) {
