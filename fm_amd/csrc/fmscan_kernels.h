@@ -70,6 +70,38 @@ __device__ __forceinline__ Segment locate_segment(int64_t slot, int32_t nseg, in
     return s;
 }
 
+// Which slot (row, or segment of a row) wave-group `local` of a block works on: rows in memory
+// order, unless rows that share their inputs are better visited together. With M > 1 the M rows
+// (b, :, d) read the same tokens; when the tokens of a batch element do not fit an L2 (4 MiB
+// per XCD), going through the rows in memory order fetches them once per slot m instead of once
+// (D = 2048, L = 8192: as many bytes fetched as written). Then blocks are renumbered so that
+// every XCD (blocks go to the 8 XCDs round robin) takes a contiguous range of them, and inside
+// a batch element the rows are taken in groups of d whose tokens (256 KiB) stay in the cache
+// while the M slots are visited one after the other; within a slot the group's rows are
+// consecutive in memory, so the output is still written in runs. Measured on the forward
+// kernel at (1, 32, 2048, 8192): 0.24 -> 0.18 ms; shapes whose tokens fit are up to a quarter
+// slower in that order (their writes jump by D rows from block to block) and keep memory order.
+template <int R, bool FOLD>
+__device__ __forceinline__ int64_t slot_of_block(int local, int32_t M, int32_t D, int32_t nseg, int64_t row_bytes) {
+    uint32_t id = blockIdx.x;
+    if constexpr (!FOLD) {
+        if (nseg == 1 && M > 1 && D % R == 0 && D * row_bytes > (4 << 20)) {
+            const uint32_t quads = (uint32_t)(D / R);  // blocks per slot
+            uint32_t group = 1;                        // blocks of one slot visited before the next slot
+            while (group * 2 <= quads && (int64_t)(group * 2) * R * row_bytes <= (256 << 10)) group *= 2;
+            while (quads % group) group /= 2;
+            if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+            const uint32_t per_b = (uint32_t)M * quads, per_group = (uint32_t)M * group;
+            const uint32_t b = id / per_b, rest = id - b * per_b;
+            const uint32_t grp = rest / per_group, in_group = rest - grp * per_group;
+            const uint32_t m = in_group / group, dq = grp * group + (in_group - m * group);
+            const uint32_t gate_row = (uint32_t)uniform((int)(b * (uint32_t)M + m));
+            return (int64_t)gate_row * D + (int64_t)uniform((int)(dq * R)) + local;
+        }
+    }
+    return (int64_t)id * R + local;
+}
+
 // Meets the W wave totals of one tile in LDS. `cin` leaves as the state that
 // enters this wave's part of the tile, `carry` as the state after the tile.
 // Slots alternate between consecutive tiles, so one barrier per tile is enough:
@@ -106,7 +138,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_forward_kernel(
     const int lane = threadIdx.x & 63;
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int w = wave % W;
-    const int64_t slot = (int64_t)blockIdx.x * R + wave / W;
+    const int64_t slot = slot_of_block<R, FOLD>(wave / W, M, D, nseg, L * (int64_t)sizeof(T));
     if (slot >= rows * nseg) return;  // whole waves only, and only in barrier-free (W == 1) blocks
     const int64_t ntiles = (L + TILE - 1) / TILE;
     const Segment seg = locate_segment(slot, nseg, seg_tiles, ntiles);
@@ -249,7 +281,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
     const int lane = threadIdx.x & 63;
     const int wave = uniform((int)(threadIdx.x >> 6));
     const int w = wave % W;
-    const int64_t slot = (int64_t)blockIdx.x * R + wave / W;
+    const int64_t slot = slot_of_block<R, FOLD>(wave / W, M, D, nseg, L * (int64_t)sizeof(T));
     if (slot >= rows * nseg) return;
     const int64_t ntiles = (L + TILE - 1) / TILE;
     const Segment seg = locate_segment(slot, nseg, seg_tiles, ntiles);
