@@ -276,6 +276,35 @@ def test_broadcast_rows_equal_explicit_rows(scan):
     assert torch.equal(dx.view(-1), dxe.view(-1)) and torch.equal(dg.view(-1), dge.view(-1))
 
 
+@pytest.mark.parametrize("shape", [(1, 16, 1024, 4096), (1, 3, 1024, 4096), (2, 2, 600, 8192)])
+def test_rows_visited_out_of_memory_order_equal_explicit_rows(scan, shape):
+    """When the tokens of a batch element are too many for one L2 (D * L * element size > 4 MiB) the
+    kernels visit the rows slot after slot in groups of d instead of in memory order. Same rows, same
+    arithmetic: bit for bit what the fold-mapped problem with gates and tokens expanded by hand gives
+    (one wave per row in the first shape, several in the others)."""
+    B, M, D, L = shape
+    dt = torch.bfloat16
+    gen = gpu_gen(31)
+    g = torch.rand(B, M, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(B, D, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    assert D * L * 2 > (4 << 20)
+    out, dx, dg = run_fwd_bwd(scan, g, x, G)
+    ge = g[:, :, None, :].expand(B, M, D, L).reshape(B * M * D, 1, L).contiguous()
+    xe = x[:, None, :, :].expand(B, M, D, L).reshape(B * M * D, 1, L).contiguous()
+    kw = {"waves_per_row": 1} if B * M * D >= 16384 else {}
+    oe, dxe, dge = run_fwd_bwd(scan, ge, xe, G.view(B * M * D, 1, 1, L), **kw)
+    if kw:
+        assert torch.equal(out.view(-1), oe.view(-1))
+        assert torch.equal(dx.view(-1), dxe.view(-1)) and torch.equal(dg.view(-1), dge.view(-1))
+    else:  # the two problems may be given different numbers of waves per row: equal to rounding
+        for a, b, name in ((out, oe, "states"), (dx, dxe, "token grad"), (dg, dge, "gate grad")):
+            check(name, a, b.double().cpu().numpy().reshape(a.shape), TOL[dt])
+    idx = torch.randperm(B * M * D, device=DEV, generator=gen)[:64]
+    h_ref = C.forward_f64(ge[idx], xe[idx])
+    check("states", out.view(B * M * D, 1, 1, L)[idx], h_ref, TOL[dt])
+
+
 def test_segment_chaining(scan):
     """scan(L) == scan(first part) followed by scan(rest, initial_state = last state),
     and backward chains through first_prop_grad the same way."""
