@@ -96,6 +96,12 @@ def load() -> ctypes.CDLL:
     lib.fmscan_forward_normed_max_d.argtypes = []
     lib.fmscan_forward_normed.restype = c_int
     lib.fmscan_forward_normed.argtypes = [c_void_p] * 5 + dims + [c_int, c_float, c_void_p]
+    lib.fmscan_sumsq_groups.restype = c_int64
+    lib.fmscan_sumsq_groups.argtypes = [c_int64]
+    lib.fmscan_forward_sumsq.restype = c_int
+    lib.fmscan_forward_sumsq.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
+    lib.fmscan_sumsq_finish.restype = c_int
+    lib.fmscan_sumsq_finish.argtypes = [c_void_p, c_int64, c_void_p] + dims + [c_float, c_void_p]
     lib.fmscan_readout_forward.restype = c_int
     lib.fmscan_readout_forward.argtypes = [c_void_p] * 5 + dims + [c_int, c_void_p]
     lib.fmscan_readout_dot.restype = c_int

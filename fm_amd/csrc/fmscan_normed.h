@@ -20,11 +20,18 @@ namespace fmscan {
 // written, against one written and read twice plus one more written when the scan, the sum
 // of squares and the scaling are separate kernels.
 // Needs 16-byte aligned rows (vector access only).
-template <typename T, int J, int NW>
+//
+// WHOLE == false, for D beyond what one block holds: a block is NW * J consecutive rows of a
+// slot (blockIdx = ((b * DB + db) * M + m): the M blocks that read the same token rows follow
+// each other, and every XCD takes a contiguous range of blocks); it stores the scanned states
+// as they are and, in place of inv_rms, the sum of squares over its rows,
+// inv_rms[(b * M + m) * DB + db][t]: (B, M, DB, L) partial sums that sumsq_finish_kernel turns
+// into inv_rms. One barrier per tile. The sum of squares then costs no pass over the states.
+template <typename T, int J, int NW, bool WHOLE = true>
 __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     const T* __restrict__ gates, const T* __restrict__ tokens, const T* __restrict__ h0,
     T* __restrict__ states_n /* (B, M, D, L) */, float* __restrict__ inv_rms /* (B, M, L) */, int32_t M,
-    int32_t D, int64_t L, float eps) {
+    int32_t D, int64_t L, float eps, int32_t DB) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     constexpr int SLICE = TILE / NW;  // elements of a tile's sum of squares each wave finishes
@@ -38,9 +45,19 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     // the same tokens, so they are renumbered to share an XCD.
     uint32_t id = blockIdx.x;
     if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
-    const int64_t bm = (int64_t)uniform((int)id);  // b * M + m
-    const int64_t b = uniform((int)(id / (uint32_t)M));
-    const int32_t d0 = w * J;
+    int64_t bm, b;  // bm = b * M + m
+    int32_t db = 0;
+    if constexpr (WHOLE) {
+        bm = (int64_t)uniform((int)id);
+        b = uniform((int)(id / (uint32_t)M));
+    } else {
+        const uint32_t per_b = (uint32_t)M * (uint32_t)DB;
+        const uint32_t bb = id / per_b, rest = id - bb * per_b;
+        db = uniform((int)(rest / (uint32_t)M));
+        b = uniform((int)bb);
+        bm = (int64_t)uniform((int)(bb * (uint32_t)M + (rest - (uint32_t)db * (uint32_t)M)));
+    }
+    const int32_t d0 = (db * NW + w) * J;
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
     const int32_t lane_off = lane * E;
     auto d_of = [&](int j) { return d0 + j < D ? d0 + j : D - 1; };  // a row past D is loaded as D - 1 and dropped
@@ -112,6 +129,7 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
             }
             held[j] = Elem<T>::pack(o);
             if (d0 + j < D) {              // the whole wave
+                if constexpr (!WHOLE) store_chunk<T, true>(states_n + (bm * D + d0 + j) * L, tw + lane_off, L, held[j]);
                 Elem<T>::unpack(held[j], o);  // the norm sees the states as they would be stored
 #pragma unroll
                 for (int i = 0; i < E; ++i) sumsq[i] = __builtin_fmaf(o[i], o[i], sumsq[i]);
@@ -129,9 +147,17 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
             float s = 0.0f;
 #pragma unroll
             for (int v = 0; v < NW; ++v) s += part[parity][v][e];  // fixed order: run-to-run identical
-            s = 1.0f / __builtin_sqrtf(s / (float)D + eps);
-            scale[parity][e] = s;
-            if (tw + e < L) inv_rms[bm * L + tw + e] = s;
+            if constexpr (WHOLE) {
+                s = 1.0f / __builtin_sqrtf(s / (float)D + eps);
+                scale[parity][e] = s;
+                if (tw + e < L) inv_rms[bm * L + tw + e] = s;
+            } else {
+                if (tw + e < L) inv_rms[(bm * DB + db) * L + tw + e] = s;
+            }
+        }
+        if constexpr (!WHOLE) {
+            parity ^= 1;  // the other buffer next: no wave writes this one again before all have read it
+            continue;
         }
         __syncthreads();
         float r[E];
@@ -152,6 +178,18 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
         }
         parity ^= 1;
     }
+}
+
+// inv_rms[r][t] = rsqrt(sum_g partial[r][g][t] / D + eps) for the (B, M, G, L) partial sums of
+// squares the kernel above leaves (r = b * M + m). One thread per (r, t).
+__global__ __launch_bounds__(256) void sumsq_finish_kernel(const float* __restrict__ partial, float* __restrict__ inv_rms,
+                                                           int64_t rows, int32_t G, int64_t L, int32_t D, float eps) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * L) return;
+    const int64_t r = i / L, t = i - r * L;
+    float s = 0.0f;
+    for (int32_t g = 0; g < G; ++g) s += partial[(r * G + g) * L + t];
+    inv_rms[i] = 1.0f / __builtin_sqrtf(s / (float)D + eps);
 }
 
 }  // namespace fmscan

@@ -458,20 +458,34 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
         initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
     states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
     kept_state = initial_state if given_state else None
-    if (mem_norm and states.numel() and D <= _raw.fmscan_forward_normed_max_d() and (L * states.element_size()) % 16 == 0
-            and _aligned(gates, tokens, states)):
-        # scan and norm in one kernel: the scanned states never reach memory
+    if mem_norm and states.numel() and (L * states.element_size()) % 16 == 0 and _aligned(gates, tokens, states, read):
         dev = gates.device
         _on_gpu("tokens", tokens, dev)
         _on_gpu("read", read, dev)
         _require(tokens.dtype == gates.dtype, f"tokens has dtype {tokens.dtype}, gates has {gates.dtype}")
+        _require(read.dtype == gates.dtype and read.is_contiguous(), "read must be contiguous, of the gates' dtype")
+        code = _dtype_code(gates)
         inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         with _on_device(dev):
-            _lib.check(_raw.fmscan_forward_normed(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
-                                                    states.data_ptr(), inv_rms.data_ptr(), B, M, D, L,
-                                                    _dtype_code(gates), float(norm_eps),
-                                                    torch.cuda.current_stream(dev).cuda_stream))
-        output, _, _ = fm_readout_forward(states, read, mem_norm=False)  # the read-out alone, of the normalised states
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            if D <= _raw.fmscan_forward_normed_max_d():
+                # scan and norm in one kernel: the scanned states never reach memory
+                _lib.check(_raw.fmscan_forward_normed(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+                                                        states.data_ptr(), inv_rms.data_ptr(), B, M, D, L, code,
+                                                        float(norm_eps), stream))
+                output, _, _ = fm_readout_forward(states, read, mem_norm=False)  # the read-out alone
+                return output, None, states, inv_rms, kept_state
+            # too many rows per slot for one block: the scan leaves the sums of squares of blocks of rows,
+            # so the norm needs no pass over the states of its own; scaling and read-out then in place
+            groups = _raw.fmscan_sumsq_groups(D)
+            partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
+            output = torch.empty((B, D, L), dtype=states.dtype, device=dev)
+            _lib.check(_raw.fmscan_forward_sumsq(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+                                                   states.data_ptr(), partial.data_ptr(), B, M, D, L, code, stream))
+            _lib.check(_raw.fmscan_sumsq_finish(partial.data_ptr(), groups, inv_rms.data_ptr(), B, M, D, L,
+                                                  float(norm_eps), stream))
+            _lib.check(_raw.fmscan_readout_forward(states.data_ptr(), inv_rms.data_ptr(), read.data_ptr(),
+                                                     states.data_ptr(), output.data_ptr(), B, M, D, L, code, stream))
         return output, None, states, inv_rms, kept_state
     fm_scan_forward(gates, tokens, initial_state, states)
     # with the norm the scanned states are needed no longer (backward takes them back from the

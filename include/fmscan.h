@@ -293,6 +293,22 @@ int fmscan_forward_normed(const void* gates, const void* tokens, const void* ini
                           int dtype, float eps, void* stream);
 
 /*
+ * The same for any D, in two steps: fmscan_forward_sumsq is fmscan_forward (16-byte aligned rows only,
+ * FMSCAN_E_UNALIGNED otherwise) that also leaves the sums of squares of the states it stores (rounded to
+ * the call's dtype first, as fmscan_readout_inv_rms reads them) over blocks of 128 consecutive d:
+ *   sumsq_partial (B, M, G, L) float32, G = fmscan_sumsq_groups(D),
+ * so that the norm (reference fm/scan/fm_scan.py:125-126) needs no pass over the states of its own;
+ * fmscan_sumsq_finish turns the partial sums into inv_rms (B, M, L) float32 =
+ * rsqrt(sum_g partial / D + eps). fmscan_readout_forward(states, inv_rms, ...) follows.
+ */
+int64_t fmscan_sumsq_groups(int64_t D);
+int fmscan_forward_sumsq(const void* gates, const void* tokens, const void* initial_state,
+                         void* states, float* sumsq_partial,
+                         int64_t B, int64_t M, int64_t D, int64_t L, int dtype, void* stream);
+int fmscan_sumsq_finish(const float* sumsq_partial, int64_t G, float* inv_rms,
+                        int64_t B, int64_t M, int64_t D, int64_t L, float eps, void* stream);
+
+/*
  * The layer's small tensors (reference fm/scan/fm_scan.py:116,118-119,130 and their
  * gradients): alpha (B, L, M), update_scale and output_scale (B, L, 1), all of the call's
  * dtype.

@@ -26,10 +26,11 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
                                     "fmscan_backward_reduced", "fmscan_build_id",
                                     "fmscan_forward", "fmscan_forward_normed", "fmscan_forward_normed_max_d",
-                                    "fmscan_forward_static", "fmscan_last_error", "fmscan_layer_finish",
+                                    "fmscan_forward_static", "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
                                     "fmscan_layer_prepare", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
-                                    "fmscan_reduced_groups", "fmscan_swap_last_two", "fmscan_workspace_bytes"]
+                                    "fmscan_reduced_groups", "fmscan_sumsq_finish", "fmscan_sumsq_groups", "fmscan_swap_last_two",
+                                    "fmscan_workspace_bytes"]
 
 
 def test_every_declared_symbol_is_exported(lib):

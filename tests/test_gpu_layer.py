@@ -239,3 +239,37 @@ def test_forward_scan_and_norm_in_one_kernel(scan, dtype):
                                      1e-6, st) == -2
     assert lib.fmscan_forward_normed(g.data_ptr(), x.data_ptr(), None, n.data_ptr(), r.data_ptr(), 1, 1, 4, 63, 0,
                                      1e-6, st) == -7
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_forward_scan_with_the_sums_of_squares(scan, dtype):
+    """fmscan_forward_sumsq + fmscan_sumsq_finish (any D: the scan leaves the sums of squares over blocks
+    of 128 rows) against the float64 oracle, and against fmscan_forward + fmscan_readout_inv_rms."""
+    lib, st = scan.module, torch.cuda.current_stream().cuda_stream
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    for (B, M, D, L), with_h0 in [((1, 2, 300, 1024), True), ((2, 3, 129, 520), False), ((1, 3, 1024, 4096), True),
+                                  ((2, 2, 5, 64), False)]:
+        gen = torch.Generator().manual_seed(D + L)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV) if with_h0 else None
+        groups = lib.fmscan_sumsq_groups(D)
+        assert groups == (D + 127) // 128
+        states = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        partial = torch.full((B, M, groups, L), float("nan"), device=DEV)
+        inv = torch.empty(B, M, L, device=DEV)
+        assert lib.fmscan_forward_sumsq(g.data_ptr(), x.data_ptr(), None if h0 is None else h0.data_ptr(),
+                                        states.data_ptr(), partial.data_ptr(), B, M, D, L, code, st) == 0, \
+            lib.fmscan_last_error()
+        assert lib.fmscan_sumsq_finish(partial.data_ptr(), groups, inv.data_ptr(), B, M, D, L, 1e-5, st) == 0
+        tag = f"{(B, M, D, L)} {dtype}"
+        o_states = O.forward(g, x, h0)
+        _, _, o_inv = O.readout_forward(o_states, np.ones((B, M, L)), True, 1e-5)
+        check_all(tag, {"states": states, "inv_rms": inv}, {"states": o_states, "inv_rms": o_inv},
+                  {"states": FWD_TOL[dtype], "inv_rms": FWD_TOL[dtype]})
+        z = torch.zeros(B, M, D, dtype=dtype, device=DEV)
+        ref = torch.empty_like(states)
+        scan.fm_scan_forward(g, x, z if h0 is None else h0, ref)
+        assert torch.equal(ref, states), tag + ": the states differ from fmscan_forward's"
+        _, _, r3 = scan.fm_readout_forward(ref, torch.ones(B, M, L, dtype=dtype, device=DEV), True, 1e-5)
+        check_all(tag + " vs the separate sum", {"inv_rms": inv}, {"inv_rms": r3.double().cpu().numpy()}, {"inv_rms": 1e-5})
