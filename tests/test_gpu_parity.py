@@ -171,6 +171,16 @@ def test_config5_native_shape_through_autograd(scan):
         tg, gg = C.backward_f64(gb, Gb, states[b:b + 1], xb, None, np.zeros((1, M, D)))
         check("d_gates", g.grad[b:b + 1], gg.sum(axis=2), TOL[dt])
         check("d_tokens", x.grad[b:b + 1], tg.sum(axis=1), TOL[dt])
+    # every batch element, at full size: the kernel with the sums inside against the reference's route
+    # (both (B, M, D, L) tensors written in full, then torch.sum); two rounded results, hence 2 * TOL
+    zeros = torch.zeros(B, M, D, dtype=dt, device=DEV)
+    dx, dg = torch.empty_like(states), torch.empty_like(states)
+    scan.fm_scan_backward(g.detach(), G, zeros, dx, states.detach(), x.detach(), dg, initial_state=zeros)
+    check("d_gates, all batch elements", g.grad, dg.sum(dim=2).double().cpu().numpy(), 2 * TOL[dt])
+    check("d_tokens, all batch elements", x.grad, dx.sum(dim=1).double().cpu().numpy(), 2 * TOL[dt])
+    for b in range(B):  # and no batch element stands out
+        e = (g.grad[b].float() - dg[b].sum(dim=1).float()).abs().max().item() / dg[b].sum(dim=1).float().abs().max().item()
+        assert e <= 2 * TOL[dt], (b, e)
 
 
 # ----------------------------------------------------------------------------- shapes, dtypes, variants
