@@ -80,6 +80,54 @@ def profiled_traffic(stem, kernel, copy_bytes):
     return int(total), " + ".join(used)
 
 
+def streaming_copy(torch, rows, row_bytes, fwd_ms, bwd_ms, reps=10):
+    """What a bare streaming kernel with the scan kernels' access pattern reaches on the same shape.
+
+    `libfmscan_probe.so` (fm_amd/csrc/stream_probe.hip) walks `rows` rows of `row_bytes` bytes, one wave
+    per row, reading 2 tensors and writing 1 (the forward scan's streams) or reading 3 and writing 2
+    (the backward scan's), with no arithmetic and no tuning of residency. The published 8 TB/s is not
+    reachable by any kernel; this is a second reference point for kernels with these streams. Timed with
+    events on the current stream, best of two prefetch depths."""
+    import ctypes
+    from pathlib import Path
+    lib_path = Path(__file__).resolve().parent / "fm_amd" / "lib" / "libfmscan_probe.so"
+    if row_bytes % 1024 or not lib_path.exists():
+        return None
+    lib = ctypes.CDLL(str(lib_path))
+    lib.fmscan_probe_stream.restype = ctypes.c_int
+    lib.fmscan_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    tensor = rows * row_bytes
+    src = torch.ones(3 * tensor, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(2 * tensor, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, reads, writes in (("forward_streams", 2, 1), ("backward_streams", 3, 2)):
+        best = None
+        for depth in (2, 4):
+            def launch():
+                rc = lib.fmscan_probe_stream(src.data_ptr(), dst.data_ptr(), rows, row_bytes, reads, writes, depth,
+                                             stream)
+                if rc:
+                    raise RuntimeError(f"fmscan_probe_stream returned {rc}")
+            for _ in range(3):
+                launch()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                launch()
+            b.record()
+            b.synchronize()
+            ms = a.elapsed_time(b) / reps
+            best = ms if best is None else min(best, ms)
+        out[name] = {"reads": reads, "writes": writes, "ms": round(best, 4),
+                     "GBps": round((reads + writes) * tensor / (best * 1e-3) / 1e9, 1)}
+    # the scan kernels on the bytes they move, over the bare kernel with the same streams
+    out["forward_kernel_over_copy"] = round(out["forward_streams"]["ms"] / fwd_ms, 3)
+    out["backward_kernel_over_copy"] = round(out["backward_streams"]["ms"] / bwd_ms, 3)
+    return out
+
+
 def make_inputs(torch, name, device):
     B, Cn, T, dtn = WORKLOADS[name]
     dt = getattr(torch, dtn)
@@ -423,6 +471,7 @@ def main() -> int:
                      "frac_of_moved_bytes": round(bwd_moved / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                      "traffic": traffic, "traffic_from": traffic_from},
     }
+    result["streaming_copy"] = streaming_copy(torch, rows, T * s, fwd_ms, bwd_ms)
     if args.graph:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())

@@ -225,3 +225,21 @@ def test_workspace_bytes(lib):
     assert wb(4, 1, 1, 512, 2, 0) == 0                      # one tile per row: nothing to cut
     assert wb(4, 1, 1, 65536, 2, 4 << 8) == 0               # caller fixed the waves per row
     assert wb(0, 1, 1, 8, 0, 0) == 0                        # invalid problem
+
+
+def test_streaming_probe_library_rejects_what_it_does_not_cover():
+    """bench.py's bare streaming kernel lives in a library of its own; no GPU is needed to see it refuse."""
+    from fm_amd import build
+    if not build.PROBE_LIB.exists():
+        build.build_probe(verbose=False)
+    probe = ctypes.CDLL(str(build.PROBE_LIB))
+    f = probe.fmscan_probe_stream
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                  ctypes.c_int, ctypes.c_void_p]
+    a, b = 1 << 20, 1 << 30
+    assert f(None, b, 4, 1024, 2, 1, 2, None) == -1        # no input
+    assert f(a, b, 4, 1000, 2, 1, 2, None) == -1           # a row is not whole steps
+    assert f(a, b, 4, 1024, 1, 1, 2, None) == -1           # a stream count it has no kernel for
+    assert f(a, b, 4, 1024, 3, 2, 3, None) == -1           # a prefetch depth it has no kernel for
+    assert f(a + 8, b, 4, 1024, 3, 2, 2, None) == -1       # not 16-byte aligned
