@@ -16,6 +16,22 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
 
+// ---- loads of one address by the whole wave ---------------------------------------
+// A 4-byte load whose address is the same in every lane becomes a scalar load, and scalar
+// loads complete out of order on a counter they share with LDS traffic: the first wait for
+// an LDS read then also waits for every scalar load in flight, however far ahead of its use
+// it was issued. Where such a load is a prefetch (the one saved state before a tile, a
+// tile or more ahead, a miss in every cache), that wait is a trip to HBM per tile.
+// Indexing with a zero the compiler cannot see through keeps the load a vector load: those
+// return in order on a counter of their own, which the kernels count.
+__device__ __forceinline__ uint32_t opaque_zero() {
+    uint32_t z;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+    return z;
+}
+template <typename V>
+__device__ __forceinline__ V load_by_wave(const V* p, uint32_t zero) { return p[zero]; }
+
 // ---- 16 bytes <-> E fp32 values -------------------------------------------------
 // One lane always moves 16 bytes per tensor per tile: 4 fp32 or 8 fp16/bf16
 // consecutive sequence positions. Narrow types are widened to fp32 on load and

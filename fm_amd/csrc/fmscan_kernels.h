@@ -309,6 +309,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
     // states of a tile are not read but made again, in float32, from the tile's gates and
     // tokens (already in registers) and the one saved state just before this wave's part of
     // the tile: a second wave scan, forward in time, in place of a fourth 16-byte stream.
+    const uint32_t vzero = opaque_zero();
     struct Entry {
         u32x4 g, G;
         u32x4 hx;  // PLAIN: saved states; otherwise tokens
@@ -327,7 +328,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
         q.G = load16<T, true>(Grow + t0);
         if constexpr (PLAIN) q.hx = load16<T, true>(hrow + t0);
         else q.hx = load16<T, FOLD>(xrow + t0);
-        q.hb = Elem<T>::widen(hrow[k * TILE + wave_off - 1]);
+        q.hb = Elem<T>::widen(load_by_wave(hrow + (k * TILE + wave_off - 1), vzero));
         q.h_first = 0.0f;  // never looked at: whole tiles are not the first of a row
         q.first = false;
     };
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(64 * W * R) void scan_backward_kernel(
         // h[-1] at the start of the row
         const int64_t tw = k * TILE + wave_off;
         const bool before = k >= seg.k_lo && tw > 0 && tw < L;
-        const float loaded = Elem<T>::widen(hrow[before ? tw - 1 : 0]);
+        const float loaded = Elem<T>::widen(load_by_wave(hrow + (before ? tw - 1 : 0), vzero));
         q.hb = before ? loaded : hinit;
         // Where the part begins the row, `hinit` is what the gate gradient at t = 0 is to see,
         // which need not be the state the forward call started from (a caller that passes no

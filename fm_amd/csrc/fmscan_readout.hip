@@ -7,7 +7,23 @@ using namespace fmscan::host;
 
 namespace {
 
-constexpr int kRowDotWaves = 8;  // waves of a block that share the D rows of a slot
+// Waves of a block that share the D rows of a slot in rowdot_kernel: one where the (b, m, tile)
+// triples alone fill the GPU (a wave then walks all D rows: no sum across waves, no short-lived
+// blocks), more where they are few.
+int rowdot_waves(int64_t triples, int64_t D) {
+    int waves = 1;
+    while (waves < 8 && triples * waves < 4096 && 2 * waves <= D) waves *= 2;
+    return waves;
+}
+template <typename F>
+void with_rowdot_waves(int waves, F&& f) {
+    switch (waves) {
+        case 1: f(std::integral_constant<int, 1>{}); break;
+        case 2: f(std::integral_constant<int, 2>{}); break;
+        case 4: f(std::integral_constant<int, 4>{}); break;
+        default: f(std::integral_constant<int, 8>{}); break;
+    }
+}
 constexpr int kReadoutRows = 4;  // consecutive d per wave in the read-out kernels
 
 struct ReadoutShape {
@@ -58,10 +74,13 @@ int fmscan_readout_inv_rms(const void* states, float* inv_rms, int64_t B, int64_
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
         with_bool(vec, [&](auto vt) {
-            fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kSumSq, false, decltype(vt)::value>
-                <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>((const T*)states, nullptr, nullptr, inv_rms,
-                                                                      nullptr, nullptr, nullptr, nullptr, nullptr,
-                                                                      nullptr, (int32_t)M, (int32_t)D, L, rs.tiles, eps);
+            with_rowdot_waves(rowdot_waves(grid, D), [&](auto wt) {
+                constexpr int WV = decltype(wt)::value;
+                fmscan::rowdot_kernel<T, WV, fmscan::RowDot::kSumSq, false, decltype(vt)::value>
+                    <<<grid, 64 * WV, 0, (hipStream_t)stream>>>((const T*)states, nullptr, nullptr, inv_rms, nullptr,
+                                                                nullptr, nullptr, nullptr, nullptr, nullptr,
+                                                                (int32_t)M, (int32_t)D, L, rs.tiles, eps);
+            });
         });
     });
     return launched("read-out (inverse rms)");
@@ -138,10 +157,13 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
         using T = typename decltype(tt)::type;
         with_bool(ext_grad != nullptr, [&](auto et) {
             with_bool(vec, [&](auto vt) {
-                fmscan::rowdot_kernel<T, kRowDotWaves, fmscan::RowDot::kDot, decltype(et)::value, decltype(vt)::value>
-                    <<<grid, 64 * kRowDotWaves, 0, (hipStream_t)stream>>>(
-                        (const T*)states_n, (const T*)out_grad, (const T*)ext_grad, q, qe, inv_rms, (const T*)read,
-                        coef_out, coef_self, rms_out, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
+                with_rowdot_waves(rowdot_waves(grid, D), [&](auto wt) {
+                    constexpr int WV = decltype(wt)::value;
+                    fmscan::rowdot_kernel<T, WV, fmscan::RowDot::kDot, decltype(et)::value, decltype(vt)::value>
+                        <<<grid, 64 * WV, 0, (hipStream_t)stream>>>(
+                            (const T*)states_n, (const T*)out_grad, (const T*)ext_grad, q, qe, inv_rms, (const T*)read,
+                            coef_out, coef_self, rms_out, (int32_t)M, (int32_t)D, L, rs.tiles, 0.0f);
+                });
             });
         });
     });

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     extern __shared__ float lds[];
-    static_assert(J % NW == 0, "the waves share the loads of the J token rows evenly");
+    constexpr int SH = (J + NW - 1) / NW;  // token rows a wave loads for the block (the last waves fewer, or none)
     float* handover = lds;                    // [2][J][E / 4][64][4]: token gradients on their way down the waves
     u32x4* shared_xy = reinterpret_cast<u32x4*>(lds + 2 * J * TILE);  // [2][J][2][64]: tokens and layer_out_grad of a tile
     float* carries = lds + 2 * J * TILE + 2 * J * 2 * 64 * 4;         // [NW][Mw * J]
@@ -103,6 +103,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // of a tile are not read but made again from its gates and tokens and the one saved state
     // before the tile, as scan_backward_kernel does.
     constexpr bool REMAKE = LAYER != 2 && !PLAIN;
+    const uint32_t vzero = opaque_zero();
     struct Row {
         u32x4 a;   // out_grad, or the normalised states (LAYER)
         u32x4 h;   // saved states (PLAIN only)
@@ -131,9 +132,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         const T* __restrict__ hsrc = LAYER == 2 ? out_grad : h_saved;
         // h just before the tile (h[-1] at the start of the row): one address for the whole wave
         const T* src = tw > 0 ? hsrc + (base - 1) : (h0 != nullptr ? h0 + row : hsrc + base);
-        r.hb = *src;
+        r.hb = load_by_wave(src, vzero);
         r.h_first = T(0);
-        if constexpr (REMAKE) r.h_first = hsrc[tw > 0 ? base - 1 : base];  // no new cache line except in the first tile
+        // (no new cache line except in the first tile)
+        if constexpr (REMAKE) r.h_first = load_by_wave(hsrc + (tw > 0 ? base - 1 : base), vzero);
     };
     auto fetch_slot = [&](Slot& s, int32_t k, int32_t mi) {
         const int64_t tw = (int64_t)k * TILE;
@@ -147,13 +149,16 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         s.hbr = 0.0f;
         if constexpr (LAYER == 2) {
             s.rr = load_float_chunk<E>(rms + base + lo);
-            s.hbr = rms[base - (tw > 0 ? 1 : 0)];
+            s.hbr = load_by_wave(rms + (base - (tw > 0 ? 1 : 0)), vzero);
         }
     };
-    // the position one slot ahead of (k, mi): the next slot of the tile, else the first slot of
+    // The steps of a tile come in pairs (below), so an odd count of slots is padded with one step
+    // that only loads.
+    const int32_t mpad = (mcount + 1) & ~1;
+    // the position one step ahead of (k, mi): the next slot of the tile, else the first slot of
     // the tile before; before the first tile there is nothing: stay (the loads are not used)
     auto ahead = [&](int32_t& k, int32_t& mi) {
-        if (mi + 1 < mcount) {
+        if (mi + 1 < mpad) {
             ++mi;
         } else if (k > 0) {
             --k;
@@ -162,18 +167,18 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     };
 
     // The J token rows of the block (and the J rows of the layer's output gradient) are the same
-    // for every slot and every wave: each tile of them is loaded once per block, J / NW rows
+    // for every slot and every wave: each tile of them is loaded once per block, about J / NW rows
     // per wave, and passed through LDS, a tile ahead of its use.
     constexpr bool kSharedX = !PLAIN, kSharedY = LAYER != 0;
     struct TokenShare {
-        u32x4 x[J / NW], y[J / NW];
+        u32x4 x[SH], y[SH];
     };
     auto fetch_share = [&](TokenShare& ts, int32_t k) {
         const int64_t tw = (int64_t)k * TILE;
         const uint32_t lo = lane_elems(k);
 #pragma unroll
-        for (int s = 0; s < J / NW; ++s) {
-            const int32_t jj = w * (J / NW) + s;
+        for (int s = 0; s < SH; ++s) {
+            const int32_t jj = w * SH + s < J ? w * SH + s : J - 1;  // (a wave beyond the J rows loads the last again, unused)
             const int32_t d = d0 + jj < D ? d0 + jj : D - 1;
             const int64_t off = (b * D + d) * L + tw + lo;
             ts.x[s] = ts.y[s] = u32x4{0u, 0u, 0u, 0u};
@@ -183,17 +188,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     };
     auto publish_share = [&](const TokenShare& ts, int par) {
 #pragma unroll
-        for (int s = 0; s < J / NW; ++s) {
-            const int32_t jj = w * (J / NW) + s;
+        for (int s = 0; s < SH; ++s) {
+            const int32_t jj = w * SH + s;
+            if (jj >= J) break;
             if constexpr (kSharedX) shared_xy[((par * J + jj) * 2 + 0) * 64 + lane] = ts.x[s];
             if constexpr (kSharedY) shared_xy[((par * J + jj) * 2 + 1) * 64 + lane] = ts.y[s];
         }
     };
 
     Row rows[J];
-    Slot next_slot;
+    // The per-slot vectors of the step at work and of the step after it, which is loading, sit in
+    // two sets of registers that swap roles from step to step: handing one set over to the other
+    // at the end of a step would have to wait for every load and store in flight.
+    Slot slot_a, slot_b;
     int32_t kf = ntiles - 1, mf = 0;  // where the loads are: one step (a slot's J rows) ahead of the work
-    fetch_slot(next_slot, kf, mf);
+    fetch_slot(slot_a, kf, mf);
 #pragma unroll
     for (int j = 0; j < J; ++j) fetch_row(rows[j], kf, mf, j);
 
@@ -210,16 +219,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         TokenShare upcoming;  // the tile before this one, on its way to LDS
         if constexpr (kSharedX || kSharedY) fetch_share(upcoming, k > 0 ? k - 1 : 0);
         const bool inside = tw + lane_off < L;  // this lane's chunk lies in the row (tiles are whole chunks)
+        const bool ragged = tw + TILE > L;      // the whole wave: only the row's last tile can end early
         float dtok[J][E];
 #pragma unroll
         for (int j = 0; j < J; ++j) {
 #pragma unroll
             for (int i = 0; i < E; ++i) dtok[j][i] = 0.0f;
         }
-        for (int32_t mi = 0; mi < mcount; ++mi) {
-            const Slot cur = next_slot;
+        auto slot_step = [&](const Slot& cur, Slot& next_slot, int32_t mi) __attribute__((always_inline)) {
             ahead(kf, mf);
             fetch_slot(next_slot, kf, mf);
+            if (mi >= mcount) {  // the padding step of an odd count
+#pragma unroll
+                for (int j = 0; j < J; ++j) fetch_row(rows[j], kf, mf, j);
+                return;
+            }
 
             // per slot: gates (1 where there is no step: identity), coefficients (0 there: no gradient)
             float g[E], co[E], cs[E];
@@ -228,14 +242,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                 spread<E>(cur.co, co);
                 spread<E>(cur.cs, cs);
             }
+            if (ragged) {
 #pragma unroll
-            for (int i = 0; i < E; ++i) {
-                g[i] = inside ? g[i] : 1.0f;
-                if constexpr (LAYER != 0) {
-                    co[i] = inside ? co[i] : 0.0f;
-                    cs[i] = inside ? cs[i] : 0.0f;
+                for (int i = 0; i < E; ++i) {
+                    g[i] = inside ? g[i] : 1.0f;
+                    if constexpr (LAYER != 0) {
+                        co[i] = inside ? co[i] : 0.0f;
+                        cs[i] = inside ? cs[i] : 0.0f;
+                    }
                 }
             }
+            float keep[E];  // 1 - g: the share of a step's gradient that goes to its token
+#pragma unroll
+            for (int i = 0; i < E; ++i) keep[i] = 1.0f - g[i];
             float a = g[E - 1];
 #pragma unroll
             for (int i = E - 2; i >= 0; --i) a *= g[i];
@@ -258,27 +277,29 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
             {
 #pragma unroll
                 for (int j = 0; j < J; ++j) {
-                    const Row r = rows[j];
-                    fetch_row(rows[j], kf, mf, j);
-
-                    float carry = carry_of[j];
+                    // (unpacked before the loads of the slot after this one reuse the registers)
                     float G[E], h[E], x[E];
-                    Elem<T>::unpack(r.a, G);
+                    Elem<T>::unpack(rows[j].a, G);
                     // what stands before the tile in the row: a state, or a normalised one (the factor
                     // follows with the slot); at k == 0 the initial state itself, or nothing
-                    const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(r.hb) : 0.0f;
+                    const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(rows[j].hb) : 0.0f;
+                    [[maybe_unused]] const float h_first = Elem<T>::widen(rows[j].h_first);
                     if constexpr (LAYER == 2) {
 #pragma unroll
                         for (int i = 0; i < E; ++i) h[i] = G[i];  // G[] holds the normalised state
                     } else if constexpr (!REMAKE) {
-                        Elem<T>::unpack(r.h, h);
+                        Elem<T>::unpack(rows[j].h, h);
                     }
+                    fetch_row(rows[j], kf, mf, j);
+                    if (d0 + j >= D) continue;  // the whole wave: a row past the last d adds nothing
+
+                    float carry = carry_of[j];
                     if constexpr (LAYER != 0) {
                         float y[E];
                         Elem<T>::unpack(shared_xy[((parity * J + j) * 2 + 1) * 64 + lane], y);
 #pragma unroll
                         for (int i = 0; i < E; ++i) G[i] = __builtin_fmaf(-cs[i], G[i], co[i] * y[i]);
-                    } else {
+                    } else if (ragged) {
 #pragma unroll
                         for (int i = 0; i < E; ++i) G[i] = inside ? G[i] : 0.0f;
                     }
@@ -288,7 +309,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                         float u[E];
 #pragma unroll
                         for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], x[i], x[i]);  // as the forward kernel forms it
-                        if (first_step) u[0] = Elem<T>::widen(r.h_first);
+                        if (first_step) u[0] = h_first;
                         float fb = u[0];
 #pragma unroll
                         for (int i = 1; i < E; ++i) fb = __builtin_fmaf(g[i], fb, u[i]);
@@ -314,18 +335,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     float c = __builtin_fmaf(levels.ea, carry, eb);
                     carry = __builtin_fmaf(levels.ta, carry, tb);
                     if (lane == 0) carry_of[j] = carry;
-                    const bool counted = d0 + j < D;  // the whole wave: a row past the last d adds nothing
 #pragma unroll
                     for (int i = E - 1; i >= 0; --i) {
                         const float delta = G[i] + c;
                         c = g[i] * delta;
-                        const float hp = hprev[i];
-                        // token gradient (1 - g) * delta = delta - g * delta
-                        dtok[j][i] += PLAIN ? delta : delta - c;
-                        if (counted) {
-                            with_state[i] = __builtin_fmaf(hp, delta, with_state[i]);
-                            if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
-                        }
+                        // token gradient (1 - g) * delta
+                        if constexpr (PLAIN) dtok[j][i] += delta;
+                        else dtok[j][i] = __builtin_fmaf(keep[i], delta, dtok[j][i]);
+                        with_state[i] = __builtin_fmaf(hprev[i], delta, with_state[i]);
+                        if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
                     }
                 }
             }
@@ -354,6 +372,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(prow + i));
                 }
             }
+        };
+        for (int32_t mi = 0; mi < mpad; mi += 2) {
+            slot_step(slot_a, slot_b, mi);
+            slot_step(slot_b, slot_a, mi + 1);
         }
 
         // the shared rows of the tile before: in place once the barriers below have been passed
