@@ -32,6 +32,15 @@ __device__ __forceinline__ uint32_t opaque_zero() {
 template <typename V>
 __device__ __forceinline__ V load_by_wave(const V* p, uint32_t zero) { return p[zero]; }
 
+// All vector loads and stores issued so far have completed. For use just before a loop that
+// prefetches: the compiler puts one wait at the loop's head for both ways into it, and sizes it
+// for the way that needs the longer wait. From the code before the loop, where the loads the
+// first pass needs are the youngest in flight, that is a wait for everything; inside the loop
+// it then waits for everything too, on every pass, the prefetch and the stores of the pass
+// before included. With nothing in flight on entry the count at the head is the one the loop
+// itself needs. (s_waitcnt vmcnt(0); the other counters at their maxima: not waited for.)
+__device__ __forceinline__ void wait_for_loads() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+
 // ---- 16 bytes <-> E fp32 values -------------------------------------------------
 // One lane always moves 16 bytes per tensor per tile: 4 fp32 or 8 fp16/bf16
 // consecutive sequence positions. Narrow types are widened to fp32 on load and

@@ -61,6 +61,7 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
     const int32_t lane_off = lane * E;
     auto d_of = [&](int j) { return d0 + j < D ? d0 + j : D - 1; };  // a row past D is loaded as D - 1 and dropped
+    auto counted = [&](int j) { return d0 + j < D; };                // the same for the whole wave
 
     float carry[J];
 #pragma unroll
@@ -76,28 +77,41 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
         u32x4 g;
         u32x4 x[J];
     };
-    auto fetch = [&](Loads& q, int32_t k) {  // k beyond the last tile: the last tile again (not used)
+    // k beyond the last tile: the last tile again (not used)
+    auto fetch_gates = [&](Loads& q, int32_t k) {
         k = k < ntiles ? k : ntiles - 1;
-        const int64_t tw = (int64_t)k * TILE;
-        const uint32_t lo = lane_elems(k);
-        q.g = load16<T, false>(gates + bm * L + tw + lo);
-#pragma unroll
-        for (int j = 0; j < J; ++j) q.x[j] = load16<T, false>(tokens + (b * D + d_of(j)) * L + tw + lo);
+        q.g = load16<T, false>(gates + bm * L + (int64_t)k * TILE + lane_elems(k));
+    };
+    auto fetch_tokens = [&](Loads& q, int32_t k, int j) {
+        k = k < ntiles ? k : ntiles - 1;
+        q.x[j] = load16<T, false>(tokens + (b * D + d_of(j)) * L + (int64_t)k * TILE + lane_elems(k));
     };
 
-    Loads next;
-    fetch(next, 0);
+    // The loads run a tile ahead, each into the registers it was just unpacked from: a second set
+    // of registers handed over at the end of a tile would make that hand-over wait for the
+    // tile's stores as well.
+    Loads q;
+    fetch_gates(q, 0);
+#pragma unroll
+    for (int j = 0; j < J; ++j) fetch_tokens(q, 0, j);
     int parity = 0;
-    for (int32_t k = 0; k < ntiles; ++k) {
-        const Loads cur = next;
-        fetch(next, k + 1);
+    wait_for_loads();
+    // One tile. `whole`: it lies wholly inside the row and nothing is tested per lane, so that
+    // every pass of the loop over such tiles issues the same loads and stores, and the waits for
+    // loads can be counted past the stores in flight. The last tile of a row that is not a
+    // whole number of tiles is done after the loop, with the tests.
+    auto tile = [&](int32_t k, auto whole) __attribute__((always_inline)) {
+        constexpr bool WHOLE_TILE = decltype(whole)::value;
         const int64_t tw = (int64_t)k * TILE;
-        const bool inside = tw + lane_off < L;  // this lane's chunk lies in the row (tiles are whole chunks)
+        const bool inside = WHOLE_TILE || tw + lane_off < L;  // this lane's chunk lies in the row (tiles are whole chunks)
 
         float g[E];
-        Elem<T>::unpack(cur.g, g);
+        Elem<T>::unpack(q.g, g);
+        fetch_gates(q, k + 1);
+        if constexpr (!WHOLE_TILE) {
 #pragma unroll
-        for (int i = 0; i < E; ++i) g[i] = inside ? g[i] : 1.0f;
+            for (int i = 0; i < E; ++i) g[i] = inside ? g[i] : 1.0f;
+        }
         float a = g[0];
 #pragma unroll
         for (int i = 1; i < E; ++i) a *= g[i];
@@ -110,7 +124,8 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
 #pragma unroll
         for (int j = 0; j < J; ++j) {
             float u[E];
-            Elem<T>::unpack(cur.x[j], u);
+            Elem<T>::unpack(q.x[j], u);
+            fetch_tokens(q, k + 1, j);
 #pragma unroll
             for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], u[i], u[i]);  // (1 - g) x, one rounding
             float bb = u[0];
@@ -128,8 +143,12 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
                 o[i] = h;
             }
             held[j] = Elem<T>::pack(o);
-            if (d0 + j < D) {              // the whole wave
-                if constexpr (!WHOLE) store_chunk<T, true>(states_n + (bm * D + d0 + j) * L, tw + lane_off, L, held[j]);
+            if (counted(j)) {
+                if constexpr (!WHOLE) {
+                    if (inside)
+                        __builtin_nontemporal_store(held[j], reinterpret_cast<u32x4*>(states_n + (bm * D + d0 + j) * L +
+                                                                                      tw + lane_off));
+                }
                 Elem<T>::unpack(held[j], o);  // the norm sees the states as they would be stored
 #pragma unroll
                 for (int i = 0; i < E; ++i) sumsq[i] = __builtin_fmaf(o[i], o[i], sumsq[i]);
@@ -150,14 +169,14 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
             if constexpr (WHOLE) {
                 s = 1.0f / __builtin_sqrtf(s / (float)D + eps);
                 scale[parity][e] = s;
-                if (tw + e < L) inv_rms[bm * L + tw + e] = s;
+                if (WHOLE_TILE || tw + e < L) inv_rms[bm * L + tw + e] = s;
             } else {
-                if (tw + e < L) inv_rms[(bm * DB + db) * L + tw + e] = s;
+                if (WHOLE_TILE || tw + e < L) inv_rms[(bm * DB + db) * L + tw + e] = s;
             }
         }
         if constexpr (!WHOLE) {
             parity ^= 1;  // the other buffer next: no wave writes this one again before all have read it
-            continue;
+            return;
         }
         __syncthreads();
         float r[E];
@@ -166,18 +185,24 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
             const float4 v = *reinterpret_cast<const float4*>(&scale[parity][lane_off + i]);
             r[i] = v.x; r[i + 1] = v.y; r[i + 2] = v.z; r[i + 3] = v.w;
         }
+        if (inside) {
 #pragma unroll
-        for (int j = 0; j < J; ++j) {
-            if (d0 + j < D) {
-                float o[E];
-                Elem<T>::unpack(held[j], o);
+            for (int j = 0; j < J; ++j) {
+                if (counted(j)) {
+                    float o[E];
+                    Elem<T>::unpack(held[j], o);
 #pragma unroll
-                for (int i = 0; i < E; ++i) o[i] *= r[i];
-                store_chunk<T, true>(states_n + (bm * D + d0 + j) * L, tw + lane_off, L, Elem<T>::pack(o));
+                    for (int i = 0; i < E; ++i) o[i] *= r[i];
+                    __builtin_nontemporal_store(Elem<T>::pack(o),
+                                                reinterpret_cast<u32x4*>(states_n + (bm * D + d0 + j) * L + tw + lane_off));
+                }
             }
         }
         parity ^= 1;
-    }
+    };
+    const int32_t whole_tiles = (int32_t)(L / TILE);
+    for (int32_t k = 0; k < whole_tiles; ++k) tile(k, std::true_type{});
+    if (whole_tiles < ntiles) tile(whole_tiles, std::false_type{});
 }
 
 // inv_rms[r][t] = rsqrt(sum_g partial[r][g][t] / D + eps) for the (B, M, G, L) partial sums of
