@@ -197,6 +197,37 @@ def test_layer_at_the_benchmark_shape(scan):
         check_all(f"fm_memory bench shape, batch element {b}", got, want, tols)
 
 
+def test_layer_with_more_than_2_31_state_elements(scan):
+    """(B, L, M, D) = (9, 65536, 32, 128): 2^31 + 2^28 elements of the states, which the reference's
+    32-bit indices could not address (fm_scan.cuh:76-82). Batch elements are independent and every
+    kernel of the layer sums in a fixed order, so the last batch element, all of it beyond element
+    2^31, must come out bit for bit as a layer call on that batch element alone does."""
+    B, L, M, D, dt = 9, 65536, 32, 128, torch.bfloat16
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    alpha = torch.softmax(rn(B, L, M), -1).to(dt)
+    us = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt)
+    osc = torch.rand(B, L, 1, device=DEV, generator=gen).to(dt)
+    inp = rn(B, L, D).to(dt)
+    w_out = rn(B, L, D).to(dt)
+
+    def run(sl):
+        leaves = [t[sl].clone().requires_grad_() for t in (alpha, us, osc, inp)]
+        y, mem = scan.fm_memory(*leaves)
+        (y.float() * w_out[sl].float()).sum().backward()
+        return [y.detach(), mem.detach()] + [t.grad for t in leaves]
+
+    whole = run(slice(0, B))
+    assert whole[1].numel() > 1 << 31
+    last = [t[B - 1:].clone() for t in whole]
+    del whole
+    torch.cuda.empty_cache()
+    alone = run(slice(B - 1, B))
+    for name, a, b in zip(("output", "memory_states", "d_alpha", "d_update_scale", "d_output_scale", "d_inputs"),
+                          last, alone):
+        assert torch.equal(a, b), name
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_forward_scan_and_norm_in_one_kernel(scan, dtype):
     """fmscan_forward_normed (through the C interface) against the float64 oracle and against the three

@@ -209,6 +209,46 @@ def test_shapes_and_variants(scan, dtype, waves, plain):
         check(tag + " gate grad", dg, gg, TOL[dtype])
 
 
+def test_more_than_2_31_elements(scan):
+    """The reference indexes with 32-bit ints (fm_scan.cuh:76-82: N < 2^31); here offsets are 64-bit.
+    Rows that lie beyond element 2^31 of a problem must come out exactly as the same rows of a small
+    problem of their own do (same kernel, same arithmetic per row: bit-exact), fold mapping and
+    Factorization-Memory shape (the kernel with the sums inside) alike."""
+    dt = torch.bfloat16
+    gen = gpu_gen(3)
+    # fold mapping: 2^17 + 8 rows of 16384 = 2^31 + 131072 elements per (rows, 1, 1, L) tensor
+    rows, L, tail = (1 << 17) + 8, 16384, 8
+    g = torch.rand(rows, 1, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(rows, 1, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(rows, 1, 1, L, device=DEV, generator=gen).to(dt)
+    assert G.numel() > 1 << 31
+    out, dx, dg = run_fwd_bwd(scan, g, x, G)
+    o2, dx2, dg2 = run_fwd_bwd(scan, g[-tail:].contiguous(), x[-tail:].contiguous(), G[-tail:].contiguous())
+    assert torch.equal(out[-tail:], o2) and torch.equal(dx[-tail:], dx2) and torch.equal(dg[-tail:], dg2)
+    h_ref, tg, gg = oracle_rows(g, x, G, out, [rows - 1])
+    check("states of the last row", out[rows - 1:], h_ref, TOL[dt])
+    check("token gradient of the last row", dx[rows - 1:], tg, TOL[dt])
+    check("gate gradient of the last row", dg[rows - 1:], gg, TOL[dt])
+    del g, x, G, out, dx, dg, o2, dx2, dg2
+    torch.cuda.empty_cache()
+
+    # (B, M, D, L) = (9, 32, 128, 65536): 2^31 + 2^28 elements; the last batch element lies beyond 2^31
+    B, M, D, L = 9, 32, 128, 65536
+    g = torch.rand(B, M, L, device=DEV, generator=gen).to(dt)
+    x = torch.randn(B, D, L, device=DEV, generator=gen).to(dt)
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    assert G.numel() > 1 << 31
+    z = torch.zeros(B, M, D, dtype=dt, device=DEV)
+    states = torch.empty(B, M, D, L, dtype=dt, device=DEV)
+    scan.fm_scan_forward(g, x, z, states)
+    d_gates, d_tokens = scan.fm_scan_backward_reduced(g, G, z, states, x)
+    s1 = torch.empty(1, M, D, L, dtype=dt, device=DEV)
+    scan.fm_scan_forward(g[-1:].contiguous(), x[-1:].contiguous(), z[-1:], s1)
+    assert torch.equal(states[-1:], s1)
+    dg1, dt1 = scan.fm_scan_backward_reduced(g[-1:].contiguous(), G[-1:].contiguous(), z[-1:], s1, x[-1:].contiguous())
+    assert torch.equal(d_gates[-1:], dg1) and torch.equal(d_tokens[-1:], dt1)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_unaligned_pointers_take_the_element_path(scan, dtype):
     """Tensors that start one element past a 16-byte boundary (still contiguous)."""
