@@ -510,6 +510,10 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
     dev, dtype = states_n.device, states_n.dtype
     if out_grad is not None:
         out_grad = out_grad.contiguous()
+    if states_n.numel() == 0:  # no batch element, slot, channel or step: nothing flows back
+        zeros32 = torch.zeros((B, M, L), dtype=torch.float32, device=dev)
+        return (zeros32.unsqueeze(2), torch.zeros((B, D, L), dtype=dtype, device=dev),
+                torch.zeros((B, M, D), dtype=dtype, device=dev) if want_initial_state_grad else None, zeros32)
 
     if ext_grad is None and _reduced_ok(gates, tokens, states_n, states_n) and _aligned(read, out_grad):
         code = _dtype_code(states_n)

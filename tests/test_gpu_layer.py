@@ -197,6 +197,31 @@ def test_layer_at_the_benchmark_shape(scan):
         check_all(f"fm_memory bench shape, batch element {b}", got, want, tols)
 
 
+@pytest.mark.parametrize("shape", [(0, 64, 4, 8), (2, 64, 4, 0)])
+def test_empty_problems_pass_through(scan, shape):
+    """No batch element, or no channel: nothing to launch (the C ABI rejects empty problems, the
+    Python side never calls it with one), the results are empty tensors of the right shapes and the
+    gradients of what is not empty are zero."""
+    B, L, M, D = shape
+    dt = torch.bfloat16
+    g = torch.rand(B, M, L, device=DEV).to(dt).requires_grad_()
+    x = torch.randn(B, D, L, device=DEV).to(dt).requires_grad_()
+    states = scan.fm_scan(g, x)
+    assert tuple(states.shape) == (B, M, D, L)
+    states.float().sum().backward()
+    assert tuple(g.grad.shape) == (B, M, L) and tuple(x.grad.shape) == (B, D, L)
+    assert not g.grad.float().abs().sum().item() and not x.grad.float().abs().sum().item()
+    alpha = torch.softmax(torch.randn(B, L, M, device=DEV), -1).to(dt).requires_grad_()
+    us = torch.rand(B, L, 1, device=DEV).to(dt).requires_grad_()
+    osc = torch.rand(B, L, 1, device=DEV).to(dt).requires_grad_()
+    inp = torch.randn(B, L, D, device=DEV).to(dt).requires_grad_()
+    y, mem = scan.fm_memory(alpha, us, osc, inp)
+    assert tuple(y.shape) == (B, L, D) and tuple(mem.shape) == (B, M, D, L)
+    y.float().sum().backward()
+    for t in (alpha, us, osc, inp):
+        assert t.grad is not None and t.grad.shape == t.shape and not t.grad.float().abs().sum().item()
+
+
 def test_layer_with_more_than_2_31_state_elements(scan):
     """(B, L, M, D) = (9, 65536, 32, 128): 2^31 + 2^28 elements of the states, which the reference's
     32-bit indices could not address (fm_scan.cuh:76-82). Batch elements are independent and every
