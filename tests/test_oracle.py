@@ -394,6 +394,29 @@ def test_norm_gradient_with_one_channel_is_all_cancellation():
     assert grad_from_stored(h4, 1e-6, 2.0 ** -8) < 1e-2      # D = 4: fine with the same rounding
 
 
+def test_single_step_gate_gradient_vanishes_under_the_norm():
+    """L = 1 without an initial state: the one state is (1 - g) x, the norm makes the output blind to
+    its length, so the gradient that reaches the gate (and with it update_scale) is what eps lets
+    through: zero up to eps / mean(h^2), a difference of terms of order one. Against a reference that
+    small, a normwise error says nothing; random-shape runs on the GPU meet their tolerance everywhere
+    but here and at a few entries of very short sequences that cancel the same way."""
+    rng = np.random.default_rng(11)
+    B, L, M, D = 2, 1, 5, 16
+    alpha = rng.random((B, L, M)) * 0.8 + 0.1
+    us, osc = rng.random((B, L, 1)) * 0.8 + 0.1, rng.random((B, L, 1)) + 0.5
+    inp, w_out = rng.standard_normal((B, L, D)), rng.standard_normal((B, L, D))
+    for eps in (1e-4, 1e-8):
+        g = O.memory_backward(alpha, us, osc, inp, w_out, None, None, True, eps)
+        assert np.abs(g["d_update_scale"]).max() < 200 * eps * np.abs(g["d_output_scale"]).max()  # eps / mean(h^2), h = (1 - g) x
+    # with a second step the first one's gate also sees what arrives from the future: not small any more
+    L = 2
+    alpha = rng.random((B, L, M)) * 0.8 + 0.1
+    us, osc = rng.random((B, L, 1)) * 0.8 + 0.1, rng.random((B, L, 1)) + 0.5
+    inp, w_out = rng.standard_normal((B, L, D)), rng.standard_normal((B, L, D))
+    g = O.memory_backward(alpha, us, osc, inp, w_out, None, None, True, 1e-8)
+    assert np.abs(g["d_update_scale"]).max() > 1e-3 * np.abs(g["d_output_scale"]).max()
+
+
 # ------------------------------------------------------------------ compiled oracle and port
 
 @pytest.mark.parametrize("plain", [False, True])
