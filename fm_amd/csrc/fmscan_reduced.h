@@ -59,6 +59,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     float* handover = lds;                    // [2][J][E / 4][64][4]: token gradients on their way down the waves
     u32x4* shared_xy = reinterpret_cast<u32x4*>(lds + 2 * J * TILE);  // [2][J][2][64]: tokens and layer_out_grad of a tile
     float* carries = lds + 2 * J * TILE + 2 * J * 2 * 64 * 4;         // [NW][Mw * J]
+    float* staging = carries + NW * Mw * J;                          // [NW][TILE], 8-element chunks only: see the partials' stores
 
     const int lane = threadIdx.x & 63;
     const int w = uniform((int)(threadIdx.x >> 6));
@@ -364,12 +365,32 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
                 for (int i = 0; i < E; ++i) dgate[i] = with_state[i] - with_token[i];
             }
-            if (inside) {
-                float* __restrict__ prow = gate_partial + ((b * M + m0 + mi) * NG + grp) * L + tw + lane_off;
+            float* __restrict__ ptile = gate_partial + ((b * M + m0 + mi) * NG + grp) * L + tw;
+            if constexpr (E == 4) {
+                if (inside) {
+                    const u32x4 v = {f2u(dgate[0]), f2u(dgate[1]), f2u(dgate[2]), f2u(dgate[3])};
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(ptile + lane_off));
+                }
+            } else {
+                // A lane holds 8 consecutive floats, 32 bytes: stored as they are, each of the two store
+                // instructions would write 16 of every 32 bytes over 2 KiB. Through LDS (private to the wave,
+                // whose LDS operations complete in order) every instruction writes 1 KiB without gaps.
+                static_assert(E == 4 || E == 8, "chunks of 4 or 8 elements");
+                float* mine = staging + w * TILE;
+                *reinterpret_cast<float4*>(mine + lane_off) = make_float4(dgate[0], dgate[1], dgate[2], dgate[3]);
+                *reinterpret_cast<float4*>(mine + lane_off + 4) = make_float4(dgate[4], dgate[5], dgate[6], dgate[7]);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const int32_t valid = L - tw < TILE ? (int32_t)(L - tw) : TILE;  // whole chunks
 #pragma unroll
-                for (int i = 0; i < E; i += 4) {
-                    const u32x4 v = {f2u(dgate[i]), f2u(dgate[i + 1]), f2u(dgate[i + 2]), f2u(dgate[i + 3])};
-                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(prow + i));
+                for (int half = 0; half < 2; ++half) {
+                    const int32_t at = half * (TILE / 2) + lane * 4;
+                    const float4 v = *reinterpret_cast<const float4*>(mine + at);
+                    if (at < valid) {
+                        const u32x4 u = {f2u(v.x), f2u(v.y), f2u(v.z), f2u(v.w)};
+                        __builtin_nontemporal_store(u, reinterpret_cast<u32x4*>(ptile + at));
+                    }
                 }
             }
         };

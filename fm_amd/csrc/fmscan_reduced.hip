@@ -73,7 +73,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     const size_t tile = (size_t)(16 / pb.esize) * 64;
     const int64_t Mw = (M + kReducedWaves - 1) / kReducedWaves;  // slots per wave
     const size_t lds = (2 * kReducedGroup * tile + 2 * kReducedGroup * 2 * 64 * 4 +
-                        (size_t)kReducedWaves * (size_t)Mw * kReducedGroup) * sizeof(float);
+                        (size_t)kReducedWaves * (size_t)Mw * kReducedGroup + (size_t)kReducedWaves * tile) * sizeof(float);
     if (lds > kMaxDynamicLds)
         return fail(FMSCAN_E_SHAPE, "%s: M = %lld needs %zu bytes of LDS (limit %u)", who, (long long)M, lds,
                     kMaxDynamicLds);
