@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint, c_void_p
 
 from . import build as _build
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 FLAG_PLAIN = 0x1
@@ -85,6 +85,8 @@ def load() -> ctypes.CDLL:
                                     c_void_p, c_size_t, c_void_p]
     lib.fmscan_reduced_groups.restype = c_int64
     lib.fmscan_reduced_groups.argtypes = [c_int64]
+    lib.fmscan_sum_groups.restype = c_int
+    lib.fmscan_sum_groups.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p]
     lib.fmscan_backward_reduced.restype = c_int
     lib.fmscan_backward_reduced.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     lib.fmscan_backward_layer.restype = c_int

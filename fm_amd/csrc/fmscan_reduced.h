@@ -446,4 +446,31 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     }
 }
 
+// out[r, t] = sum over g of partial[r, g, t], rounded once to T: the pass that follows the kernel above
+// when the caller wants d_gates itself (reference fm/scan/fm_scan.py:76, there a torch.sum over a
+// (B, M, D, L) tensor). A thread takes V consecutive t (V = 4: 16-byte loads) of one r.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void sum_groups_kernel(const float* __restrict__ partial, T* __restrict__ out,
+                                                         int64_t rows, int32_t G, int64_t L) {
+    const int64_t per_row = (L + V - 1) / V;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * per_row) return;
+    const int64_t r = i / per_row, t = (i - r * per_row) * V;
+    const float* __restrict__ p = partial + r * G * L + t;
+    float acc[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = 0.0f;
+#pragma unroll 8
+    for (int32_t g = 0; g < G; ++g) {  // in the order of the groups: run-to-run identical
+        if constexpr (V == 4) {
+            const float4 x = *reinterpret_cast<const float4*>(p + (int64_t)g * L);
+            acc[0] += x.x; acc[1] += x.y; acc[2] += x.z; acc[3] += x.w;
+        } else {
+            acc[0] += p[(int64_t)g * L];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < V; ++v) out[r * L + t + v] = (T)acc[v];
+}
+
 }  // namespace fmscan

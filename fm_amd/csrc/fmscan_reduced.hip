@@ -128,4 +128,33 @@ int fmscan_backward_layer(const void* gates, const void* states_n, const float* 
                             out_grad, rms, B, M, D, L, dtype, flags, stream);
 }
 
+int fmscan_sum_groups(const float* partial, int64_t G, void* out, int64_t rows, int64_t L, int dtype,
+                      void* stream) {
+    const char* who = "fmscan_sum_groups";
+    if (!partial || !out) return fail(FMSCAN_E_NULL, "%s: partial and out must not be NULL", who);
+    if (rows < 1 || L < 1 || G < 1 || G > INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: rows, G, L must be >= 1 and G fit 32 bits (got %lld, %lld, %lld)", who,
+                    (long long)rows, (long long)G, (long long)L);
+    if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16)
+        return fail(FMSCAN_E_DTYPE, "%s: unknown dtype %d", who, dtype);
+    const int esize = dtype == FMSCAN_DTYPE_F32 ? 4 : 2;
+    if ((__int128)rows * G * L * 4 > (__int128)INT64_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: rows * G * L is too large", who);
+    if (overlap({"out", out, rows * L * esize}, {"partial", partial, rows * G * L * 4}))
+        return fail(FMSCAN_E_ALIAS, "%s: out overlaps partial", who);
+    const bool vec = L % 4 == 0 && aligned16(partial);
+    const __int128 threads = (__int128)rows * (vec ? L / 4 : L);
+    if ((threads + 255) / 256 > (__int128)INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: rows * L is too large for one launch", who);
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        if (vec)
+            fmscan::sum_groups_kernel<T, 4><<<grid, 256, 0, (hipStream_t)stream>>>(partial, (T*)out, rows, (int32_t)G, L);
+        else
+            fmscan::sum_groups_kernel<T, 1><<<grid, 256, 0, (hipStream_t)stream>>>(partial, (T*)out, rows, (int32_t)G, L);
+    });
+    return launched(who);
+}
+
 }  // extern "C"

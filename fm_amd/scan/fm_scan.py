@@ -237,8 +237,21 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
                 None if initial_state is None else initial_state.data_ptr(),
                 None if initial_state_grad is None else initial_state_grad.data_ptr(),
                 B, M, D, L, code, _lib.FLAG_PLAIN if plain else 0, stream))
-    d_gates = partial.sum(dim=2).to(gates.dtype)  # the few groups of d, still in float32
-    return d_gates, d_tokens
+    return _sum_groups(partial, gates.dtype), d_tokens
+
+
+def _sum_groups(partial, dtype):
+    """(B, M, L) of `dtype` from the float32 (B, M, G, L) partials of the gates' gradient: their sum over
+    G (what the reference does with torch.sum over a (B, M, D, L) tensor, fm_scan.py:76), rounded once."""
+    B, M, G, L = partial.shape
+    if G == 1 and dtype == torch.float32:
+        return partial.squeeze(2)
+    out = torch.empty((B, M, L), dtype=dtype, device=partial.device)
+    if out.numel():
+        with _on_device(partial.device):
+            _lib.check(_raw.fmscan_sum_groups(partial.data_ptr(), G, out.data_ptr(), B * M, L, _dtype_code(out),
+                                                torch.cuda.current_stream(partial.device).cuda_stream))
+    return out
 
 
 class FM_Scan(torch.autograd.Function):
@@ -578,8 +591,7 @@ class FM_Layer(torch.autograd.Function):
             return None, None, None, None, None, None
         partial, d_tokens, d_h0, q = _layer_gradients(gates, tokens, states, initial_state, read, normed,
                                                       inv_rms, out_grad, ext_grad, ctx.needs_input_grad[2])
-        d_gates = partial.sum(dim=2) if partial.shape[2] > 1 else partial.squeeze(2)
-        return d_gates.to(gates.dtype), d_tokens, d_h0, q.to(gates.dtype), None, None
+        return _sum_groups(partial.contiguous(), gates.dtype), d_tokens, d_h0, q.to(gates.dtype), None, None
 
 
 class FM_Memory(torch.autograd.Function):
@@ -631,7 +643,7 @@ class FM_Memory(torch.autograd.Function):
         d_update_scale, d_output_scale = torch.empty_like(update_scale), torch.empty_like(output_scale)
         if partial.shape[2] > 64:
             # many groups of d: the finishing kernel walks them one by one, a reduction does better
-            partial = partial.sum(dim=2, keepdim=True)
+            partial = _sum_groups(partial.contiguous(), torch.float32).unsqueeze(2)
         partial = partial.contiguous()
         if alpha.numel():
             with _on_device(dev):

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FMSCAN_ABI_VERSION 4
+#define FMSCAN_ABI_VERSION 5
 
 /* element type of every tensor in one call (reference fm_scan.cuh:333-342) */
 #define FMSCAN_DTYPE_F32  0
@@ -185,6 +185,11 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
  * flags: only FMSCAN_FLAG_PLAIN.
  */
 int64_t fmscan_reduced_groups(int64_t D);
+/* out[r, t] = sum over g of partial[r, g, t] for float32 partial (rows, G, L), rounded once to
+ * the call's dtype: d_gates (B, M, L) from gate_grad_partial with rows = B * M (the reference's
+ * torch.sum at fm/scan/fm_scan.py:76). Groups are added in their order: deterministic. */
+int fmscan_sum_groups(const float* partial, int64_t G, void* out, int64_t rows, int64_t L, int dtype,
+                      void* stream);
 int fmscan_backward_reduced(const void* gates, const void* out_grad, const void* first_prop_grad,
                             void* token_grad,
                             const void* cached_output, const void* input_tokens,

@@ -29,7 +29,8 @@ def test_header_declares_the_expected_entry_points():
                                     "fmscan_forward_static", "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
                                     "fmscan_layer_prepare", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
-                                    "fmscan_reduced_groups", "fmscan_sumsq_finish", "fmscan_sumsq_groups", "fmscan_swap_last_two",
+                                    "fmscan_reduced_groups", "fmscan_sum_groups", "fmscan_sumsq_finish", "fmscan_sumsq_groups",
+                                    "fmscan_swap_last_two",
                                     "fmscan_workspace_bytes"]
 
 
@@ -243,3 +244,15 @@ def test_streaming_probe_library_rejects_what_it_does_not_cover():
     assert f(a, b, 4, 1024, 1, 1, 2, None) == -1           # a stream count it has no kernel for
     assert f(a, b, 4, 1024, 3, 2, 3, None) == -1           # a prefetch depth it has no kernel for
     assert f(a + 8, b, 4, 1024, 3, 2, 2, None) == -1       # not 16-byte aligned
+
+
+def test_rejected_sum_groups_arguments(lib):
+    f = lib.fmscan_sum_groups
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                  ctypes.c_void_p]
+    a, b = 1 << 30, 1 << 44
+    assert f(None, 4, b, 8, 64, 2, None) == -1            # FMSCAN_E_NULL
+    assert f(a, 0, b, 8, 64, 2, None) == -2               # FMSCAN_E_SHAPE: no group
+    assert f(a, 4, b, 8, 64, 7, None) == -3               # FMSCAN_E_DTYPE
+    assert f(a, 4, a + 64, 8, 64, 2, None) == -5          # FMSCAN_E_ALIAS: out inside partial

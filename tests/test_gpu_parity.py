@@ -467,6 +467,25 @@ def test_backward_with_sums_inside(scan, dtype, plain):
         check(tag + " vs two-tensor route (tokens)", d_x, dx.sum(dim=1).double().cpu().numpy(), 2 * TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_sum_of_the_gate_gradient_partials(scan, dtype):
+    """fmscan_sum_groups through the C ABI: the (rows, G, L) float32 partials added over G in float32 and
+    rounded once, for rows of whole 16-byte vectors and not, one group and many; twice the same bits."""
+    lib = scan.module
+    stream = torch.cuda.current_stream().cuda_stream
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    for rows, G, L in ((6, 32, 2048), (3, 5, 1001), (2, 1, 64), (1, 130, 7)):
+        partial = torch.randn(rows, G, L, device=DEV, generator=gpu_gen(rows + G + L))
+        out = torch.empty(rows, L, dtype=dtype, device=DEV)
+        assert lib.fmscan_sum_groups(partial.data_ptr(), G, out.data_ptr(), rows, L, code, stream) == 0
+        want = partial.double().sum(dim=1)
+        assert torch.equal(out, want.to(dtype)) or float((out.double() - want).abs().max()) <= (
+            2e-6 if dtype == torch.float32 else 2.0 ** -8) * float(want.abs().max())
+        again = torch.empty_like(out)
+        assert lib.fmscan_sum_groups(partial.data_ptr(), G, again.data_ptr(), rows, L, code, stream) == 0
+        assert torch.equal(out, again)
+
+
 def test_backward_with_sums_inside_is_deterministic(scan):
     B, M, D, L, dt = 2, 8, 24, 2048, torch.bfloat16
     gen = gpu_gen(21)
