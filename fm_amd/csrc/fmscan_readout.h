@@ -292,6 +292,45 @@ __global__ __launch_bounds__(256) void swap_last_two_pairs_kernel(const uint16_t
                 (uint32_t)tile[2 * pair][j] | ((uint32_t)tile[2 * pair + 1][j] << 16);
 }
 
+// The same for 2-byte elements when R and C are multiples of 8 and both pointers 16-byte aligned:
+// every lane moves 8 neighbouring elements (16 bytes) on both sides, 8 lanes per 128-byte run of a
+// 64 x 64 tile; between the two, each lane gathers its 8 elements of one column from LDS.
+__global__ __launch_bounds__(256) void swap_last_two_wide_kernel(const uint16_t* __restrict__ src,
+                                                                 uint16_t* __restrict__ dst, int64_t R, int64_t C,
+                                                                 int32_t tiles_c, int32_t tiles_r) {
+    constexpr int PITCH = 66;  // elements: rows of 33 words, so that the gather below meets each bank at most twice
+    __shared__ __attribute__((aligned(4))) uint16_t tile[64 * PITCH];
+    const int64_t per_b = (int64_t)tiles_c * tiles_r;
+    const int64_t b = blockIdx.x / per_b;
+    const int64_t rest = blockIdx.x - b * per_b;
+    const int64_t r0 = (rest / tiles_c) * 64, c0 = (rest % tiles_c) * 64;
+    const uint16_t* __restrict__ s = src + b * R * C;
+    uint16_t* __restrict__ d = dst + b * R * C;
+    const int group = threadIdx.x & 7, line = threadIdx.x >> 3;  // 8 lanes of 16 bytes per run, 32 runs per pass
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int i = line + 32 * pass;
+        if (r0 + i < R && c0 + 8 * group < C) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(s + (r0 + i) * C + c0 + 8 * group);
+            uint32_t* row = reinterpret_cast<uint32_t*>(&tile[i * PITCH + 8 * group]);  // 4-byte aligned only
+            row[0] = v.x; row[1] = v.y; row[2] = v.z; row[3] = v.w;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int j = line + 32 * pass;  // the column of the tile this lane writes a run of
+        if (c0 + j < C && r0 + 8 * group < R) {
+            uint32_t v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                v[k] = (uint32_t)tile[(8 * group + 2 * k) * PITCH + j] |
+                       ((uint32_t)tile[(8 * group + 2 * k + 1) * PITCH + j] << 16);
+            *reinterpret_cast<u32x4*>(d + (c0 + j) * R + r0 + 8 * group) = u32x4{v[0], v[1], v[2], v[3]};
+        }
+    }
+}
+
 // gates[b, m, t] = 1 - alpha[b, t, m] * update_scale[b, t], read[b, m, t] = alpha[b, t, m] *
 // output_scale[b, t] (reference fm_scan.py:116,118-119,130: two products, two transposed
 // copies and a subtraction). 64 x 64 tiles of (t, m) through LDS; float32 arithmetic, one

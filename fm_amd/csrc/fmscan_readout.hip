@@ -296,7 +296,10 @@ int fmscan_swap_last_two(const void* src, void* dst, int64_t B, int64_t R, int64
     if (overlap({"dst", dst, bytes}, {"src", src, bytes}))
         return fail(FMSCAN_E_ALIAS, "fmscan_swap_last_two: dst overlaps src");
     const unsigned grid = (unsigned)(B * tiles_r * tiles_c);
-    if (element_size == 2 && R % 2 == 0 && C % 2 == 0 && ((uintptr_t)src & 3u) == 0 && ((uintptr_t)dst & 3u) == 0)
+    if (element_size == 2 && R % 8 == 0 && C % 8 == 0 && aligned16(src) && aligned16(dst))
+        fmscan::swap_last_two_wide_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, (uint16_t*)dst, R, C, (int32_t)tiles_c, (int32_t)tiles_r);
+    else if (element_size == 2 && R % 2 == 0 && C % 2 == 0 && ((uintptr_t)src & 3u) == 0 && ((uintptr_t)dst & 3u) == 0)
         fmscan::swap_last_two_pairs_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
             (const uint16_t*)src, (uint16_t*)dst, R, C, (int32_t)tiles_c, (int32_t)tiles_r);
     else if (element_size == 2)

@@ -753,7 +753,8 @@ def test_swap_last_two_is_exact(scan):
     for shape, dt in [((2, 5, 7), torch.float32), ((3, 64, 64), torch.bfloat16), ((1, 1000, 33), torch.float16),
                       ((2, 129, 2048), torch.bfloat16), ((1, 1, 1), torch.float32),
                       ((2, 130, 2048), torch.bfloat16), ((3, 2048, 32), torch.float16), ((1, 2, 2), torch.bfloat16),
-                      ((2, 300, 258), torch.bfloat16)]:
+                      ((2, 300, 258), torch.bfloat16), ((2, 136, 200), torch.bfloat16), ((1, 8, 8), torch.float16),
+                      ((2, 2048, 128), torch.bfloat16), ((3, 72, 2056), torch.float16)]:
         t = torch.randn(*shape, device=DEV).to(dt)
         assert torch.equal(_swap_last_two(t), t.transpose(1, 2).contiguous()), (shape, dt)
 
