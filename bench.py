@@ -259,7 +259,7 @@ def run_layer(torch, args) -> int:
     normed, sg = torch.empty_like(states), torch.empty_like(states)
     out = torch.empty(B, D, L, dtype=dt, device=dev)
     coef, dtok = rn(B, M, L), torch.empty(B, D, L, dtype=dt, device=dev)  # coefficient vectors are float32
-    partial = torch.empty(B, M, lib.fmscan_reduced_groups(D), L, device=dev)  # float32: groups of 4 consecutive d
+    partial = torch.empty(B, M, lib.fmscan_reduced_groups(B, D), L, device=dev)  # float32: groups of 8 (or 4) consecutive d
     code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
     P = lambda t: t.data_ptr()
     calls = {

@@ -84,7 +84,7 @@ def load() -> ctypes.CDLL:
                                     c_int64, c_int64, c_int64, c_int64, c_int, c_uint,
                                     c_void_p, c_size_t, c_void_p]
     lib.fmscan_reduced_groups.restype = c_int64
-    lib.fmscan_reduced_groups.argtypes = [c_int64]
+    lib.fmscan_reduced_groups.argtypes = [c_int64, c_int64]
     lib.fmscan_sum_groups.restype = c_int
     lib.fmscan_sum_groups.argtypes = [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_void_p]
     lib.fmscan_backward_reduced.restype = c_int

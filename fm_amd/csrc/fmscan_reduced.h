@@ -113,8 +113,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     };
     struct Slot {
         u32x4 g;
-        FloatChunk<E> co, cs, rr;  // LAYER; rr: LAYER == 2
-        float hbr;                 // LAYER == 2: rms at the step hb belongs to
+        FloatChunk<E> co, cs;  // LAYER
+    };
+    struct Rms {  // LAYER == 2; needed at the end of a step only, so loaded at its start and not a step ahead
+        FloatChunk<E> rr;
+        float hbr;  // rms at the step hb belongs to
     };
     // lane offset (elements) inside tile k, clamped into the row (a chunk past the end reads the last one)
     auto lane_elems = [&](int32_t k) {
@@ -147,11 +150,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
             s.co = load_float_chunk<E>(coef_out + base + lo);
             s.cs = load_float_chunk<E>(coef_self + base + lo);
         }
-        s.hbr = 0.0f;
-        if constexpr (LAYER == 2) {
-            s.rr = load_float_chunk<E>(rms + base + lo);
-            s.hbr = load_by_wave(rms + (base - (tw > 0 ? 1 : 0)), vzero);
-        }
+    };
+    auto fetch_rms = [&](Rms& s, int32_t k, int32_t mi) {
+        const int64_t tw = (int64_t)k * TILE;
+        const int64_t base = (b * M + slot_of(mi)) * L + tw;
+        s.rr = load_float_chunk<E>(rms + base + lane_elems(k));
+        s.hbr = load_by_wave(rms + (base - (tw > 0 ? 1 : 0)), vzero);
     };
     // The steps of a tile come in pairs (below), so an odd count of slots is padded with one step
     // that only loads.
@@ -235,6 +239,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                 for (int j = 0; j < J; ++j) fetch_row(rows[j], kf, mf, j);
                 return;
             }
+            [[maybe_unused]] Rms rms_now;
+            if constexpr (LAYER == 2) fetch_rms(rms_now, k, mi);
 
             // per slot: gates (1 where there is no step: identity), coefficients (0 there: no gradient)
             float g[E], co[E], cs[E];
@@ -253,9 +259,6 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     }
                 }
             }
-            float keep[E];  // 1 - g: the share of a step's gradient that goes to its token
-#pragma unroll
-            for (int i = 0; i < E; ++i) keep[i] = 1.0f - g[i];
             float a = g[E - 1];
 #pragma unroll
             for (int i = E - 2; i >= 0; --i) a *= g[i];
@@ -342,7 +345,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                         c = g[i] * delta;
                         // token gradient (1 - g) * delta
                         if constexpr (PLAIN) dtok[j][i] += delta;
-                        else dtok[j][i] = __builtin_fmaf(keep[i], delta, dtok[j][i]);
+                        else dtok[j][i] += delta - c;  // (1 - g) * delta = delta - g * delta
                         with_state[i] = __builtin_fmaf(hprev[i], delta, with_state[i]);
                         if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
                     }
@@ -356,8 +359,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                 // first from the lane that owns the chunk before (lane 63: from before the tile; at
                 // k == 0 what stands there is the initial state itself: factor 1)
                 float rr[E];
-                spread<E>(cur.rr, rr);
-                const float before = dpp<kWaveShl1>(k > 0 ? cur.hbr : 1.0f, rr[E - 1]);
+                spread<E>(rms_now.rr, rr);
+                const float before = dpp<kWaveShl1>(k > 0 ? rms_now.hbr : 1.0f, rr[E - 1]);
 #pragma unroll
                 for (int i = 0; i < E; ++i)
                     dgate[i] = __builtin_fmaf(i > 0 ? rr[i > 0 ? i - 1 : 0] : before, with_state[i], -with_token[i]);

@@ -7,14 +7,22 @@ using namespace fmscan::host;
 
 namespace {
 
-constexpr int kReducedGroup = 4;  // consecutive d one block of the reduced backward kernel sums over
 constexpr int kReducedWaves = 4;  // waves of a block: they split the M memory slots between them
+
+// Consecutive d that one block of the reduced backward kernel sums over: 8 where that still leaves two
+// blocks (eight waves, all the kernel's registers allow) for each of the 256 compute units, halving the
+// partials and the work per slot that does not depend on the row; 4 otherwise, for twice the blocks.
+int reduced_group(int64_t B, int64_t D) { return (__int128)B * ((D + 7) / 8) >= 512 ? 8 : 4; }
 
 }  // namespace
 
 extern "C" {
 
-int64_t fmscan_reduced_groups(int64_t D) { return D < 1 ? 0 : (D + kReducedGroup - 1) / kReducedGroup; }
+int64_t fmscan_reduced_groups(int64_t B, int64_t D) {
+    if (B < 1 || D < 1) return 0;
+    const int64_t group = reduced_group(B, D);
+    return (D + group - 1) / group;
+}
 
 // Shared by fmscan_backward_reduced and fmscan_backward_layer (coef_out != NULL): in the second
 // form `out_grad` carries the normalised states and the gradient of the states is made in the kernel.
@@ -40,10 +48,10 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
         return fail(FMSCAN_E_NULL, "%s: coef_self and out_grad must not be NULL", who);
     if (!pb.plain && !input_tokens)
         return fail(FMSCAN_E_NULL, "%s: input_tokens must not be NULL without FMSCAN_FLAG_PLAIN", who);
-    if (B > INT32_MAX / fmscan_reduced_groups(D))
-        return fail(FMSCAN_E_SHAPE, "%s: B * ceil(D/%d) must be < 2^31", who, kReducedGroup);
+    const int group = reduced_group(B, D);
+    const int64_t groups = fmscan_reduced_groups(B, D);
+    if (B > INT32_MAX / groups) return fail(FMSCAN_E_SHAPE, "%s: B * ceil(D/%d) must be < 2^31", who, group);
     const int64_t full = pb.rows * L * pb.esize;
-    const int64_t groups = fmscan_reduced_groups(D);
     const Range outs[] = {{"token_grad", token_grad, B * D * L * pb.esize},
                           {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
                           {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
@@ -72,8 +80,8 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
         return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
     const size_t tile = (size_t)(16 / pb.esize) * 64;
     const int64_t Mw = (M + kReducedWaves - 1) / kReducedWaves;  // slots per wave
-    const size_t lds = (2 * kReducedGroup * tile + 2 * kReducedGroup * 2 * 64 * 4 +
-                        (size_t)kReducedWaves * (size_t)Mw * kReducedGroup + (size_t)kReducedWaves * tile) * sizeof(float);
+    const size_t lds = (2 * group * tile + 2 * (size_t)group * 2 * 64 * 4 +
+                        (size_t)kReducedWaves * (size_t)Mw * group + (size_t)kReducedWaves * tile) * sizeof(float);
     if (lds > kMaxDynamicLds)
         return fail(FMSCAN_E_SHAPE, "%s: M = %lld needs %zu bytes of LDS (limit %u)", who, (long long)M, lds,
                     kMaxDynamicLds);
@@ -84,8 +92,8 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     int rc = 0;
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
-        auto go = [&](auto pt, auto lt) {
-            auto kern = fmscan::scan_backward_reduced_kernel<T, kReducedGroup, kReducedWaves, decltype(pt)::value,
+        auto go = [&](auto jt, auto pt, auto lt) {
+            auto kern = fmscan::scan_backward_reduced_kernel<T, decltype(jt)::value, kReducedWaves, decltype(pt)::value,
                                                              decltype(lt)::value>;  // lt: 0 plain call, 1 layer, 2 layer + recovered states
             static std::atomic<uint64_t> armed{0};
             if ((rc = raise_lds_limit((const void*)kern, armed, who)) != 0) return;
@@ -96,8 +104,13 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                 recover ? rms : nullptr, (int32_t)M, (int32_t)D, L, (int32_t)Mw);
         };
         auto with_plain = [&](auto lt) {
-            if (pb.plain) go(BoolTag<true>{}, lt);
-            else go(BoolTag<false>{}, lt);
+            if (group == 8) {
+                if (pb.plain) go(IntTag<8>{}, BoolTag<true>{}, lt);
+                else go(IntTag<8>{}, BoolTag<false>{}, lt);
+            } else {
+                if (pb.plain) go(IntTag<4>{}, BoolTag<true>{}, lt);
+                else go(IntTag<4>{}, BoolTag<false>{}, lt);
+            }
         };
         if (recover) with_plain(IntTag<2>{});
         else if (layer) with_plain(IntTag<1>{});

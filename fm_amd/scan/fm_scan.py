@@ -225,7 +225,7 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
         if t is not None:
             _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
     code = _dtype_code(gates)
-    groups = _raw.fmscan_reduced_groups(D)
+    groups = _raw.fmscan_reduced_groups(B, D)
     d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
     partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
     if cached_output.numel():
@@ -533,7 +533,7 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         coef_out, coef_self = torch.empty_like(q), torch.empty_like(q)  # float32, like q
         rms = torch.empty_like(q) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
-        groups = _raw.fmscan_reduced_groups(D)
+        groups = _raw.fmscan_reduced_groups(B, D)
         d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
         zeros = torch.zeros((B, M, D), dtype=dtype, device=dev)

@@ -176,15 +176,16 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
  * full, fm/scan/fm_scan.cuh:200-207, and names the fused form as a TODO). Meant for
  * M > 1 and D > 1; the per-pair tensors are never written.
  *   token_grad         (B, D, L)     out, element dtype: sum over m of (1 - g) * delta
- *   gate_grad_partial  (B, M, G, L)  out, float32, G = fmscan_reduced_groups(D): the sum of
- *                      (h[t-1] - x[t]) * delta over each group of 4 consecutive d;
+ *   gate_grad_partial  (B, M, G, L)  out, float32, G = fmscan_reduced_groups(B, D): the sum of
+ *                      (h[t-1] - x[t]) * delta over each group of 8 consecutive d (of 4 where 8
+ *                      would leave too few blocks for the GPU: small B * D);
  *                      d_gates[b,m,t] is the sum of the G partials (one more small pass
  *                      for the caller; sums are accumulated in float32 throughout)
  * Other arguments as fmscan_backward. Needs 16-byte aligned pointers and
  * L * sizeof(element) % 16 == 0 (FMSCAN_E_UNALIGNED otherwise: use fmscan_backward);
  * flags: only FMSCAN_FLAG_PLAIN.
  */
-int64_t fmscan_reduced_groups(int64_t D);
+int64_t fmscan_reduced_groups(int64_t B, int64_t D);
 /* out[r, t] = sum over g of partial[r, g, t] for float32 partial (rows, G, L), rounded once to
  * the call's dtype: d_gates (B, M, L) from gate_grad_partial with rows = B * M (the reference's
  * torch.sum at fm/scan/fm_scan.py:76). Groups are added in their order: deterministic. */

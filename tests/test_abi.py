@@ -111,7 +111,9 @@ def test_rejected_arguments(lib):
     assert lay(h=None) == E_NULL                      # no saved states and no inv_rms to take them back with
     assert lay(h=None, r=3 * P) == E_ALIAS            # inv_rms under token_grad
     assert lay(dx=9 * P) == E_ALIAS                   # token_grad on top of the layer's out_grad
-    assert lib.fmscan_reduced_groups(128) == 32 and lib.fmscan_reduced_groups(9) == 3
+    # groups of 8 rows where B * ceil(D / 8) fills the GPU twice over, of 4 otherwise
+    assert lib.fmscan_reduced_groups(32, 128) == 16 and lib.fmscan_reduced_groups(1, 128) == 32
+    assert lib.fmscan_reduced_groups(2, 9) == 3 and lib.fmscan_reduced_groups(512, 9) == 2 and lib.fmscan_reduced_groups(0, 9) == 0
     assert fwd(lib, out=P) == E_ALIAS                 # out on top of gates
     assert fwd(lib, out=2 * P + 16) == E_ALIAS        # out inside tokens
     assert bwd(lib, h=None) == E_NULL

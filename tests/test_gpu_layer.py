@@ -79,6 +79,8 @@ LAYER_SHAPES = [
     ((1, 1001, 3, 12), 1e-4, "rows that are not 16-byte multiples"),
     ((3, 40, 2, 9), 1e-4, "row shorter than a tile, ragged D"),
     ((1, 2048, 2, 130), 1e-4, "D beyond one block of the read-out"),
+    ((64, 40, 3, 60), 1e-4, "enough blocks for groups of 8 rows in backward, the last group ragged"),
+    ((16, 520, 5, 256), 1e-4, "groups of 8 rows, a ragged last tile, waves with one slot or none"),
 ]
 
 

@@ -440,8 +440,11 @@ def test_segment_requests_without_room_fail_loudly(scan):
 def test_backward_with_sums_inside(scan, dtype, plain):
     """fm_scan_backward_reduced (d_gates, d_tokens straight from one kernel) against the
     float64 oracle's summed gradients, and against the two-tensor path plus torch.sum."""
+    # (the last three: enough blocks for groups of 8 rows, with a ragged last group, a ragged last
+    # tile, an odd count of slots per wave and waves without a slot)
     for (B, M, D, L) in [(2, 3, 5, 512), (1, 2, 2, 8), (2, 4, 8, 4096), (1, 33, 17, 1000 // 8 * 8),
-                         (3, 2, 9, 2048), (1, 70, 3, 640), (2, 3, 4, 2568)]:
+                         (3, 2, 9, 2048), (1, 70, 3, 640), (2, 3, 4, 2568),
+                         (64, 3, 60, 40), (16, 5, 256, 520), (128, 2, 28, 1032)]:
         gen = torch.Generator().manual_seed(M * 100 + D)
         g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
         x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
