@@ -259,7 +259,9 @@ def run_layer(torch, args) -> int:
     normed, sg = torch.empty_like(states), torch.empty_like(states)
     out = torch.empty(B, D, L, dtype=dt, device=dev)
     coef, dtok = rn(B, M, L), torch.empty(B, D, L, dtype=dt, device=dev)  # coefficient vectors are float32
-    partial = torch.empty(B, M, lib.fmscan_reduced_groups(B, D), L, device=dev)  # float32: groups of 8 (or 4) consecutive d
+    groups = lib.fmscan_reduced_groups(B, D)  # of 8 (or 4) consecutive d
+    partial = torch.empty(B, M, groups, L, device=dev)  # float32
+    partial_bytes = 4 * B * M * groups * L
     code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
     P = lambda t: t.data_ptr()
     calls = {
@@ -272,7 +274,7 @@ def run_layer(torch, args) -> int:
         # the form that makes the states' gradient itself (no readout_backward_kernel, no G) and takes the
         # scanned states back from the normalised ones (reads one (B,M,D,L) tensor)
         "rowdot_kernel (dot)": (s * N, lambda: lib.fmscan_readout_dot(P(normed), P(og), None, P(q), None, None, None, None, None, None, B, M, D, L, code, st)),
-        "scan_backward_reduced_kernel (layer form)": (s * N + 4 * N // 4, lambda: lib.fmscan_backward_layer(
+        "scan_backward_reduced_kernel (layer form)": (s * N + partial_bytes, lambda: lib.fmscan_backward_layer(
             P(gates), P(normed), P(coef), P(coef), P(og), P(zeros), P(dtok), None, P(rms), P(tokens), P(partial),
             None, None, B, M, D, L, code, 0, st)),
         # the same steps as separate kernels (what runs for D beyond one block's rows, or with the
@@ -283,7 +285,7 @@ def run_layer(torch, args) -> int:
             P(states), P(inv), P(read), P(normed), P(out), B, M, D, L, code, st)),
         "readout_backward_kernel": (2 * s * N, lambda: lib.fmscan_readout_backward(
             P(normed), P(inv), P(read), P(og), None, P(q), None, P(sg), B, M, D, L, code, st)),
-        "scan_backward_reduced_kernel": (2 * s * N + 4 * N // 4, lambda: lib.fmscan_backward_reduced(
+        "scan_backward_reduced_kernel": (2 * s * N + partial_bytes, lambda: lib.fmscan_backward_reduced(
             P(gates), P(G), P(zeros), P(dtok), P(states), P(tokens), P(partial), None, None, B, M, D, L, code, 0, st)),
     }
     if args.probe:  # for rocprofv3 --pmc: a copy of known size, then every kernel a few times
