@@ -674,6 +674,50 @@ def test_layer_backward_kernel_equals_the_two_step_route(scan, dtype, mem_norm):
         check(tag + " d_read", leaves[3].grad, o_dr, tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("plain", [False, True])
+def test_layer_form_of_the_backward_kernel_through_the_c_abi(scan, dtype, plain):
+    """fmscan_backward_layer with arbitrary coefficient vectors, with the saved states or with rms in
+    their place, plain form included, against fmscan_backward_reduced fed the states' gradient
+    G = coef_out * out_grad - coef_self * states_n as a tensor. Blocks of 4 rows and of 8."""
+    lib = scan.module
+    st = torch.cuda.current_stream().cuda_stream
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    flags = 1 if plain else 0
+    P = lambda t: t.data_ptr()
+    for (B, M, D, L) in [(2, 5, 12, 520), (64, 3, 60, 40), (16, 6, 256, 1032)]:
+        gen = gpu_gen(B + M + D)
+        g = torch.sigmoid(torch.randn(B, M, L, device=DEV, generator=gen) + 2).to(dtype)
+        x = torch.randn(B, D, L, device=DEV, generator=gen).to(dtype)
+        og = torch.randn(B, D, L, device=DEV, generator=gen).to(dtype)
+        co = torch.randn(B, M, L, device=DEV, generator=gen)
+        cs = torch.randn(B, M, L, device=DEV, generator=gen) * 0.3
+        rms = torch.rand(B, M, L, device=DEV, generator=gen) + 0.5
+        zeros = torch.zeros(B, M, D, dtype=dtype, device=DEV)
+        states = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        scan.fm_scan_forward(g, x, zeros, states, plain=plain)
+        groups = lib.fmscan_reduced_groups(B, D)
+        assert groups == ((D + 7) // 8 if B * ((D + 7) // 8) >= 512 else (D + 3) // 4)
+        for recover in (False, True):
+            # with rms in place of the saved states, the kernel takes them to be states_n * rms
+            states_n = (states.float() / rms.unsqueeze(2)).to(dtype) if recover else states
+            saved = (states_n.float() * rms.unsqueeze(2)).to(dtype) if recover else states
+            G = (co.unsqueeze(2) * og.float().unsqueeze(1) - cs.unsqueeze(2) * states_n.float()).to(dtype)
+            want_tok = torch.empty(B, D, L, dtype=dtype, device=DEV)
+            want_part = torch.empty(B, M, groups, L, device=DEV)
+            assert lib.fmscan_backward_reduced(P(g), P(G), P(zeros), P(want_tok), P(saved), P(x), P(want_part), None,
+                                               None, B, M, D, L, code, flags, st) == 0
+            got_tok, got_part = torch.empty_like(want_tok), torch.empty_like(want_part)
+            assert lib.fmscan_backward_layer(P(g), P(states_n), P(co), P(cs), P(og), P(zeros), P(got_tok),
+                                             None if recover else P(states), P(rms) if recover else None, P(x),
+                                             P(got_part), None, None, B, M, D, L, code, flags, st) == 0, \
+                lib.fmscan_last_error()
+            tag = f"{(B, M, D, L)} {dtype} plain={plain} recover={recover}"
+            # G rounded to the storage type on one side, made in float32 on the other: 2 * TOL
+            check(tag + " d_tokens", got_tok, want_tok.double().cpu().numpy(), 2 * TOL[dtype])
+            check(tag + " gate gradient", got_part.sum(dim=2), want_part.sum(dim=2).double().cpu().numpy(), 2 * TOL[dtype])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_layer_prepare_and_finish_kernels(scan, dtype):
     """The layer's small tensors: gates and read weights with time last, and the gradients of
