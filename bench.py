@@ -12,8 +12,9 @@ bfloat16, (B, C, T) = (16, 2048, 16384), passed as B' = B*C rows with M = D = 1.
 Prints one JSON line. `value` is the effective HBM bandwidth of the step:
 algorithmic bytes (9 * element size per element: forward reads g, x and writes h;
 backward reads g, dL/dh, h, x and writes the two gradients) divided by wall
-time. `roofline` prices the backward kernel, the dominant one, from HIP events
-recorded around it inside the timed region. `cpu_baseline` times the compiled CPU
+time over K steps that hold nothing but the calls. `roofline` prices the backward
+kernel, the dominant one, from HIP events recorded around it in a second pass of the
+same K steps right after. `cpu_baseline` times the compiled CPU
 port of the same scan (oracle/fmscan_cpu.c) on this host's cores on a bounded
 row sample of the same workload.
 
