@@ -31,7 +31,10 @@ namespace fmscan {
 // ahead: while the J rows of a slot are worked on, the J tiles of the next slot (or of the
 // first slot of the tile before) are in flight, as are its per-slot vectors; every step
 // issues the same loads whatever its position (addresses are clamped into the tensors), so
-// the count of loads in flight is a compile-time number.
+// the count of loads in flight is a compile-time number. (The per-slot vectors of the step at
+// work and of the step after it sit in two sets of registers that swap roles, steps come in
+// pairs; what a step needs only at its end, the layer form's rms vector, is loaded at its
+// start. J = 8 uses all 256 registers two waves per SIMD leave.)
 // HBM traffic per element of (B, M, D, L): G and h (2s), or the normalised states alone in
 // the layer form (s), plus 4/J bytes of partials, against 6s for the unfused kernel plus the
 // two torch.sum passes.
