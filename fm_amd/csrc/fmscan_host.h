@@ -128,8 +128,9 @@ inline unsigned lds_share(unsigned blocks_per_cu) {
 // MI355X over the benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536
 // in 16-bit types and 8192 x 4096 in float32, forward and backward separately. What it
 // encodes: one or two waves per row stream best when there are many rows of moderate
-// length; long rows want eight waves side by side so that fewer rows are open at a
-// time; with few rows a block per row keeps every compute unit busy. One to two waves
+// length; long rows want eight waves side by side (sixteen in backward, which only the library
+// chooses: 0.501 -> 0.478 ms at (4096 rows, 65536); forward gains nothing from them) so that fewer
+// rows are open at a time; with few rows a block per row keeps every compute unit busy. One to two waves
 // per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few rows
 // that even eight waves per row leave compute units idle (fewer than 32 rows), and a
 // workspace to hold the segment pairs, rows are cut into segments (two passes).
@@ -180,13 +181,13 @@ inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
     unsigned w = pb.waves;
     if (!w) {
         if (shared_inputs && pb.rows >= 16384) w = 1;
-        else if (long_rows) w = 8;
+        else if (long_rows) w = backward ? 16 : 8;
         else if (few_rows) w = 4;
         else if (tiles1 >= 16) w = 1;
         else if (tiles1 >= 8) w = backward ? 2 : 1;
         else w = 1;
         while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
-        while (w < 8 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
+        while (w < 8 && w != 16 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
     }
     t.waves = w;
     plan_segments(pb, t, may_split);
@@ -194,6 +195,7 @@ inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
     const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
     unsigned bpc, depth;
     if (shared_inputs) { bpc = 8; depth = 2; }
+    else if (w == 16) { bpc = 1; depth = 2; }  // backward, long rows: 16 waves leave 128 registers each
     else if (w == 8) { bpc = 1; depth = backward ? 2 : 4; }
     else if (w == 4) { bpc = 4; depth = backward ? 4 : 2; }
     else if (w == 2) { bpc = 4; depth = 2; }
@@ -202,6 +204,7 @@ inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
     else { bpc = 4; depth = 2; }
     t.blocks_per_cu = pb.blocks_per_cu ? pb.blocks_per_cu : bpc;
     t.depth = pb.depth ? pb.depth : depth;
+    if (w == 16) t.depth = 2;  // deeper does not fit the registers of a 16-wave block
     return t;
 }
 
@@ -276,6 +279,7 @@ void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f
             case 1: with_waves(IntTag<1>{}, IntTag<4>{}); break;  // 4 independent rows per block
             case 2: with_waves(IntTag<2>{}, IntTag<1>{}); break;
             case 4: with_waves(IntTag<4>{}, IntTag<1>{}); break;
+            case 16: with_waves(IntTag<16>{}, IntTag<1>{}); break;
             default: with_waves(IntTag<8>{}, IntTag<1>{}); break;
         }
     });

@@ -209,6 +209,34 @@ def test_shapes_and_variants(scan, dtype, waves, plain):
         check(tag + " gate grad", dg, gg, TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_long_rows_with_rows_enough_not_to_be_cut(scan, dtype):
+    """Rows of 64 tiles or more, 32 rows or more: the library's own choice there is 8 waves per row
+    forward and 16 backward (a choice only it makes). Whole tiles and a ragged end, aligned rows and
+    rows one element off (element access)."""
+    for rows, L in ((40, 40000), (33, 40001), (64, 65536)):
+        if dtype == torch.float32:
+            L = L // 2 + (L & 1)  # still 64 tiles or more of 256 elements
+        gen = torch.Generator().manual_seed(L)
+        g = torch.sigmoid(torch.randn(rows, 1, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(rows, 1, L, generator=gen).to(dtype).to(DEV)
+        G = torch.randn(rows, 1, 1, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(rows, 1, 1, generator=gen).to(dtype).to(DEV)
+        fpg = torch.randn(rows, 1, 1, generator=gen).to(dtype).to(DEV)
+        for plain in (False, True):
+            out, dx, dg = run_fwd_bwd(scan, g, x, G, h0, fpg, plain=plain)
+            h_ref = C.forward_f64(g, x, h0, plain)
+            tg, gg = C.backward_f64(g, G, out, x, fpg, h0, plain)
+            tag = f"{(rows, L)} {dtype} plain={plain}"
+            check(tag + " states", out, h_ref, TOL[dtype])
+            check(tag + " token grad", dx, tg, TOL[dtype])
+            check(tag + " gate grad", dg, gg, TOL[dtype])
+            # the same rows with 8 waves per row, as asked for by the caller: the same mathematics
+            _, dx8, dg8 = run_fwd_bwd(scan, g, x, G, h0, fpg, plain=plain, waves_per_row=8)
+            check(tag + " token grad vs 8 waves", dx, dx8.double().cpu().numpy(), 2 * TOL[dtype])
+            check(tag + " gate grad vs 8 waves", dg, dg8.double().cpu().numpy(), 2 * TOL[dtype])
+
+
 def test_more_than_2_31_elements(scan):
     """The reference indexes with 32-bit ints (fm_scan.cuh:76-82: N < 2^31); here offsets are 64-bit.
     Rows that lie beyond element 2^31 of a problem must come out exactly as the same rows of a small
