@@ -81,23 +81,55 @@ def profiled_traffic(stem, kernel, copy_bytes):
     return int(total), " + ".join(used)
 
 
+PROBE_SRC = ROOT / "bench_stream_probe.hip"
+PROBE_LIB = ROOT / "bench_stream_probe.so"
+
+
+def build_probe(verbose=False):
+    """Compiles the bare streaming kernel this benchmark compares the scan kernels with into a small
+    library of its own, beside this file. The product library (fm_amd) does not contain it."""
+    import subprocess
+
+    from fm_amd import build as hip_build
+
+    tmp = PROBE_LIB.with_suffix(".so.tmp%d" % os.getpid())
+    cmd = [hip_build.hipcc_path(), *hip_build.HIPCC_FLAGS, "-shared", "-o", str(tmp), str(PROBE_SRC)]
+    if verbose:
+        print("[bench] " + " ".join(cmd), flush=True)
+    try:
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode:
+            raise RuntimeError("hipcc failed on bench_stream_probe.hip:\n" + res.stderr)
+        os.replace(tmp, PROBE_LIB)
+    finally:
+        tmp.unlink(missing_ok=True)
+    return PROBE_LIB
+
+
+def load_probe():
+    """The streaming probe, built first when it is missing or older than its source."""
+    import ctypes
+
+    if not PROBE_LIB.exists() or PROBE_LIB.stat().st_mtime < PROBE_SRC.stat().st_mtime:
+        build_probe()
+    lib = ctypes.CDLL(str(PROBE_LIB))
+    lib.fmscan_probe_stream.restype = ctypes.c_int
+    lib.fmscan_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    return lib
+
+
 def streaming_copy(torch, rows, row_bytes, fwd_ms, bwd_ms, reps=10):
     """What a bare streaming kernel with the scan kernels' access pattern reaches on the same shape.
 
-    `libfmscan_probe.so` (fm_amd/csrc/stream_probe.hip) walks `rows` rows of `row_bytes` bytes, one wave
+    `bench_stream_probe.so` (bench_stream_probe.hip, beside this file) walks `rows` rows of `row_bytes` bytes, one wave
     per row, reading 2 tensors and writing 1 (the forward scan's streams) or reading 3 and writing 2
     (the backward scan's), with no arithmetic and no tuning of residency. The published 8 TB/s is not
     reachable by any kernel; this is a second reference point for kernels with these streams. Timed with
     events on the current stream, best of two prefetch depths."""
-    import ctypes
-    from pathlib import Path
-    lib_path = Path(__file__).resolve().parent / "fm_amd" / "lib" / "libfmscan_probe.so"
-    if row_bytes % 1024 or not lib_path.exists():
+    if row_bytes % 1024:
         return None
-    lib = ctypes.CDLL(str(lib_path))
-    lib.fmscan_probe_stream.restype = ctypes.c_int
-    lib.fmscan_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
-                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib = load_probe()
     tensor = rows * row_bytes
     src = torch.ones(3 * tensor, dtype=torch.uint8, device="cuda")
     dst = torch.empty(2 * tensor, dtype=torch.uint8, device="cuda")

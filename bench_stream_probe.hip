@@ -1,4 +1,5 @@
-// libfmscan_probe.so: a bare streaming kernel for bench.py, not part of libfmscan_hip.so.
+// bench_stream_probe.so: a bare streaming kernel for bench.py (which builds it when it is not there),
+// not part of the fm_amd package or of libfmscan_hip.so.
 //
 // It walks memory the way the scan kernels do (one 64-lane wave per row, 16 bytes per lane and step,
 // four rows per block, the next steps' loads in flight while the current one is stored) but does no

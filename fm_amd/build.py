@@ -30,10 +30,6 @@ HEADERS = ["fmscan_host.h", "fmscan_device.h", "fmscan_kernels.h", "fmscan_reduc
            "fmscan_normed.h"]
 DEPS = [CSRC / n for n in UNITS + HEADERS] + [PKG.parent / "include" / "fmscan.h"]
 LIB = PKG / "lib" / "libfmscan_hip.so"
-# bench.py's bare streaming kernel: a library of its own, so that the product library holds only the path
-PROBE_SRC = CSRC / "stream_probe.hip"
-PROBE_LIB = PKG / "lib" / "libfmscan_probe.so"
-
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
@@ -91,20 +87,7 @@ def build(verbose: bool = True, extra_flags=(), jobs: int | None = None) -> Path
             os.replace(tmp, LIB)
         finally:
             tmp.unlink(missing_ok=True)
-    build_probe(verbose, extra_flags)
     return LIB
-
-
-def build_probe(verbose: bool = True, extra_flags=()) -> Path:
-    """Compiles bench.py's streaming probe (`stream_probe.hip`) into its own small library."""
-    PROBE_LIB.parent.mkdir(parents=True, exist_ok=True)
-    tmp = PROBE_LIB.with_suffix(".so.tmp%d" % os.getpid())
-    try:
-        _run([hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-shared", "-o", str(tmp), str(PROBE_SRC)], verbose)
-        os.replace(tmp, PROBE_LIB)
-    finally:
-        tmp.unlink(missing_ok=True)
-    return PROBE_LIB
 
 
 if __name__ == "__main__":

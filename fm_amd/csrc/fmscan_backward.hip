@@ -89,7 +89,7 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
     }
     const bool fold = M == 1 && D == 1;
     int rc = 0;
-    dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
+    dispatch<true>(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;
         rc = launch_bwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
                    decltype(vt)::value, decltype(ft)::value>(pb, tune, gates, out_grad, first_prop_grad,

@@ -99,7 +99,7 @@ int forward(const char* who, const void* gates, const void* tokens, const void* 
     }
     const bool fold = M == 1 && D == 1;
     int rc = 0;
-    dispatch(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
+    dispatch<false>(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;
         rc = launch_fwd<T, decltype(wt)::value, decltype(rt)::value, decltype(dt)::value, decltype(pt)::value,
                    decltype(vt)::value, decltype(ft)::value>(pb, tune, gates, tokens, initial_state, out,

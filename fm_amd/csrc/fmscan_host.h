@@ -67,8 +67,8 @@ inline int parse(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned
         return fail(FMSCAN_E_FLAGS, "fmscan: waves per row must be 0 (auto), 1, 2, 4 or 8 (got %u)",
                     waves);
     const unsigned depth = (flags & FMSCAN_FLAG_DEPTH_MASK) >> FMSCAN_FLAG_DEPTH_SHIFT;
-    if (depth != 0 && (depth < 2 || depth > 4))
-        return fail(FMSCAN_E_FLAGS, "fmscan: prefetch depth must be 0 (auto), 2, 3 or 4 (got %u)", depth);
+    if (depth != 0 && depth != 2 && depth != 4)
+        return fail(FMSCAN_E_FLAGS, "fmscan: prefetch depth must be 0 (auto), 2 or 4 (got %u)", depth);
     // rows*L elements must be addressable and the grid must fit 31 bits
     const __int128 rows = (__int128)B * M * D;
     if (rows > (__int128)INT32_MAX || rows * L > ((__int128)1 << 46))
@@ -252,8 +252,10 @@ void with_bool(bool v, F&& f) {
 }
 
 // dtype, waves per row (with the rows per block that go with it), prefetch depth, plain,
-// vector access, fold -> f(tt, wt, rt, dt, pt, vt, ft)
-template <typename F>
+// vector access, fold -> f(tt, wt, rt, dt, pt, vt, ft). Only what choose() and the flags can ask
+// for is instantiated: depths 2 and 4, and 16 waves per row for the backward kernel alone
+// (WITH16), the only one choose() gives them to.
+template <bool WITH16, typename F>
 void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f) {
     with_dtype(dtype, [&](auto tt) {
         auto with_waves = [&](auto wt, auto rt) {
@@ -269,17 +271,19 @@ void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f
                 if (fold) with_depth(dt, BoolTag<true>{}, BoolTag<true>{});
                 else with_depth(dt, BoolTag<true>{}, BoolTag<false>{});
             };
-            switch (t.depth) {
-                case 2: with_fold(IntTag<2>{}); break;
-                case 3: with_fold(IntTag<3>{}); break;
-                default: with_fold(IntTag<4>{}); break;
-            }
+            if (t.depth == 2) with_fold(IntTag<2>{});
+            else with_fold(IntTag<4>{});
         };
         switch (t.waves) {
             case 1: with_waves(IntTag<1>{}, IntTag<4>{}); break;  // 4 independent rows per block
             case 2: with_waves(IntTag<2>{}, IntTag<1>{}); break;
             case 4: with_waves(IntTag<4>{}, IntTag<1>{}); break;
-            case 16: with_waves(IntTag<16>{}, IntTag<1>{}); break;
+            case 16:
+                if constexpr (WITH16) {
+                    with_waves(IntTag<16>{}, IntTag<1>{});
+                    break;
+                }
+                [[fallthrough]];
             default: with_waves(IntTag<8>{}, IntTag<1>{}); break;
         }
     });

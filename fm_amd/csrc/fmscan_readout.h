@@ -333,8 +333,18 @@ __global__ __launch_bounds__(256) void swap_last_two_wide_kernel(const uint16_t*
 
 // gates[b, m, t] = 1 - alpha[b, t, m] * update_scale[b, t], read[b, m, t] = alpha[b, t, m] *
 // output_scale[b, t] (reference fm_scan.py:116,118-119,130: two products, two transposed
-// copies and a subtraction). 64 x 64 tiles of (t, m) through LDS; float32 arithmetic, one
-// rounding. grid: B * tiles_t * tiles_m.
+// copies and a subtraction). The reference's `update_weight = alpha * update_scale` is a tensor
+// of the storage type and `1.0 - update_weight` another: the product is rounded to T, and one
+// minus the rounded product is rounded to T again. The same two roundings are made here (a gate
+// near one decides a decay: it has to be the gate the reference forms, bit for bit); the
+// multiply and the subtraction are kept apart (no fused multiply-add), so that float32 gets the
+// two roundings of its two operations as well. read is one product, one rounding.
+// 64 x 64 tiles of (t, m) through LDS. grid: B * tiles_t * tiles_m.
+__device__ __forceinline__ float product_rounded(float a, float b) {
+#pragma clang fp contract(off)  // a product of its own, never one half of a fused multiply-add
+    return a * b;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void layer_prepare_kernel(
     const T* __restrict__ alpha /* (B, L, M) */, const T* __restrict__ update_scale /* (B, L) */,
@@ -352,8 +362,9 @@ __global__ __launch_bounds__(256) void layer_prepare_kernel(
         const int64_t t = t0 + i;
         if (t < L && m0 + lane < M) {
             const float a = (float)alpha[(b * L + t) * M + m0 + lane];
-            tg[i][lane] = 1.0f - a * (float)update_scale[b * L + t];
-            tr[i][lane] = a * (float)output_scale[b * L + t];
+            const T update_weight = (T)product_rounded(a, (float)update_scale[b * L + t]);
+            tg[i][lane] = 1.0f - (float)update_weight;
+            tr[i][lane] = product_rounded(a, (float)output_scale[b * L + t]);
         }
     }
     __syncthreads();

@@ -457,27 +457,32 @@ def fm_readout(states, read, mem_norm=True, norm_eps=1e-6):
 def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
     """Scan, RMS norm and read-out (reference fm_scan.py:121-131), time last. Returns what the
     layer hands back and what its gradient needs."""
+    _require(gates.dim() == 3 and tokens.dim() == 3, "gates must be (B, M, L) and tokens (B, D, L)")
     B_g, M, L_g = gates.shape
     B, D, L = tokens.shape
-    assert L_g == L
-    assert B_g == B
-    assert gates.is_contiguous()
-    assert tokens.is_contiguous()
+    _require(L_g == L and B_g == B, f"gates {tuple(gates.shape)} and tokens {tuple(tokens.shape)} must agree in B and L")
+    # Every tensor whose address goes to the library is checked here, before the route is chosen:
+    # the fused routes below hand over raw pointers, and a tensor on the host or on another GPU, or
+    # one of another element size, would be a memory fault in the kernel instead of an error here.
+    dev = gates.device
     given_state = initial_state is not None
+    named = [("gates", gates), ("tokens", tokens), ("read", read)]
     if given_state:
-        assert initial_state.shape == (B, M, D)
-        assert initial_state.is_contiguous()
+        named.append(("initial_state", initial_state))
+    for name, t in named:
+        _on_gpu(name, t, dev)
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        _require(t.dtype == gates.dtype, f"{name} has dtype {t.dtype}, gates has {gates.dtype}")
+    _require(tuple(read.shape) == (B, M, L), f"read must be {(B, M, L)}, got {tuple(read.shape)}")
+    if given_state:
+        _require(tuple(initial_state.shape) == (B, M, D),
+                 f"initial_state must be {(B, M, D)}, got {tuple(initial_state.shape)}")
     else:
-        initial_state = torch.zeros((B, M, D), device=gates.device, dtype=gates.dtype)
-    states = torch.empty((B, M, D, L), device=gates.device, dtype=gates.dtype)
+        initial_state = torch.zeros((B, M, D), device=dev, dtype=gates.dtype)
+    code = _dtype_code(gates)
+    states = torch.empty((B, M, D, L), device=dev, dtype=gates.dtype)
     kept_state = initial_state if given_state else None
     if mem_norm and states.numel() and (L * states.element_size()) % 16 == 0 and _aligned(gates, tokens, states, read):
-        dev = gates.device
-        _on_gpu("tokens", tokens, dev)
-        _on_gpu("read", read, dev)
-        _require(tokens.dtype == gates.dtype, f"tokens has dtype {tokens.dtype}, gates has {gates.dtype}")
-        _require(read.dtype == gates.dtype and read.is_contiguous(), "read must be contiguous, of the gates' dtype")
-        code = _dtype_code(gates)
         inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
@@ -559,8 +564,10 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         inv_rms, read_grad_float32=True)
     if ext_grad is not None and not mem_norm:
         state_grad += ext_grad
-    if mem_norm:  # the scanned states were not kept: take them back from the normalised ones
-        states = normed * (1.0 / inv_rms).to(dtype).unsqueeze(2)
+    if mem_norm:
+        # the scanned states were not kept: take them back from the normalised ones, with rms in the
+        # float32 it is held in and one rounding, as the fused route's kernel does
+        states = (normed.float() * (1.0 / inv_rms).unsqueeze(2)).to(dtype)
     d_gates, d_tokens, d_h0 = _scan_gradients(gates, tokens, states, initial_state, state_grad,
                                               want_initial_state_grad)
     return d_gates.float().unsqueeze(2), d_tokens, d_h0, q

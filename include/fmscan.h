@@ -61,7 +61,7 @@ extern "C" {
                                          time (1..15); 0 = let the library choose */
 #define FMSCAN_FLAG_BLOCKS_MASK  0xF000u
 #define FMSCAN_FLAG_DEPTH_SHIFT  16   /* bits 16..19: tiles whose loads a wave keeps in flight
-                                         ahead of the one it scans (2, 3 or 4); 0 = library's choice */
+                                         ahead of the one it scans (2 or 4); 0 = library's choice */
 #define FMSCAN_FLAG_DEPTH_MASK   0xF0000u
 #define FMSCAN_FLAG_SEGMENTS_SHIFT 20 /* bits 20..27: segments a row is cut into (2..255, needs the
                                          workspace); 1 = never cut; 0 = library's choice */
@@ -145,7 +145,14 @@ int fmscan_forward_static(const void* gates, const void* tokens, const void* ini
  *   first_prop_grad  (B, M, D)     in, may be NULL (= zeros): gradient flowing in
  *                                       from beyond the last step (:360)
  *   token_grad_out   (B, M, D, L)  out  (1 - g) * delta per (m, d)
- *   cached_output    (B, M, D, L)  in   h saved by the forward call
+ *   cached_output    (B, M, D, L)  in   h as the forward call wrote it for these gates, tokens
+ *                    and initial state. With FMSCAN_FLAG_PLAIN every element is read (h[t-1]
+ *                    enters the gate gradient, as in the reference kernel, :189-197). Without the
+ *                    flag it is read at one position per wave and tile only (the element just
+ *                    before the wave's part of the tile, and h[0]); the states in between are
+ *                    made again in float32 from gates and input_tokens. A buffer that is not the
+ *                    forward output for these inputs therefore gives a gate gradient the
+ *                    reference kernel would not give for it; the other outputs do not depend on it.
  *   input_tokens     (B, D, L)     in   (ignored with FMSCAN_FLAG_PLAIN)
  *   gate_grad_out    (B, M, D, L)  out  (h[t-1] - x[t]) * delta per (m, d)
  *   initial_state    (B, M, D)     in, may be NULL: h[-1] used by gate_grad at t = 0.
@@ -181,7 +188,10 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
  *                      would leave too few blocks for the GPU: small B * D);
  *                      d_gates[b,m,t] is the sum of the G partials (one more small pass
  *                      for the caller; sums are accumulated in float32 throughout)
- * Other arguments as fmscan_backward. Needs 16-byte aligned pointers and
+ * Other arguments as fmscan_backward, cached_output included: without FMSCAN_FLAG_PLAIN it
+ * must be the forward call's output for these gates and tokens and is read at one position per
+ * row and tile (the element before the tile, and h[0]); the rest is made again from gates and
+ * input_tokens. Needs 16-byte aligned pointers and
  * L * sizeof(element) % 16 == 0 (FMSCAN_E_UNALIGNED otherwise: use fmscan_backward);
  * flags: only FMSCAN_FLAG_PLAIN.
  */
@@ -209,12 +219,13 @@ int fmscan_backward_reduced(const void* gates, const void* out_grad, const void*
  * the read-out alone when coef_out = read, coef_self = 0 and states_n = cached_output.
  *   states_n   (B, M, D, L)  the normalised states      coef_out, coef_self  (B, M, L) float32
  *   out_grad   (B, D, L)     gradient of the layer's output, time last
- * states_n and out_grad of the call's dtype. cached_output may be NULL when rms ((B, M, L)
- * float32, 1 / inv_rms:
+ * states_n and out_grad of the call's dtype. cached_output, when given, is the forward
+ * call's output for these gates and tokens, read as fmscan_backward_reduced reads it (one
+ * position per row and tile). It may be NULL when rms ((B, M, L) float32, 1 / inv_rms:
  * fmscan_readout_dot writes it) is given: the scanned states are then taken back from the
- * normalised ones, states_n * rms, and the layer need not keep them (the reference keeps
- * them for autograd, fm/scan/fm_scan.py:53-55). Everything else, and the limits, as
- * fmscan_backward_reduced.
+ * normalised ones, states_n * rms (every element of states_n is read anyway), and the layer
+ * need not keep them (the reference keeps them for autograd, fm/scan/fm_scan.py:53-55).
+ * Everything else, and the limits, as fmscan_backward_reduced.
  */
 int fmscan_backward_layer(const void* gates, const void* states_n,
                           const float* coef_out, const float* coef_self, const void* out_grad,

@@ -199,13 +199,17 @@ def readout_backward(out_grad, ext_grad, read, states, mem_norm=True, eps=1e-6):
 
 def _layer_operands(alpha, update_scale, output_scale, inputs, storage):
     """gates (B, M, L), tokens (B, D, L), read (B, M, L) as the layer hands them to the scan and
-    the read-out. `storage`, when given, rounds an array to the layer's storage dtype: the
-    reference materialises the gates and the read weights in that dtype before the scan sees
-    them (fm_scan.py:116-119,130 are PyTorch operations on bfloat16 tensors), and a gate near
-    one moves by up to 2^-9 when stored in bfloat16, which changes the decay it stands for.
-    A comparison with a storage-dtype implementation therefore starts from the stored gates."""
+    the read-out. `storage`, when given, rounds an array to the layer's storage dtype, and it is
+    applied wherever the reference holds a tensor of that dtype: fm_scan.py:116 makes
+    `update_weight = alpha * update_scale` (one tensor, rounded), :119 makes
+    `decay_weight = 1.0 - update_weight` from the rounded product (a second tensor, rounded
+    again), :130 makes `alpha * output_scale` (rounded once). Two roundings for the gates, not
+    one: 1 - round(a * u) and round(1 - a * u) differ by a unit in the last place for about one
+    gate in a hundred, and a gate near one moves by up to 2^-9 per rounding in bfloat16, which
+    changes the decay it stands for. Pinned bit for bit against those PyTorch operations on
+    bfloat16, float16 and float32 tensors in tests/test_oracle.py."""
     storage = storage or (lambda a: a)
-    write = np.ascontiguousarray(np.transpose(alpha * update_scale, (0, 2, 1)))        # :116,118
+    write = storage(np.ascontiguousarray(np.transpose(alpha * update_scale, (0, 2, 1))))  # :116,118
     tokens = np.ascontiguousarray(np.transpose(inputs, (0, 2, 1)))                    # :117
     gates = storage(1.0 - write)                                                       # :119
     read = storage(np.ascontiguousarray(np.transpose(alpha * output_scale, (0, 2, 1))))  # :130

@@ -111,6 +111,10 @@ def main():
         make_case("plain_with_state", 2, 2, 2, 6, seed=5, plain=True, zero_state=False),
         make_case("fm_gates_outside_unit_interval", 1, 2, 2, 5, seed=6, plain=False, zero_state=False,
                   special="gates_above_one"),
+        # rows of 8 float32 = 32 bytes: 16-byte vector access on the GPU, and M > 1 with D > 1 for the
+        # backward kernel that sums over d and m itself
+        make_case("fm_vector_rows", 2, 3, 2, 8, seed=7, plain=False, zero_state=False),
+        make_case("plain_vector_rows", 1, 2, 3, 8, seed=8, plain=True, zero_state=False),
     ]
     OUT.write_text(json.dumps({"cases": cases}, indent=None, separators=(",", ":")) + "\n")
     print("wrote", OUT, OUT.stat().st_size, "bytes")

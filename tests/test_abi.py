@@ -88,6 +88,7 @@ def test_rejected_arguments(lib):
     assert fwd(lib, flags=0x2) == E_FLAGS
     assert fwd(lib, flags=3 << 8) == E_FLAGS          # 3 waves per row is not offered
     assert fwd(lib, flags=5 << 16) == E_FLAGS         # prefetch depth 5 is not offered
+    assert fwd(lib, flags=3 << 16) == E_FLAGS         # nor 3: the library holds depths 2 and 4
     assert fwd(lib, flags=1 << 28) == E_FLAGS         # unknown bit
     assert fwd(lib, L=1 << 16, flags=4 << 20) == E_WORKSPACE   # 4 segments asked for, no workspace
     assert b"workspace" in lib.fmscan_last_error()
@@ -231,15 +232,15 @@ def test_workspace_bytes(lib):
 
 
 def test_streaming_probe_library_rejects_what_it_does_not_cover():
-    """bench.py's bare streaming kernel lives in a library of its own; no GPU is needed to see it refuse."""
+    """bench.py's bare streaming kernel lives in a library of its own, outside the package (bench.py builds it
+    when it is not there); no GPU is needed to see it refuse."""
+    import sys
+    sys.path.insert(0, str(ROOT))
+    import bench
+
+    f = bench.load_probe().fmscan_probe_stream
     from fm_amd import build
-    if not build.PROBE_LIB.exists():
-        build.build_probe(verbose=False)
-    probe = ctypes.CDLL(str(build.PROBE_LIB))
-    f = probe.fmscan_probe_stream
-    f.restype = ctypes.c_int
-    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
-                  ctypes.c_int, ctypes.c_void_p]
+    assert not hasattr(build, "PROBE_LIB") and not list((ROOT / "fm_amd").rglob("*probe*"))  # not in the product
     a, b = 1 << 20, 1 << 30
     assert f(None, b, 4, 1024, 2, 1, 2, None) == -1        # no input
     assert f(a, b, 4, 1000, 2, 1, 2, None) == -1           # a row is not whole steps

@@ -224,6 +224,26 @@ def test_empty_problems_pass_through(scan, shape):
         assert t.grad is not None and t.grad.shape == t.shape and not t.grad.float().abs().sum().item()
 
 
+def test_layer_rejects_a_misplaced_initial_state(scan):
+    """An initial state on the host, or of another dtype than the rest, is an error raised in Python
+    (the fused forward route passes raw pointers: it must never reach a kernel), for shapes of both routes;
+    a valid call still works afterwards."""
+    for (B, L, M, D) in ((2, 512, 4, 24), (1, 1001, 3, 12)):
+        dt = torch.bfloat16
+        alpha = torch.softmax(torch.randn(B, L, M, device=DEV), -1).to(dt)
+        us, osc = torch.rand(B, L, 1, device=DEV).to(dt), torch.rand(B, L, 1, device=DEV).to(dt)
+        inp = torch.randn(B, L, D, device=DEV).to(dt)
+        h0 = torch.randn(B, M, D, device=DEV)
+        with pytest.raises(RuntimeError, match="initial_state has dtype"):
+            scan.fm_memory(alpha, us, osc, inp, h0)  # float32 state, bfloat16 layer
+        with pytest.raises(RuntimeError, match="GPU tensor"):
+            scan.fm_memory(alpha, us, osc, inp, h0.to(dt).cpu())
+        with pytest.raises(RuntimeError, match="initial_state must be"):
+            scan.fm_memory(alpha, us, osc, inp, torch.zeros(B, M, D + 1, dtype=dt, device=DEV))
+        y, mem = scan.fm_memory(alpha, us, osc, inp, h0.to(dt))
+        assert torch.isfinite(y.float()).all() and torch.isfinite(mem.float()).all()
+
+
 def test_layer_with_more_than_2_31_state_elements(scan):
     """(B, L, M, D) = (9, 65536, 32, 128): 2^31 + 2^28 elements of the states, which the reference's
     32-bit indices could not address (fm_scan.cuh:76-82). Batch elements are independent and every

@@ -5,7 +5,10 @@ Tolerance (stated by the benchmark definition): normwise error against the float
 sequential oracle evaluated on the same, already quantised inputs,
     max|y - ref| / max|ref| <= tol   and   ||y - ref||_2 / ||ref||_2 <= tol,
 tol = 1e-5 for float32, 1e-2 for bfloat16 / float16. Backward is checked against
-the oracle fed with the states the GPU stored, which is what the kernel reads.
+the oracle fed with the states the GPU stored: the plain form reads them all, the
+default form reads one of them per wave and tile and makes the others again from the
+gates and tokens in float32 (closer to the exact states than the stored ones by up to
+one rounding of the storage type, which the tolerance covers).
 Where the arithmetic allows it the checks are bit-exact (resets, scaling by two,
 row permutation, run-to-run determinism).
 """
@@ -207,6 +210,119 @@ def test_shapes_and_variants(scan, dtype, waves, plain):
         check(tag + " states", out, h_ref, TOL[dtype])
         check(tag + " token grad", dx, tg, TOL[dtype])
         check(tag + " gate grad", dg, gg, TOL[dtype])
+
+
+def test_every_compiled_variant_runs_once(scan):
+    """A fixed-seed walk over the kernel variants the library holds, each asked for explicitly through the
+    flags: element type x waves per row (1, 2, 4, 8) x prefetch depth (2, 4) x plain / FM form x access
+    (fold rows with 16-byte vectors, shared rows with 16-byte vectors, rows off 16-byte alignment), with
+    the cap on resident blocks cycling through its range; then the same for rows cut into segments, and
+    the 16-wave backward that only the library chooses, with shared rows. Random small shapes, forward
+    and backward against the compiled float64 oracle at the usual tolerance."""
+    rnd = np.random.default_rng(20240607)
+    caps = [1, 2, 3, 4, 6, 8, 12, 15]
+    n = 0
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        vec = 16 // torch.empty(0, dtype=dtype).element_size()  # elements per 16 bytes
+        for waves in (1, 2, 4, 8):
+            for depth in (2, 4):
+                for plain in (False, True):
+                    for access in ("fold", "shared", "unaligned"):
+                        tile = vec * 64 * waves
+                        # a few tiles, so that the loops with unchecked whole tiles (2 * depth and more) and
+                        # the checked ends both run; every third case is shorter than that
+                        tiles = int(rnd.integers(1, 4)) if n % 3 == 0 else int(rnd.integers(2 * depth, 3 * depth + 2))
+                        L = tiles * tile - int(rnd.integers(0, tile // vec)) * vec
+                        if access == "unaligned":
+                            L += int(rnd.integers(1, vec))
+                        B = int(rnd.integers(1, 4))
+                        M, D = (1, 1) if access == "fold" else (int(rnd.integers(1, 4)), int(rnd.integers(2, 5)))
+                        if access == "fold":
+                            B = int(rnd.integers(3, 9))
+                        gen = torch.Generator().manual_seed(1000 + n)
+                        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+                        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+                        G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+                        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+                        fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+                        kw = dict(plain=plain, waves_per_row=waves, depth=depth, blocks_per_cu=caps[n % len(caps)])
+                        tag = f"case {n}: {(B, M, D, L)} {dtype} {access} {kw}"
+                        print(tag, flush=True)
+                        out, dx, dg = run_fwd_bwd(scan, g, x, G, h0, fpg, **kw)
+                        h_ref = C.forward_f64(g, x, h0, plain)
+                        tg, gg = C.backward_f64(g, G, out, x, fpg, h0, plain)
+                        check(tag + " states", out, h_ref, TOL[dtype])
+                        check(tag + " token grad", dx, tg, TOL[dtype])
+                        check(tag + " gate grad", dg, gg, TOL[dtype])
+                        n += 1
+        # rows cut into segments (single waves, both depths), and 16 waves per row in backward with shared rows
+        for depth, segments, (B, M, D, L) in ((2, 3, (2, 1, 1, 40 * vec * 64)), (4, 5, (1, 2, 2, 50 * vec * 64 + vec)),
+                                              (2, 0, (2, 4, 5, 70 * vec * 64)), (4, 0, (3, 2, 7, 64 * vec * 64 + 3))):
+            for plain in (False, True):
+                gen = torch.Generator().manual_seed(2000 + n)
+                g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+                x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+                G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+                h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+                fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+                kw = dict(plain=plain, depth=depth, segments=segments)
+                tag = f"case {n}: {(B, M, D, L)} {dtype} {kw}"
+                print(tag, flush=True)
+                out, dx, dg = run_fwd_bwd(scan, g, x, G, h0, fpg, **kw)
+                h_ref = C.forward_f64(g, x, h0, plain)
+                tg, gg = C.backward_f64(g, G, out, x, fpg, h0, plain)
+                check(tag + " states", out, h_ref, TOL[dtype])
+                check(tag + " token grad", dx, tg, TOL[dtype])
+                check(tag + " gate grad", dg, gg, TOL[dtype])
+                n += 1
+    assert n == 3 * (4 * 2 * 2 * 3 + 8)
+
+
+def test_exact_rational_vectors_on_the_gpu(scan, exact_cases):
+    """The committed exact vectors (tests/golden/fm_scan_exact.json: small problems solved in rational
+    arithmetic, derivatives by dual numbers) through fmscan_forward, fmscan_backward and, where the shape
+    fits it, fmscan_backward_reduced. Every input is a small dyadic rational that float32, float16 and
+    bfloat16 hold exactly, so the only error is the kernels' own arithmetic: 1e-6 in float32 (the states
+    need up to 27 bits, more than a float32 holds: not bit-exact), the storage type's 1e-2 otherwise."""
+    lib, st = scan.module, torch.cuda.current_stream().cuda_stream
+    for name, c in exact_cases.items():
+        B, M, D, L, plain = c["B"], c["M"], c["D"], c["L"], c["plain"]
+        a = lambda k: np.array(c[k], dtype=np.float64)
+        for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2), (torch.float16, 1e-2)):
+            t = lambda k: torch.from_numpy(a(k)).to(dtype).to(DEV)
+            g, x, G, h0, fpg = t("gates"), t("tokens"), t("out_grad"), t("initial_state"), t("first_prop_grad")
+            for k, v in (("gates", g), ("tokens", x), ("out_grad", G), ("initial_state", h0), ("first_prop_grad", fpg)):
+                assert np.array_equal(v.double().cpu().numpy(), a(k)), (name, k, dtype)  # held exactly
+            out = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+            dx, dg, dh0 = torch.empty_like(out), torch.empty_like(out), torch.empty_like(h0)
+            scan.fm_scan_forward(g, x, h0, out, plain=plain)
+            tag = f"{name} {dtype}"
+            check(tag + " states", out, a("states"), tol)
+            if dtype == torch.float32 and L == 1:
+                assert np.array_equal(out.double().cpu().numpy(), a("states")), tag  # one step: representable, exact
+            # backward from the exact states (what a float64 forward would have stored, rounded to the dtype)
+            saved = t("states")
+            scan.fm_scan_backward(g, G, fpg, dx, saved, x, dg, initial_state=h0, initial_state_grad=dh0, plain=plain)
+            check(tag + " token grad", dx, a("token_grad"), tol)
+            check(tag + " gate grad", dg, a("gate_grad"), tol)
+            check(tag + " initial state grad", dh0, a("d_initial_state"), tol)
+            aligned = (L * out.element_size()) % 16 == 0
+            if M > 1 and D > 1 and aligned:
+                dh0r = torch.empty_like(h0)
+                d_g, d_x = scan.fm_scan_backward_reduced(g, G, fpg, saved, x, initial_state=h0,
+                                                         initial_state_grad=dh0r, plain=plain)
+                check(tag + " d_gates (sums inside)", d_g, a("gate_grad").sum(axis=2), tol)
+                check(tag + " d_tokens (sums inside)", d_x, a("token_grad").sum(axis=1), tol)
+                check(tag + " initial state grad (sums inside)", dh0r, a("d_initial_state"), tol)
+            elif M > 1 and D > 1:
+                groups = lib.fmscan_reduced_groups(B, D)
+                part = torch.empty(B, M, groups, L, device=DEV)
+                dxr = torch.empty(B, D, L, dtype=dtype, device=DEV)
+                code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+                rc = lib.fmscan_backward_reduced(g.data_ptr(), G.data_ptr(), fpg.data_ptr(), dxr.data_ptr(),
+                                                 saved.data_ptr(), x.data_ptr(), part.data_ptr(), None, None,
+                                                 B, M, D, L, code, 1 if plain else 0, st)
+                assert rc == -7, (tag, rc)  # rows that are not 16-byte multiples: refused, nothing launched
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
@@ -562,6 +678,66 @@ def test_notebook_design(scan):
     check("d_tokens", res["fp32"][1], d_x, 1e-5)
 
 
+def test_notebook_usage_cell_shape(scan):
+    """The reference's usage cell (fm_test.ipynb:29-45): batch 1, dim 2048, seqlen 8192, mem 32, bfloat16;
+    fm_scan on gates 0.9 + 0.1 rand and tokens rand, then fm_memory on alpha = softmax(rand), scales
+    rand + 0.001, inputs rand, mem_norm, eps 1e-6. The notebook only prints shapes; here the results are
+    checked. fm_scan: states and both gradients (upstream gradient randn) against the compiled float64
+    oracle on sampled slots and channels, every step of their rows. fm_memory: see below."""
+    B, D, L, M, dt = 1, 2048, 8192, 32, torch.bfloat16
+    gen = gpu_gen(29)
+    gates = (0.9 + 0.1 * torch.rand(B, M, L, device=DEV, generator=gen)).to(dt).requires_grad_()
+    tokens = torch.rand(B, D, L, device=DEV, generator=gen).to(dt).requires_grad_()
+    states = scan.fm_scan(gates, tokens, initial_state=None)
+    assert tuple(states.shape) == (B, M, D, L) and states.dtype == dt
+    G = torch.randn(B, M, D, L, device=DEV, generator=gen).to(dt)
+    states.backward(G)
+    torch.cuda.synchronize()
+    g, x, h = gates.detach(), tokens.detach(), states.detach()
+    ms, ds = [0, 13, 31], [0, 1, 777, 2047]
+    for m in ms:  # a slot with all its channels: the states of sampled channels, and d_gates (a sum over all d)
+        gm, Gm, hm = g[:, m:m + 1], G[:, m:m + 1], h[:, m:m + 1]
+        h_ref = C.forward_f64(gm, x[:, ds])
+        check(f"states of slot {m}", hm[:, :, ds], h_ref, TOL[dt])
+        _, gg = C.backward_f64(gm, Gm, hm, x, None, np.zeros((B, 1, D)))
+        check(f"d_gates of slot {m}", gates.grad[:, m:m + 1], gg.sum(axis=2), TOL[dt])
+    tg, _ = C.backward_f64(g, G[:, :, ds].contiguous(), h[:, :, ds].contiguous(), x[:, ds].contiguous(), None,
+                           np.zeros((B, M, len(ds))))
+    check("d_tokens of sampled channels", tokens.grad[:, ds], tg.sum(axis=1), TOL[dt])
+    del G, states, h, tg
+    gates.grad = tokens.grad = None
+    torch.cuda.empty_cache()
+
+    # fm_memory at the same shape. The float64 oracle of the whole layer on 2^29 states would take minutes
+    # and tens of GiB, so the check leans on causality: outputs and memory states up to step T0 depend on
+    # the inputs up to T0 only, and with a loss that weighs the output up to T0 only, every gradient is
+    # that of the layer cut at T0 (and exactly zero afterwards). The oracle runs on that cut, 640 steps: a
+    # whole tile of 512 and a part of the next. The kernels run over all 8192 steps of the D = 2048 route
+    # (scan with the sums of squares per block of rows, groups of 8 channels in backward).
+    T0 = 640
+    alpha = torch.softmax(torch.rand(B, L, M, device=DEV, generator=gen).to(dt).float(), -1).to(dt).requires_grad_()
+    us = (torch.rand(B, L, 1, device=DEV, generator=gen) + 0.001).to(dt).requires_grad_()
+    osc = (torch.rand(B, L, 1, device=DEV, generator=gen) + 0.001).to(dt).requires_grad_()
+    inp = torch.rand(B, L, D, device=DEV, generator=gen).to(dt).requires_grad_()
+    out, mem = scan.fm_memory(alpha, us, osc, inp, initial_state=None, mem_norm=True, norm_eps=1e-6)
+    assert tuple(out.shape) == (B, L, D) and tuple(mem.shape) == (B, M, D, L) and out.dtype == dt
+    w = torch.randn(B, L, D, device=DEV, generator=gen).to(dt)
+    w[:, T0:] = 0
+    (out.float() * w.float()).sum().backward()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(mem.float()).all()
+    rounded = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dt).to(torch.float64).numpy()
+    cut = lambda t: t.detach()[:, :T0].double().cpu()
+    a, u, o, xi, wc = cut(alpha), cut(us), cut(osc), cut(inp), cut(w)
+    o_out, o_mem = O.memory_forward(a, u, o, xi, None, True, 1e-6, rounded)
+    want = O.memory_backward(a, u, o, xi, wc, None, None, True, 1e-6, rounded)
+    check("fm_memory output up to T0", out[:, :T0], o_out, TOL[dt])
+    check("fm_memory memory states up to T0", mem[..., :T0], o_mem, TOL[dt])
+    for name, leaf in (("d_alpha", alpha), ("d_update_scale", us), ("d_output_scale", osc), ("d_inputs", inp)):
+        check(f"fm_memory {name} up to T0", leaf.grad[:, :T0], want[name], TOL[dt])
+        assert not leaf.grad[:, T0:].float().abs().max().item(), name + " beyond the last weighted step"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_autograd_with_initial_state(scan, dtype):
     """FM_Scan with a non-zero initial state: gradients equal the derivative of the
@@ -748,9 +924,9 @@ def test_layer_form_of_the_backward_kernel_through_the_c_abi(scan, dtype, plain)
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_layer_prepare_and_finish_kernels(scan, dtype):
-    """The layer's small tensors: gates and read weights with time last, and the gradients of
-    alpha and the two scales from those of gates (as partial sums) and read; against the same
-    formulas in float64."""
+    """The layer's small tensors: gates and read weights with time last, bit for bit as the
+    reference's PyTorch lines form them; and the gradients of alpha and the two scales from those
+    of gates (as partial sums) and read, against the same formulas in float64."""
     lib, st = scan.module, torch.cuda.current_stream().cuda_stream
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
     for (B, L, M, G) in [(2, 64, 3, 1), (1, 1000, 33, 2), (3, 130, 70, 3), (2, 2048, 32, 16), (1, 5, 1, 1)]:
@@ -763,8 +939,18 @@ def test_layer_prepare_and_finish_kernels(scan, dtype):
                                         read.data_ptr(), B, L, M, code, st) == 0
         a64, u64, o64 = (O.to_f64(t) for t in (alpha, us, osc))
         tag = f"{(B, L, M, G)} {dtype}"
-        check(tag + " gates", gates, np.transpose(1.0 - a64 * u64, (0, 2, 1)), 1e-6 if dtype == torch.float32 else 4e-3)
-        check(tag + " read", read, np.transpose(a64 * o64, (0, 2, 1)), 1e-6 if dtype == torch.float32 else 4e-3)
+        # bit for bit what the reference's lines give (fm_scan.py:116-119,130), evaluated by PyTorch on
+        # CPU tensors of the storage type: the product is a tensor of its own, so the gates are
+        # rounded twice; and the same from the oracle's layer, which the layer tests compare with
+        a_c, u_c, o_c = alpha.cpu(), us.cpu(), osc.cpu()
+        want_gates = 1.0 - (a_c * u_c).transpose(1, 2).contiguous()
+        want_read = (a_c * o_c).transpose(1, 2).contiguous()
+        assert torch.equal(gates.cpu(), want_gates), tag + " gates"
+        assert torch.equal(read.cpu(), want_read), tag + " read"
+        rounded = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dtype).to(torch.float64).numpy()
+        o_gates, _, o_read = O._layer_operands(a64, u64, o64, np.zeros((B, L, 1)), rounded)
+        assert np.array_equal(gates.double().cpu().numpy(), o_gates), tag + " gates vs oracle"
+        assert np.array_equal(read.double().cpu().numpy(), o_read), tag + " read vs oracle"
         partial = torch.randn(B, M, G, L, generator=gen).to(DEV)
         q = torch.randn(B, M, L, generator=gen).to(DEV)
         d_alpha, d_us, d_os = torch.empty_like(alpha), torch.empty_like(us), torch.empty_like(osc)

@@ -59,6 +59,45 @@ def test_cpu_tensors_are_rejected_loudly():
         fm_memory(torch.rand(1, 32, 2), torch.rand(1, 32, 1), torch.rand(1, 32, 1), torch.rand(1, 32, 3))
 
 
+def test_layer_checks_every_tensor_before_anything_is_launched(monkeypatch):
+    """fm_memory / fm_layer hand raw pointers to the library; every tensor that goes there is checked for
+    device, dtype, contiguity and shape first, whichever route the shape then takes. Run on the CPU with
+    the device test relaxed to "same device as the gates" and a library that fails the test when called."""
+    import fm_amd.scan.fm_scan as m
+
+    class NoLaunch:
+        def __getattr__(self, name):
+            raise AssertionError(f"{name} was called before the arguments were checked")
+
+    def same_device(name, t, dev):
+        m._require(t.device == dev, f"{name} is on {t.device}, expected {dev}")
+
+    monkeypatch.setattr(m, "_raw", NoLaunch())
+    monkeypatch.setattr(m, "_on_gpu", same_device)
+    B, M, D, L = 2, 3, 4, 64
+    g, x, r = torch.rand(B, M, L), torch.rand(B, D, L), torch.rand(B, M, L)
+    h0 = torch.rand(B, M, D)
+    bad = [
+        (dict(initial_state=h0.to("meta")), "initial_state is on meta"),
+        (dict(initial_state=h0.double()), "initial_state has dtype"),
+        (dict(initial_state=h0.to(torch.bfloat16)), "initial_state has dtype"),
+        (dict(initial_state=torch.rand(B, D, M).transpose(1, 2)), "initial_state must be contiguous"),
+        (dict(initial_state=torch.rand(B, M, D + 1)), "initial_state must be"),
+        (dict(read=r.to("meta")), "read is on meta"),
+        (dict(read=r.half()), "read has dtype"),
+        (dict(read=torch.rand(B, M + 1, L)), "read must be"),
+        (dict(tokens=x.to("meta")), "tokens is on meta"),
+        (dict(tokens=x.to(torch.float16)), "tokens has dtype"),
+        (dict(tokens=torch.rand(B, D, L + 8)), "must agree in B and L"),
+    ]
+    for mem_norm in (True, False):
+        for change, message in bad:
+            args = dict(gates=g, tokens=x, initial_state=h0, read=r)
+            args.update(change)
+            with pytest.raises(RuntimeError, match=message):
+                m._layer_forward(args["gates"], args["tokens"], args["initial_state"], args["read"], mem_norm, 1e-6)
+
+
 def test_fm_scan_shape_asserts_match_reference_behaviour():
     from fm.scan.fm_scan import fm_scan
 

@@ -30,7 +30,7 @@ def rand_problem(B, M, D, L, seed=0, state=True):
 # ------------------------------------------------------------------ exact vectors
 
 CASES = ["fm_zero_state", "fm_with_state", "fm_single_row", "fm_length_one", "plain_with_state",
-         "fm_gates_outside_unit_interval"]
+         "fm_gates_outside_unit_interval", "fm_vector_rows", "plain_vector_rows"]
 
 
 @pytest.mark.parametrize("name", CASES)
@@ -361,6 +361,40 @@ def test_memory_backward_against_autograd_and_finite_differences(mem_norm, loss_
 
     for name, arr in zip(names, (alpha, us, osc, x, h0)):
         np.testing.assert_allclose(got[name], fd_grad(f, arr), rtol=2e-6, atol=1e-7, err_msg=name)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_layer_operands_round_where_the_reference_holds_a_tensor(dtype):
+    """The `storage=` branch of the oracle's layer: gates and read weights bit for bit what the PyTorch
+    operations of fm_scan.py:116-119,130 give on tensors of the storage type,
+        update_weight = alpha * update_scale; update_weight.transpose(1, 2).contiguous();
+        decay_weight = 1.0 - update_weight;  output_weight = alpha * output_scale
+    (evaluated here by PyTorch on CPU tensors, not retyped): the product is a tensor of its own, so the
+    gate is rounded twice. The single-rounded gate round(1 - alpha * update_scale) must differ from it
+    somewhere in the 16-bit types, or this test could not tell the two orders apart."""
+    gen = torch.Generator().manual_seed(7)
+    B, L, M = 3, 257, 32
+    alpha = torch.softmax(torch.randn(B, L, M, generator=gen), -1).to(dtype)
+    us = torch.rand(B, L, 1, generator=gen).to(dtype)
+    osc = torch.rand(B, L, 1, generator=gen).to(dtype)
+    want_gates = 1.0 - (alpha * us).transpose(1, 2).contiguous()
+    want_read = (alpha * osc).transpose(1, 2).contiguous()
+    assert want_gates.dtype == dtype and want_read.dtype == dtype
+
+    storage = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dtype).to(torch.float64).numpy()
+    x = np.zeros((B, L, 1))
+    gates, _, read = O._layer_operands(O.to_f64(alpha), O.to_f64(us), O.to_f64(osc), x, storage)
+    assert np.array_equal(gates, want_gates.double().numpy())
+    assert np.array_equal(read, want_read.double().numpy())
+
+    once = storage(1.0 - np.transpose(O.to_f64(alpha) * O.to_f64(us), (0, 2, 1)))
+    differ = np.mean(once != gates)
+    if dtype != torch.float32:
+        assert 1e-3 < differ < 0.1, differ  # about one gate in a hundred, each by one unit in the last place
+    # without `storage` nothing is rounded: the float64 layer the other tests pin
+    g64, _, r64 = O._layer_operands(O.to_f64(alpha), O.to_f64(us), O.to_f64(osc), x, None)
+    assert np.array_equal(g64, 1.0 - np.transpose(O.to_f64(alpha) * O.to_f64(us), (0, 2, 1)))
+    assert np.array_equal(r64, np.transpose(O.to_f64(alpha) * O.to_f64(osc), (0, 2, 1)))
 
 
 def test_norm_gradient_with_one_channel_is_all_cancellation():
