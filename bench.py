@@ -18,6 +18,10 @@ same K steps right after. `cpu_baseline` times the compiled CPU
 port of the same scan (oracle/fmscan_cpu.c) on this host's cores on a bounded
 row sample of the same workload.
 
+The default run also carries `per_config`: the same step timed the same way on the other
+benchmark configurations (cfg1, cfg2, cfg4, cfg5, cfg5 in float16) and on the layer, after the
+headline's timed region (20 steps each; `--workload X` prints the full line for one of them).
+
 `--workload layer` is a secondary measurement, the Factorization-Memory layer
 around the scan (`fm_memory`: scan, RMS norm over D, read-out over M) at the
 FM-native reading of configuration 5, (B, L, M, D) = (32, 2048, 32, 128) bfloat16:
@@ -241,13 +245,90 @@ def reference_cpu_path(torch, g, x, G):
             "elements_per_s": round(n / (t2 - t0), 1), "fwd_s": round(t1 - t0, 3), "bwd_s": round(t2 - t1, 3)}
 
 
+def scan_buffers(torch, g, x, G, waves_per_row=0):
+    """Pre-allocated outputs of one workload and the step over them: one forward scan and one
+    backward scan through the extension entry points, optionally with events around each."""
+    from fm.scan.fm_scan import fm_scan_backward, fm_scan_forward
+
+    rows, _, T = g.shape
+    zeros = torch.zeros(rows, 1, 1, dtype=g.dtype, device=g.device)
+    out = torch.empty(rows, 1, 1, T, dtype=g.dtype, device=g.device)
+    dx, dg = torch.empty_like(out), torch.empty_like(out)
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        fm_scan_forward(g, x, zeros, out, waves_per_row=waves_per_row)
+        if ev:
+            ev[1].record()
+        fm_scan_backward(g, G, zeros, dx, out, x, dg, waves_per_row=waves_per_row)
+        if ev:
+            ev[2].record()
+
+    return zeros, out, dx, dg, step
+
+
+def time_steps(torch, step, steps, warmup):
+    """(wall seconds of `steps` steps that hold nothing but the calls, forward kernel ms, backward
+    kernel ms). The split between the two kernels comes from a pass of its own right after: the
+    kernels run on torch's current stream, so torch events bracket them (kept out of the timed steps,
+    where they would be extra work in the stream)."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for k in range(steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / steps
+    return elapsed, fwd_ms, bwd_ms
+
+
+def per_config(torch, dev, skip, steps, warmup):
+    """Every benchmark configuration but `skip` (the headline, timed before), and the layer: the same
+    step, the same timing, fewer fields. Effective GB/s prices a step at 9 element sizes per element
+    (forward 3, backward 6), moved GB/s at the 8 the kernels move."""
+    out = {}
+    for name, (B, Cn, T, dtn) in WORKLOADS.items():
+        if name == skip:
+            continue
+        g, x, G = make_inputs(torch, name, dev)
+        buffers = scan_buffers(torch, g, x, G)
+        elapsed, fwd_ms, bwd_ms = time_steps(torch, buffers[-1], steps, warmup)
+        s, N = g.element_size(), B * Cn * T
+        ms = elapsed * 1e3 / steps
+        out[name] = {"workload": f"(B,C,T)=({B},{Cn},{T}) {dtn}", "ms_per_step": round(ms, 4),
+                     "GBps": round(9 * s * N / ms / 1e6, 1), "pct_of_peak": round(9 * s * N / ms / 1e6 / PEAK_HBM_GBPS * 100, 2),
+                     "moved_GBps": round(8 * s * N / ms / 1e6, 1), "elements_per_s": round(N / ms * 1e3, 1),
+                     "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
+                     "fwd_frac_of_peak": round(3 * s * N / fwd_ms / 1e6 / PEAK_HBM_GBPS, 4),
+                     "bwd_frac_of_peak": round(6 * s * N / bwd_ms / 1e6 / PEAK_HBM_GBPS, 4),
+                     "bwd_frac_of_moved_bytes": round(5 * s * N / bwd_ms / 1e6 / PEAK_HBM_GBPS, 4)}
+        del g, x, G, buffers
+        torch.cuda.empty_cache()
+    step, N, name = layer_step(torch, dev)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    out["layer"] = {"workload": name, "ms_per_step": round(ms, 4), "Gelem_per_s": round(N / ms / 1e6, 2)}
+    return out
+
+
 LAYER = (32, 2048, 32, 128, "bfloat16")  # B, L, M, D
 
 
-def run_layer(torch, args) -> int:
-    import fm.scan.fm_scan as S
-
-    dev = torch.device("cuda", 0)
+def layer_inputs(torch, dev):
     B, L, M, D, dtn = LAYER
     dt = getattr(torch, dtn)
     gen = torch.Generator(device=dev).manual_seed(0)
@@ -257,6 +338,34 @@ def run_layer(torch, args) -> int:
     osc = torch.rand(B, L, 1, device=dev, generator=gen).to(dt).requires_grad_()
     inp = rn(B, L, D).to(dt).requires_grad_()
     w_out = rn(B, L, D).to(dt)
+    return alpha, us, osc, inp, w_out, gen
+
+
+def layer_step(torch, dev):
+    """(step, elements of the states, name): fm_memory forward + backward through autograd."""
+    import fm.scan.fm_scan as S
+
+    B, L, M, D, dtn = LAYER
+    alpha, us, osc, inp, w_out, _ = layer_inputs(torch, dev)
+    leaves = (alpha, us, osc, inp)
+
+    def step():
+        out, _ = S.fm_memory(alpha, us, osc, inp)
+        out.backward(w_out)
+        for t in leaves:
+            t.grad = None
+
+    return step, B * M * D * L, f"fm_memory (B,L,M,D)=({B},{L},{M},{D}) {dtn}, mem_norm, fwd+bwd via autograd"
+
+
+def run_layer(torch, args) -> int:
+    import fm.scan.fm_scan as S
+
+    dev = torch.device("cuda", 0)
+    B, L, M, D, dtn = LAYER
+    dt = getattr(torch, dtn)
+    alpha, us, osc, inp, w_out, gen = layer_inputs(torch, dev)
+    rn = lambda *sh: torch.randn(*sh, device=dev, generator=gen)
     leaves = (alpha, us, osc, inp)
 
     def step():
@@ -398,6 +507,9 @@ def main() -> int:
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["layer"])
     ap.add_argument("--waves-per-row", type=int, default=0, help="0 = library's choice")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-config", action="store_true",
+                    help="headline workload only: leave out the `per_config` object (the other benchmark "
+                         "configurations and the layer, timed after the headline)")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replays (what a launch-bound "
                          "caller, e.g. the small configuration 1, gets without the per-call Python cost)")
@@ -416,31 +528,16 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the scan has no CPU path to benchmark", file=sys.stderr)
         return 1
-    from fm.scan.fm_scan import fm_scan_backward, fm_scan_forward
-
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     if args.workload == "layer":
         return run_layer(torch, args)
     B, Cn, T, dtn = WORKLOADS[args.workload]
-    g, x, G = make_inputs(torch, args.workload, dev)
     rows = B * Cn
-    zeros = torch.zeros(rows, 1, 1, dtype=g.dtype, device=dev)
-    out = torch.empty(rows, 1, 1, T, dtype=g.dtype, device=dev)
-    dx, dg = torch.empty_like(out), torch.empty_like(out)
     W = args.waves_per_row
-
-    def step(ev=None):
-        if ev:
-            ev[0].record()
-        fm_scan_forward(g, x, zeros, out, waves_per_row=W)
-        if ev:
-            ev[1].record()
-        fm_scan_backward(g, G, zeros, dx, out, x, dg, waves_per_row=W)
-        if ev:
-            ev[2].record()
-
     if args.probe:
+        g, x, G = make_inputs(torch, args.workload, dev)
+        zeros, out, dx, dg, step = scan_buffers(torch, g, x, G, W)
         for _ in range(4):
             torch.neg(out, out=dx)
         for _ in range(4):
@@ -451,24 +548,9 @@ def main() -> int:
               f"backward {6 * g.element_size() * rows * T}")
         return 0
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    # the split between the two kernels, from a pass of its own: the kernels run on torch's current
-    # stream, so torch events bracket them (kept out of the timed steps, where they would be extra
-    # work in the stream)
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    for k in range(args.steps):
-        step(events[k])
-    torch.cuda.synchronize()
-
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    g, x, G = make_inputs(torch, args.workload, dev)
+    zeros, out, dx, dg, step = scan_buffers(torch, g, x, G, W)
+    elapsed, fwd_ms, bwd_ms = time_steps(torch, step, args.steps, args.warmup)
     s = g.element_size()
     N = rows * T
     ms_per_step = elapsed * 1e3 / args.steps
@@ -537,6 +619,11 @@ def main() -> int:
         result["cpu_baseline"] = cpu_baseline(torch, g, x, G)
         if args.workload == "cfg1":
             result["reference_cpu_path"] = reference_cpu_path(torch, g, x, G)
+    if args.workload == "cfg3" and not args.no_per_config:
+        # the other configurations and the layer, after the headline's timed region and with its tensors freed
+        del g, x, G, zeros, out, dx, dg, step
+        torch.cuda.empty_cache()
+        result["per_config"] = per_config(torch, dev, args.workload, steps=20, warmup=5)
     print(json.dumps(result), flush=True)
     return 0
 
