@@ -499,6 +499,100 @@ def layer_cpu_baseline(torch, alpha, us, osc, inp, w_out, batch=16):
                       f"backward once in {el:.1f} s, float64 numpy oracle oracle/fm_scan_oracle.py"}
 
 
+GRID_ROWS = (256, 2048, 16384, 131072)
+GRID_L = (1024, 4096, 16384, 65536)
+GRID_NATIVE = ((32, 32, 64, 2048), (8, 16, 64, 16384), (4, 32, 1024, 4096), (1, 32, 1024, 8192))  # (B, M, D, L)
+GRID_MAX_ELEMENTS = 1 << 31  # per tensor; larger cells of the grid are left out
+
+
+def run_grid(torch, args) -> int:
+    """The library's choice of kernel variant against every variant a caller can ask for, off the
+    benchmark shapes: rows x L x {bfloat16, float32} in the fold mapping (M = D = 1), and a few
+    Factorization-Memory shapes with shared gate and token rows. Forward and backward kernels apart,
+    HIP events around `reps` launches after 3 untimed ones. One text line per cell and direction:
+    time and fraction of peak of the library's choice (on the metric's bytes, forward 3 and backward 6
+    element sizes per element, and on the bytes moved, 3 and 5), the best override (waves per row /
+    resident blocks per compute unit / prefetch depth), and how far the choice is behind it."""
+    from fm.scan.fm_scan import fm_scan_backward, fm_scan_forward
+
+    dev = torch.device("cuda", 0)
+    overrides = [(w, b, d) for w in (1, 2, 4, 8) for b in (1, 2, 4, 8) for d in (2, 4)]
+    raw = open(args.grid_raw, "w") if args.grid_raw else None
+
+    def timed(call):
+        """ms per launch: the better of two rounds of launches that fill about 3 ms each (5 to 100)."""
+        for _ in range(3):
+            call()
+        best, reps = None, 5
+        for _ in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                call()
+            b.record()
+            b.synchronize()
+            ms = a.elapsed_time(b) / reps
+            best = ms if best is None else min(best, ms)
+            reps = max(5, min(100, int(3.0 / ms)))
+        return best
+
+    print("# python bench.py --grid   (fold mapping: (rows, 1, L) gates and tokens; native: (B, M, D, L))")
+    print("# frac = of 8 TB/s on the metric's bytes / on the bytes moved; behind = library's time / best override's - 1")
+    print(f"# {'shape':<26} {'dtype':<9} {'dir':<4} {'lib ms':>9} {'frac':>6} {'moved':>6}   {'best override (w/b/d)':<22} {'ms':>9} {'behind':>7}")
+    worst = []
+    cells = [((r, 1, 1, L), dtn) for dtn in ("bfloat16", "float32") for r in GRID_ROWS for L in GRID_L]
+    cells += [(shape, "bfloat16") for shape in GRID_NATIVE]
+    for (B, M, D, L), dtn in cells:
+        dt = getattr(torch, dtn)
+        N = B * M * D * L
+        if N > GRID_MAX_ELEMENTS:
+            print(f"# {str((B, M, D, L)):<26} {dtn:<9} left out: more than 2^31 elements per tensor")
+            continue
+        gen = torch.Generator(device=dev).manual_seed(N % 9973)
+        g = (0.5 + 0.5 * torch.rand(B, M, L, device=dev, generator=gen)).to(dt)
+        x = torch.randn(B, D, L, device=dev, generator=gen).to(dt)
+        G = torch.randn(B, M, D, L, device=dev, generator=gen).to(dt)
+        zeros = torch.zeros(B, M, D, dtype=dt, device=dev)
+        out = torch.empty(B, M, D, L, dtype=dt, device=dev)
+        dx, dg = torch.empty_like(out), torch.empty_like(out)
+        s = g.element_size()
+        small = (B * M + B * D) * L  # gates and tokens
+        for direction in ("fwd", "bwd"):
+            if direction == "fwd":
+                run = lambda **kw: fm_scan_forward(g, x, zeros, out, **kw)
+                metric_bytes = moved_bytes = s * (N + small)
+                if M == 1 and D == 1:
+                    metric_bytes = moved_bytes = 3 * s * N
+            else:
+                run = lambda **kw: fm_scan_backward(g, G, zeros, dx, out, x, dg, **kw)
+                metric_bytes, moved_bytes = s * (4 * N + small), s * (3 * N + small)
+                if M == 1 and D == 1:
+                    metric_bytes, moved_bytes = 6 * s * N, 5 * s * N
+            lib_ms = timed(lambda: run())
+            best, best_ms = None, None
+            for (w, b, d) in overrides:
+                ms = timed(lambda: run(waves_per_row=w, blocks_per_cu=b, depth=d))
+                if raw:
+                    raw.write(json.dumps({"shape": [B, M, D, L], "dtype": dtn, "dir": direction, "w": w, "b": b, "d": d,
+                                          "ms": round(ms, 5)}) + "\n")
+                if best_ms is None or ms < best_ms:
+                    best, best_ms = (w, b, d), ms
+            lib_ms = min(lib_ms, timed(lambda: run()))  # once more, after the sweep: the better of two
+            if raw:
+                raw.write(json.dumps({"shape": [B, M, D, L], "dtype": dtn, "dir": direction, "w": 0, "b": 0, "d": 0,
+                                      "ms": round(lib_ms, 5)}) + "\n")
+                raw.flush()
+            behind = lib_ms / best_ms - 1.0
+            print(f"  {str((B, M, D, L)):<26} {dtn:<9} {direction:<4} {lib_ms:9.4f} {metric_bytes / lib_ms / 1e6 / PEAK_HBM_GBPS:6.3f} "
+                  f"{moved_bytes / lib_ms / 1e6 / PEAK_HBM_GBPS:6.3f}   {'%d/%d/%d' % best:<22} {best_ms:9.4f} {100 * behind:6.1f}%", flush=True)
+            if behind > 0.07:
+                worst.append(((B, M, D, L), dtn, direction, round(100 * behind, 1)))
+        del g, x, G, zeros, out, dx, dg
+        torch.cuda.empty_cache()
+    print(f"# cells where the library's choice is more than 7 % behind the best override: {worst if worst else 'none'}")
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -510,6 +604,10 @@ def main() -> int:
     ap.add_argument("--no-per-config", action="store_true",
                     help="headline workload only: leave out the `per_config` object (the other benchmark "
                          "configurations and the layer, timed after the headline)")
+    ap.add_argument("--grid", action="store_true",
+                    help="no benchmark line: a text table of the library's choice of kernel variant against "
+                         "every override, over a grid of shapes off the benchmark configurations")
+    ap.add_argument("--grid-raw", default="", help="with --grid: also write every timing, one JSON object a line, to this file")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replays (what a launch-bound "
                          "caller, e.g. the small configuration 1, gets without the per-call Python cost)")
@@ -530,6 +628,8 @@ def main() -> int:
         return 1
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.grid:
+        return run_grid(torch, args)
     if args.workload == "layer":
         return run_layer(torch, args)
     B, Cn, T, dtn = WORKLOADS[args.workload]

@@ -125,14 +125,19 @@ inline unsigned lds_share(unsigned blocks_per_cu) {
 
 // Waves per row, resident blocks per compute unit, prefetch depth and segments per row
 // when the caller leaves the choice to the library. The table comes from sweeps on an
-// MI355X over the benchmark shapes (rows x L): 131072 x 2048, 32768 x 16384, 4096 x 65536
-// in 16-bit types and 8192 x 4096 in float32, forward and backward separately. What it
-// encodes: one or two waves per row stream best when there are many rows of moderate
-// length; long rows want eight waves side by side (sixteen in backward, which only the library
-// chooses: 0.501 -> 0.478 ms at (4096 rows, 65536); forward gains nothing from them) so that fewer
-// rows are open at a time; with few rows a block per row keeps every compute unit busy. One to two waves
-// per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few rows
-// that even eight waves per row leave compute units idle (fewer than 32 rows), and a
+// MI355X over rows x row length x element type, forward and backward apart, every
+// combination of waves (1, 2, 4, 8), cap (1, 2, 4, 8) and depth (2, 4) a caller can ask for
+// (`python bench.py --grid` prints the choice against the best of them). What decides is
+// the length of a row in bytes and, for rows of 32 to 64 KiB, how many rows there are:
+//   up to 4 KiB     a wave per row, four rows per block, 4 to 8 blocks per compute unit;
+//   8 to 16 KiB     2 to 4 waves per row;
+//   32 to 64 KiB    with 32768 rows or more a wave per row and few rows open at a time (one or two
+//                   blocks per compute unit), with fewer rows 8 waves side by side;
+//   128 KiB up      8 waves per row, one block per compute unit, four tiles in flight (16 waves
+//                   in backward, which only the library chooses: 0.501 -> 0.478 ms at 4096 rows of
+//                   65536; forward gains nothing from them).
+// One to two waves per SIMD is where HBM efficiency peaks; more resident rows lower it. With so few
+// rows that even eight waves per row leave compute units idle (fewer than 32 rows), and a
 // workspace to hold the segment pairs, rows are cut into segments (two passes).
 struct Tuning {
     unsigned waves, blocks_per_cu, depth;
@@ -172,36 +177,53 @@ inline void plan_segments(const Problem& pb, Tuning& t, bool may_split) {
 inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
     Tuning t;
     const int64_t tile1 = (16 / pb.esize) * 64;          // elements one wave covers per tile
-    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;   // tiles per row for one wave
+    const int64_t tiles1 = (pb.L + tile1 - 1) / tile1;   // tiles per row for one wave = KiB per row
     // Gates shared by D rows and tokens shared by M rows come from the caches: the kernel
     // then mostly writes (forward) and the limit on concurrent rows no longer applies.
-    // Measured on (B, M, D, L) = (32,32,128,2048), (1,32,2048,8192), (2,32,512,16384).
+    // Measured on (B, M, D, L) = (32,32,128,2048), (1,32,2048,8192), (2,32,512,16384), (4,32,1024,4096).
     const bool shared_inputs = pb.M > 1 || pb.D > 1;
-    const bool long_rows = tiles1 >= 64, few_rows = pb.rows < 16384 && tiles1 >= 8;
-    unsigned w = pb.waves;
-    if (!w) {
-        if (shared_inputs && pb.rows >= 16384) w = 1;
+    const bool many_rows = pb.rows >= 32768;
+    unsigned w, bpc, depth;
+    if (shared_inputs) {
+        const bool long_rows = tiles1 >= 64, few_rows = pb.rows < 16384 && tiles1 >= 8;
+        if (pb.rows >= 16384) w = 1;
         else if (long_rows) w = backward ? 16 : 8;
         else if (few_rows) w = 4;
-        else if (tiles1 >= 16) w = 1;
-        else if (tiles1 >= 8) w = backward ? 2 : 1;
         else w = 1;
-        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                               // row shorter than a tile
-        while (w < 8 && w != 16 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;     // very few rows
+        // rows taken out of memory order (tokens of a batch element beyond an L2, see slot_of_block):
+        // fewer of them open at a time
+        const bool regrouped = pb.M > 1 && pb.D * pb.L * pb.esize > (4 << 20);
+        bpc = regrouped ? 4 : 8;
+        depth = 2;
+    } else if (!backward) {
+        if (tiles1 <= 2) { w = 1; bpc = 8; depth = 2; }
+        else if (tiles1 <= 4) { w = 1; bpc = 4; depth = 2; }
+        else if (tiles1 <= 8) { w = 2; bpc = 8; depth = 2; }
+        else if (tiles1 <= 16) { w = 4; bpc = 4; depth = 2; }
+        else if (tiles1 <= 32) { w = many_rows ? 1 : 8; bpc = 2; depth = 2; }
+        else if (tiles1 <= 64) { w = many_rows ? 1 : 8; bpc = 1; depth = many_rows ? 4 : 2; }
+        else { w = 8; bpc = 1; depth = 4; }
+    } else {
+        if (tiles1 <= 4) { w = 1; bpc = 4; depth = 2; }
+        else if (tiles1 <= 8) { w = 4; bpc = 8; depth = 2; }
+        else if (tiles1 <= 16) { w = 4; bpc = 4; depth = 2; }
+        else if (tiles1 <= 32) { w = pb.rows >= 16384 ? 1 : 8; bpc = pb.rows >= 16384 ? 2 : 4; depth = 2; }
+        else if (tiles1 <= 64) { w = many_rows ? 2 : 8; bpc = many_rows ? 2 : 1; depth = many_rows ? 4 : 2; }
+        else { w = 16; bpc = 1; depth = 2; }  // 16 waves leave 128 registers each: no deeper prefetch
+    }
+    if (pb.waves) {
+        w = pb.waves;
+    } else {
+        while (w > 1 && tiles1 < (int64_t)w) w /= 2;                                        // row shorter than a tile
+        while (w < 8 && w != 16 && pb.rows * w < 1024 && tiles1 >= 2 * (int64_t)w) w *= 2;  // very few rows
     }
     t.waves = w;
     plan_segments(pb, t, may_split);
     w = t.waves;
-    const int64_t tiles_per_slot = t.nseg > 1 ? t.seg_tiles : tiles1;
-    unsigned bpc, depth;
-    if (shared_inputs) { bpc = 8; depth = 2; }
-    else if (w == 16) { bpc = 1; depth = 2; }  // backward, long rows: 16 waves leave 128 registers each
-    else if (w == 8) { bpc = 1; depth = backward ? 2 : 4; }
-    else if (w == 4) { bpc = 4; depth = backward ? 4 : 2; }
-    else if (w == 2) { bpc = 4; depth = 2; }
-    else if (tiles_per_slot >= 16) { bpc = 2; depth = 2; }
-    else if (tiles_per_slot >= 8) { bpc = 2; depth = 2; }
-    else { bpc = 4; depth = 2; }
+    if (t.nseg > 1) {  // a cut row is scanned by single waves, as short rows are
+        bpc = (t.seg_tiles >= 8) ? 2 : 4;
+        depth = 2;
+    }
     t.blocks_per_cu = pb.blocks_per_cu ? pb.blocks_per_cu : bpc;
     t.depth = pb.depth ? pb.depth : depth;
     if (w == 16) t.depth = 2;  // deeper does not fit the registers of a 16-wave block
