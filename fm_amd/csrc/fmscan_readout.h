@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void readout_forward_kernel(
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     const int lane = threadIdx.x & 63;
-    const int w = threadIdx.x >> 6;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // the same in all lanes: scalar branches on d
     const int64_t b = blockIdx.x / (uint32_t)tiles;
     const int32_t d0 = ((int32_t)blockIdx.y * 4 + w) * J;
     if (d0 >= D) return;  // whole waves; no barrier in this kernel
@@ -139,6 +139,66 @@ __global__ __launch_bounds__(256) void readout_forward_kernel(
     for (int j = 0; j < J; ++j) {
 #pragma unroll
         for (int i = 0; i < E; ++i) acc[j][i] = 0.0f;
+    }
+    if constexpr (VEC) {
+        // A wave walks the M slots one after the other, and what it has in flight is what bounds its
+        // pace: the loads of the slot after the one at work are issued before the work starts (a slot
+        // beyond the last is the last again, unused: every pass issues the same loads, so the waits
+        // are counted). Rows of d beyond D (last block) are loaded as row D - 1 and dropped. In place
+        // (states_out == states) this is safe: a slot's rows are read before any of them is written,
+        // and no other slot's rows are written in between.
+        struct Slot {
+            u32x4 wr;
+            FloatChunk<E> r;
+            u32x4 h[J];
+        };
+        const bool live = t0 < L;                            // this lane's chunk lies in the row
+        const int64_t tl = live ? t0 : L - E;                // a chunk past the end reads the last one
+        auto fetch = [&](Slot& q, int32_t m) {
+            const int64_t bm = b * M + (m < M ? m : M - 1);
+            q.wr = load16<T, false>(read + bm * L + tl);
+            if constexpr (NORM) q.r = load_float_chunk<E>(inv_rms + bm * L + tl);
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                const int32_t d = d0 + j < D ? d0 + j : D - 1;
+                q.h[j] = load16<T, true>(states + (bm * D + d) * L + tl);
+            }
+        };
+        auto work = [&](const Slot& q, int32_t m) {
+            const int64_t bm = b * M + m;
+            float r[E], wr[E];
+            Elem<T>::unpack(q.wr, wr);
+            if constexpr (NORM) spread<E>(q.r, r);
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                if (d0 + j >= D) continue;  // the whole wave
+                float h[E];
+                Elem<T>::unpack(q.h[j], h);
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int i = 0; i < E; ++i) h[i] *= r[i];
+                    const u32x4 packed = Elem<T>::pack(h);
+                    if (live) store16<T>(states_out + (bm * D + d0 + j) * L + t0, packed);
+                    Elem<T>::unpack(packed, h);  // the read-out sees what was stored
+                }
+#pragma unroll
+                for (int i = 0; i < E; ++i) acc[j][i] = __builtin_fmaf(wr[i], h[i], acc[j][i]);
+            }
+        };
+        Slot qa, qb;  // two sets of registers that swap roles: no copy from one to the other
+        fetch(qa, 0);
+        for (int32_t m = 0; m < M; m += 2) {
+            fetch(qb, m + 1);
+            work(qa, m);
+            fetch(qa, m + 2);
+            if (m + 1 < M) work(qb, m + 1);
+        }
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < J; ++j)
+                if (d0 + j < D) store16<T>(output + (b * D + d0 + j) * L + t0, Elem<T>::pack(acc[j]));
+        }
+        return;
     }
     for (int32_t m = 0; m < M; ++m) {
         const int64_t bm = b * M + m;
