@@ -119,18 +119,21 @@ def load_probe():
     lib = ctypes.CDLL(str(PROBE_LIB))
     lib.fmscan_probe_stream.restype = ctypes.c_int
     lib.fmscan_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
-                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+                                        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                        ctypes.c_void_p]
     return lib
 
 
-def streaming_copy(torch, rows, row_bytes, fwd_ms, bwd_ms, reps=10):
+def streaming_copy(torch, rows, row_bytes, fwd_ms, bwd_ms, reps=5):
     """What a bare streaming kernel with the scan kernels' access pattern reaches on the same shape.
 
-    `bench_stream_probe.so` (bench_stream_probe.hip, beside this file) walks `rows` rows of `row_bytes` bytes, one wave
-    per row, reading 2 tensors and writing 1 (the forward scan's streams) or reading 3 and writing 2
-    (the backward scan's), with no arithmetic and no tuning of residency. The published 8 TB/s is not
-    reachable by any kernel; this is a second reference point for kernels with these streams. Timed with
-    events on the current stream, best of two prefetch depths."""
+    `bench_stream_probe.so` (bench_stream_probe.hip, beside this file) walks `rows` rows of `row_bytes` bytes,
+    reading 2 tensors and writing 1 (the forward scan's streams) or reading 3 and writing 2 (the backward
+    scan's), with no arithmetic. It has the scan kernels' three knobs (waves side by side on a row, cap on
+    the blocks a compute unit holds, tiles of loads in flight) and is swept over all of them: `best` is the
+    fastest combination, `untuned` a wave per row with no cap (the better of the two depths). The published
+    8 TB/s is not reachable by any kernel; this is the second reference point for kernels with these streams.
+    Timed with events on the current stream."""
     if row_bytes % 1024:
         return None
     lib = load_probe()
@@ -140,28 +143,38 @@ def streaming_copy(torch, rows, row_bytes, fwd_ms, bwd_ms, reps=10):
     stream = torch.cuda.current_stream().cuda_stream
     out = {}
     for name, reads, writes in (("forward_streams", 2, 1), ("backward_streams", 3, 2)):
-        best = None
-        for depth in (2, 4):
-            def launch():
-                rc = lib.fmscan_probe_stream(src.data_ptr(), dst.data_ptr(), rows, row_bytes, reads, writes, depth,
-                                             stream)
-                if rc:
-                    raise RuntimeError(f"fmscan_probe_stream returned {rc}")
-            for _ in range(3):
-                launch()
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for _ in range(reps):
-                launch()
-            b.record()
-            b.synchronize()
-            ms = a.elapsed_time(b) / reps
-            best = ms if best is None else min(best, ms)
-        out[name] = {"reads": reads, "writes": writes, "ms": round(best, 4),
-                     "GBps": round((reads + writes) * tensor / (best * 1e-3) / 1e9, 1)}
-    # the scan kernels on the bytes they move, over the bare kernel with the same streams
-    out["forward_kernel_over_copy"] = round(out["forward_streams"]["ms"] / fwd_ms, 3)
-    out["backward_kernel_over_copy"] = round(out["backward_streams"]["ms"] / bwd_ms, 3)
+        best, untuned = None, None
+        for waves in (1, 2, 4, 8):
+            if row_bytes % (1024 * waves):
+                continue
+            for cap in (0, 1, 2, 4):
+                for depth in (2, 4):
+                    def launch():
+                        rc = lib.fmscan_probe_stream(src.data_ptr(), dst.data_ptr(), rows, row_bytes, reads, writes,
+                                                     depth, waves, cap, stream)
+                        if rc:
+                            raise RuntimeError(f"fmscan_probe_stream returned {rc}")
+                    for _ in range(2):
+                        launch()
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                    for _ in range(reps):
+                        launch()
+                    b.record()
+                    b.synchronize()
+                    ms = a.elapsed_time(b) / reps
+                    if best is None or ms < best[0]:
+                        best = (ms, waves, cap, depth)
+                    if waves == 1 and cap == 0 and (untuned is None or ms < untuned):
+                        untuned = ms
+        gbps = lambda ms: round((reads + writes) * tensor / (ms * 1e-3) / 1e9, 1)
+        out[name] = {"reads": reads, "writes": writes,
+                     "best": {"ms": round(best[0], 4), "GBps": gbps(best[0]), "waves_per_row": best[1],
+                              "blocks_per_cu": best[2] or "no cap", "depth": best[3]},
+                     "untuned": {"ms": round(untuned, 4), "GBps": gbps(untuned)}}
+    # the scan kernels on the bytes they move, over the best bare kernel with the same streams
+    out["forward_kernel_over_copy"] = round(out["forward_streams"]["best"]["ms"] / fwd_ms, 3)
+    out["backward_kernel_over_copy"] = round(out["backward_streams"]["best"]["ms"] / bwd_ms, 3)
     return out
 
 
@@ -311,6 +324,13 @@ def per_config(torch, dev, skip, steps, warmup):
                      "bwd_frac_of_peak": round(6 * s * N / bwd_ms / 1e6 / PEAK_HBM_GBPS, 4),
                      "bwd_frac_of_moved_bytes": round(5 * s * N / bwd_ms / 1e6 / PEAK_HBM_GBPS, 4)}
         del g, x, G, buffers
+        torch.cuda.empty_cache()
+        copy = streaming_copy(torch, B * Cn, T * s, fwd_ms, bwd_ms)
+        if copy:  # the best bare streaming kernel with the same streams on this shape (see streaming_copy)
+            out[name]["best_copy_GBps"] = {"forward_streams": copy["forward_streams"]["best"]["GBps"],
+                                           "backward_streams": copy["backward_streams"]["best"]["GBps"]}
+            out[name]["fwd_kernel_over_copy"] = copy["forward_kernel_over_copy"]
+            out[name]["bwd_kernel_over_copy"] = copy["backward_kernel_over_copy"]
         torch.cuda.empty_cache()
     step, N, name = layer_step(torch, dev)
     for _ in range(warmup):
@@ -503,6 +523,7 @@ GRID_ROWS = (256, 2048, 16384, 131072)
 GRID_L = (1024, 4096, 16384, 65536)
 GRID_NATIVE = ((32, 32, 64, 2048), (8, 16, 64, 16384), (4, 32, 1024, 4096), (1, 32, 1024, 8192))  # (B, M, D, L)
 GRID_MAX_ELEMENTS = 1 << 31  # per tensor; larger cells of the grid are left out
+GRID_DEPTHS = (2, 4)
 
 
 def run_grid(torch, args) -> int:
@@ -516,7 +537,7 @@ def run_grid(torch, args) -> int:
     from fm.scan.fm_scan import fm_scan_backward, fm_scan_forward
 
     dev = torch.device("cuda", 0)
-    overrides = [(w, b, d) for w in (1, 2, 4, 8) for b in (1, 2, 4, 8) for d in (2, 4)]
+    overrides = [(w, b, d) for w in (1, 2, 4, 8) for b in (1, 2, 4, 8) for d in GRID_DEPTHS]
     raw = open(args.grid_raw, "w") if args.grid_raw else None
 
     def timed(call):

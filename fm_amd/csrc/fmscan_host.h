@@ -208,7 +208,7 @@ inline Tuning choose(const Problem& pb, bool backward, bool may_split) {
         else if (tiles1 <= 8) { w = 4; bpc = 8; depth = 2; }
         else if (tiles1 <= 16) { w = 4; bpc = 4; depth = 2; }
         else if (tiles1 <= 32) { w = pb.rows >= 16384 ? 1 : 8; bpc = pb.rows >= 16384 ? 2 : 4; depth = 2; }
-        else if (tiles1 <= 64) { w = many_rows ? 2 : 8; bpc = many_rows ? 2 : 1; depth = many_rows ? 4 : 2; }
+        else if (tiles1 <= 64) { w = many_rows ? 2 : 8; bpc = many_rows ? 2 : 1; depth = 2; }
         else { w = 16; bpc = 1; depth = 2; }  // 16 waves leave 128 registers each: no deeper prefetch
     }
     if (pb.waves) {

@@ -477,8 +477,6 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
     if given_state:
         _require(tuple(initial_state.shape) == (B, M, D),
                  f"initial_state must be {(B, M, D)}, got {tuple(initial_state.shape)}")
-    else:
-        initial_state = torch.zeros((B, M, D), device=dev, dtype=gates.dtype)
     code = _dtype_code(gates)
     states = torch.empty((B, M, D, L), device=dev, dtype=gates.dtype)
     kept_state = initial_state if given_state else None
@@ -488,7 +486,8 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
             stream = torch.cuda.current_stream(dev).cuda_stream
             if D <= _raw.fmscan_forward_normed_max_d():
                 # scan and norm in one kernel: the scanned states never reach memory
-                _lib.check(_raw.fmscan_forward_normed(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+                # (no initial state: NULL, which the library reads as zeros; no fill kernel)
+                _lib.check(_raw.fmscan_forward_normed(gates.data_ptr(), tokens.data_ptr(), _ptr(kept_state),
                                                         states.data_ptr(), inv_rms.data_ptr(), B, M, D, L, code,
                                                         float(norm_eps), stream))
                 output, _, _ = fm_readout_forward(states, read, mem_norm=False)  # the read-out alone
@@ -498,13 +497,15 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
             groups = _raw.fmscan_sumsq_groups(D)
             partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
             output = torch.empty((B, D, L), dtype=states.dtype, device=dev)
-            _lib.check(_raw.fmscan_forward_sumsq(gates.data_ptr(), tokens.data_ptr(), initial_state.data_ptr(),
+            _lib.check(_raw.fmscan_forward_sumsq(gates.data_ptr(), tokens.data_ptr(), _ptr(kept_state),
                                                    states.data_ptr(), partial.data_ptr(), B, M, D, L, code, stream))
             _lib.check(_raw.fmscan_sumsq_finish(partial.data_ptr(), groups, inv_rms.data_ptr(), B, M, D, L,
                                                   float(norm_eps), stream))
             _lib.check(_raw.fmscan_readout_forward(states.data_ptr(), inv_rms.data_ptr(), read.data_ptr(),
                                                      states.data_ptr(), output.data_ptr(), B, M, D, L, code, stream))
         return output, None, states, inv_rms, kept_state
+    if not given_state:
+        initial_state = torch.zeros((B, M, D), device=dev, dtype=gates.dtype)
     fm_scan_forward(gates, tokens, initial_state, states)
     # with the norm the scanned states are needed no longer (backward takes them back from the
     # normalised ones): normalise in place, one (B, M, D, L) tensor at any time
@@ -541,8 +542,7 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         groups = _raw.fmscan_reduced_groups(B, D)
         d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
-        zeros = torch.zeros((B, M, D), dtype=dtype, device=dev)
-        d_h0 = torch.empty_like(zeros) if want_initial_state_grad else None
+        d_h0 = torch.empty((B, M, D), dtype=dtype, device=dev) if want_initial_state_grad else None
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(_raw.fmscan_readout_dot(
@@ -550,7 +550,7 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
                 read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), _ptr(rms), B, M, D, L, code, stream))
             _lib.check(_raw.fmscan_backward_layer(
                 gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
-                out_grad.data_ptr(), zeros.data_ptr(), d_tokens.data_ptr(),
+                out_grad.data_ptr(), None, d_tokens.data_ptr(),  # nothing arrives from beyond the last step
                 None if mem_norm else states.data_ptr(),  # with the norm: states = states_n * rms
                 _ptr(rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0),
                 B, M, D, L, code, 0, stream))

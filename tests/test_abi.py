@@ -242,11 +242,14 @@ def test_streaming_probe_library_rejects_what_it_does_not_cover():
     from fm_amd import build
     assert not hasattr(build, "PROBE_LIB") and not list((ROOT / "fm_amd").rglob("*probe*"))  # not in the product
     a, b = 1 << 20, 1 << 30
-    assert f(None, b, 4, 1024, 2, 1, 2, None) == -1        # no input
-    assert f(a, b, 4, 1000, 2, 1, 2, None) == -1           # a row is not whole steps
-    assert f(a, b, 4, 1024, 1, 1, 2, None) == -1           # a stream count it has no kernel for
-    assert f(a, b, 4, 1024, 3, 2, 3, None) == -1           # a prefetch depth it has no kernel for
-    assert f(a + 8, b, 4, 1024, 3, 2, 2, None) == -1       # not 16-byte aligned
+    assert f(None, b, 4, 1024, 2, 1, 2, 1, 0, None) == -1        # no input
+    assert f(a, b, 4, 1000, 2, 1, 2, 1, 0, None) == -1           # a row is not whole steps
+    assert f(a, b, 4, 1024, 2, 1, 2, 2, 0, None) == -1           # nor whole steps of two waves side by side
+    assert f(a, b, 4, 1024, 1, 1, 2, 1, 0, None) == -1           # a stream count it has no kernel for
+    assert f(a, b, 4, 1024, 3, 2, 3, 1, 0, None) == -1           # a prefetch depth it has no kernel for
+    assert f(a, b, 4, 4096, 3, 2, 2, 3, 0, None) == -1           # three waves per row: not offered
+    assert f(a, b, 4, 1024, 3, 2, 2, 1, 16, None) == -1          # a cap beyond 15 blocks
+    assert f(a + 8, b, 4, 1024, 3, 2, 2, 1, 0, None) == -1       # not 16-byte aligned
 
 
 def test_rejected_sum_groups_arguments(lib):
