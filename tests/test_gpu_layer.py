@@ -2,10 +2,13 @@
 over D, read-out over M, and every gradient) with the float64 CPU oracle of the same layer
 (reference fm/scan/fm_scan.py:102-133, gradients by the chain rule), on an MI355X.
 
-Both sides start from the same, already quantised inputs, and the oracle takes the gates
-1 - alpha * update_scale and the read weights alpha * output_scale rounded to the storage dtype,
-as the layer (the reference's as well as this one) hands them to the scan: stored in bfloat16 a
-gate near one moves by up to 2^-9, which is a different decay and not an error of the scan.
+Both sides start from the same, already quantised inputs, and the oracle forms the gates and the
+read weights where the reference's lines hold tensors of the storage dtype (fm_scan.py:116-119,130):
+alpha * update_scale rounded, one minus that rounded again, alpha * output_scale rounded once. The
+layer's prepare kernel gives the same bits (tests/test_gpu_parity.py::
+test_layer_prepare_and_finish_kernels; the oracle's side is pinned against the PyTorch operations in
+tests/test_oracle.py), so both sides scan with the reference's gates: stored in bfloat16 a gate near
+one moves by up to 2^-9 per rounding, which is a different decay and not an error of the scan.
 Errors are normwise,
     max|y - ref| / max|ref|   and   ||y - ref||_2 / ||ref||_2,
 per returned quantity. Tolerances, with what they pay for:
