@@ -460,13 +460,13 @@ __global__ __launch_bounds__(256) void layer_finish_kernel(
     const float os = t < L ? (float)output_scale[b * L + t] : 0.0f;
     float d_us = 0.0f, d_os = 0.0f;
     for (int64_t m0 = 0; m0 < M; m0 += 64) {
-        __syncthreads();  // the tiles of the round before are no longer read
+        __syncthreads();  // the tiles of the pass before are no longer read
 #pragma unroll 4
         for (int i = w; i < 64; i += 4)  // alpha tile, rows are steps
             ta[i][lane] = (t0 + i < L && m0 + lane < M) ? (float)alpha[(b * L + t0 + i) * M + m0 + lane] : 0.0f;
         __syncthreads();
 #pragma unroll 2
-        for (int i = w; i < 64; i += 4) {  // row i of this round: slot m0 + i, lanes are steps
+        for (int i = w; i < 64; i += 4) {  // row i of this pass: slot m0 + i, lanes are steps
             const int64_t m = m0 + i;
             float dg = 0.0f, dr = 0.0f;
             if (m < M && t < L) {
