@@ -27,14 +27,16 @@ namespace fmscan {
 //     wave to wave through LDS (each adds its own; fixed order, hence deterministic) and the
 //     last stores d_tokens[b, d, tile].
 // No wave waits for another except in that hand-over, once per tile. The running state of
-// every row lives in LDS (one float per row, private to its wave). Loads run one slot
-// ahead: while the J rows of a slot are worked on, the J tiles of the next slot (or of the
-// first slot of the tile before) are in flight, as are its per-slot vectors; every step
-// issues the same loads whatever its position (addresses are clamped into the tensors), so
-// the count of loads in flight is a compile-time number. (The per-slot vectors of the step at
-// work and of the step after it sit in two sets of registers that swap roles, steps come in
-// pairs; what a step needs only at its end, the layer form's rms vector, is loaded at its
-// start. J = 8 uses all 256 registers two waves per SIMD leave.)
+// every row lives in LDS (one float per row, private to its wave). Loads run ahead: the
+// per-slot vectors by one slot, the rows' tiles by J rows, or by J / 2 where J = 8 and the
+// elements have 2 bytes (the first rows of the next slot, or of the first slot of the tile
+// before, are then loaded while the last rows of this one are worked on: half the registers
+// for tiles in flight, which the compiler turns into a shorter schedule of the whole step);
+// every step issues the same loads whatever its position (addresses are clamped into the
+// tensors), so the count of loads in flight is a compile-time number. (The per-slot vectors
+// of the step at work and of the step after it sit in two sets of registers that swap roles,
+// steps come in pairs; what a step needs only at its end, the layer form's rms vector, is
+// loaded at its start.)
 // HBM traffic per element of (B, M, D, L): G and h (2s), or the normalised states alone in
 // the layer form (s), plus 4/J bytes of partials, against 6s for the unfused kernel plus the
 // two torch.sum passes.
@@ -204,15 +206,18 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         }
     };
 
-    Row rows[J];
+    // The rows' tiles in flight: RING of them, so a row is loaded RING rows ahead of its use (the first
+    // rows of the next step from the last rows of this one).
+    constexpr int RING = (J >= 8 && sizeof(T) == 2) ? J / 2 : J;
+    Row rows[RING];
     // The per-slot vectors of the step at work and of the step after it, which is loading, sit in
     // two sets of registers that swap roles from step to step: handing one set over to the other
     // at the end of a step would have to wait for every load and store in flight.
     Slot slot_a, slot_b;
-    int32_t kf = ntiles - 1, mf = 0;  // where the loads are: one step (a slot's J rows) ahead of the work
+    int32_t kf = ntiles - 1, mf = 0;  // the step after the one at work: where the loads that run ahead are
     fetch_slot(slot_a, kf, mf);
 #pragma unroll
-    for (int j = 0; j < J; ++j) fetch_row(rows[j], kf, mf, j);
+    for (int j = 0; j < RING; ++j) fetch_row(rows[j], kf, mf, j);
 
     int parity = 0;
     if constexpr (kSharedX || kSharedY) {
@@ -239,7 +244,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
             fetch_slot(next_slot, kf, mf);
             if (mi >= mcount) {  // the padding step of an odd count
 #pragma unroll
-                for (int j = 0; j < J; ++j) fetch_row(rows[j], kf, mf, j);
+                for (int j = 0; j < RING; ++j) fetch_row(rows[j], kf, mf, j);
                 return;
             }
             [[maybe_unused]] Rms rms_now;
@@ -262,6 +267,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     }
                 }
             }
+            [[maybe_unused]] float one_minus_g[E];  // the token gradient's factor, once per slot
+#pragma unroll
+            for (int i = 0; i < E; ++i) one_minus_g[i] = 1.0f - g[i];
             float a = g[E - 1];
 #pragma unroll
             for (int i = E - 2; i >= 0; --i) a *= g[i];
@@ -286,18 +294,20 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                 for (int j = 0; j < J; ++j) {
                     // (unpacked before the loads of the slot after this one reuse the registers)
                     float G[E], h[E], x[E];
-                    Elem<T>::unpack(rows[j].a, G);
+                    Row& held = rows[j % RING];
+                    Elem<T>::unpack(held.a, G);
                     // what stands before the tile in the row: a state, or a normalised one (the factor
                     // follows with the slot); at k == 0 the initial state itself, or nothing
-                    const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(rows[j].hb) : 0.0f;
-                    [[maybe_unused]] const float h_first = Elem<T>::widen(rows[j].h_first);
+                    const float hb = (k > 0 || h0 != nullptr) ? Elem<T>::widen(held.hb) : 0.0f;
+                    [[maybe_unused]] const float h_first = Elem<T>::widen(held.h_first);
                     if constexpr (LAYER == 2) {
 #pragma unroll
                         for (int i = 0; i < E; ++i) h[i] = G[i];  // G[] holds the normalised state
                     } else if constexpr (!REMAKE) {
-                        Elem<T>::unpack(rows[j].h, h);
+                        Elem<T>::unpack(held.h, h);
                     }
-                    fetch_row(rows[j], kf, mf, j);
+                    if (j + RING < J) fetch_row(held, k, mi, j + RING);  // further on in this slot
+                    else fetch_row(held, kf, mf, j + RING - J);         // the first rows of the step after
                     if (d0 + j >= D) continue;  // the whole wave: a row past the last d adds nothing
 
                     float carry = carry_of[j];
@@ -348,7 +358,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                         c = g[i] * delta;
                         // token gradient (1 - g) * delta
                         if constexpr (PLAIN) dtok[j][i] += delta;
-                        else dtok[j][i] += delta - c;  // (1 - g) * delta = delta - g * delta
+                        else dtok[j][i] = __builtin_fmaf(one_minus_g[i], delta, dtok[j][i]);
                         with_state[i] = __builtin_fmaf(hprev[i], delta, with_state[i]);
                         if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
                     }
