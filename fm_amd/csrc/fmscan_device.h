@@ -30,7 +30,10 @@ __device__ __forceinline__ uint32_t opaque_zero() {
     return z;
 }
 template <typename V>
-__device__ __forceinline__ V load_by_wave(const V* p, uint32_t zero) { return p[zero]; }
+__device__ __forceinline__ V load_by_wave(const V* p, uint32_t zero) {
+    // (a byte offset: uniform base + 32-bit lane offset is an addressing mode of the load itself)
+    return *reinterpret_cast<const V*>(reinterpret_cast<const char*>(p) + zero);
+}
 
 // All vector loads and stores issued so far have completed. For use just before a loop that
 // prefetches: the compiler puts one wait at the loop's head for both ways into it, and sizes it

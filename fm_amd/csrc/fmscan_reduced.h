@@ -82,6 +82,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
     const int32_t lane_off = (63 - lane) * E;  // lane l owns the chunk l chunks before the end of the tile
     float* mycarry = carries + w * Mw * J;
+    const int32_t rows_here = uniform(D - d0 < J ? D - d0 : J);  // rows of this block that exist (the last group may be short)
 
     // (the trip count is the same for all lanes and only the access is predicated: a loop that
     // some lanes skip would leave the values it shares with the code below in vector registers,
@@ -93,9 +94,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         if (idx < mcount * J)
             mycarry[idx] = first_prop_grad ? Elem<T>::widen(first_prop_grad[((b * M + m0 + mi) * D + d)]) : 0.0f;
     }
-    // Row j of the block's group of d, clamped: a d beyond D (last group) is loaded like any
-    // other (as D - 1), never accumulated or stored. Everything here is wave-uniform.
-    auto d_of = [&](int j) { return d0 + j < D ? d0 + j : D - 1; };
+    // Everything here is wave-uniform. A row j of the block's group past the last d (last group) is
+    // loaded like any other (as row D - 1), never accumulated or stored.
     auto slot_of = [&](int32_t mi) {  // clamped: a wave without slots still issues (unused) loads
         const int32_t m = m0 + mi;
         return m < M ? m : M - 1;
@@ -130,21 +130,34 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         const int32_t rem = left < TILE ? (int32_t)left : TILE;
         return (uint32_t)(lane_off < rem ? lane_off : rem - E);
     };
-    auto fetch_row = [&](Row& r, int32_t k, int32_t mi, int j) {
-        const int64_t tw = (int64_t)k * TILE;
-        const uint32_t lo = lane_elems(k);
-        const int64_t row = (b * M + slot_of(mi)) * D + d_of(j);
-        const int64_t base = row * L + tw;
-        r.a = load16<T, true>(out_grad + base + lo);
+    // What the addresses of a step's J rows share, all of it wave-uniform: made once per step.
+    struct Place {
+        int64_t row0;  // (b, slot, d0) as a row of the (B, M, D) tensors
+        int64_t base;  // where that row's tile starts in the (B, M, D, L) tensors
+        int32_t k;     // the tile
+    };
+    auto place_of = [&](int32_t k, int32_t mi) {
+        Place p;
+        p.row0 = (b * M + slot_of(mi)) * D + d0;
+        p.base = p.row0 * L + (int64_t)k * TILE;
+        p.k = k;
+        return p;
+    };
+    // (the tile comes from a uniform base and a 32-bit lane offset: no vector address arithmetic)
+    auto fetch_row = [&](Row& r, const Place& p, int j) {
+        const int32_t jc = j < rows_here ? j : rows_here - 1;  // (past the last d: row D - 1 again)
+        const int64_t base = p.base + (int64_t)jc * L;
+        const uint32_t lo = lane_elems(p.k) * (uint32_t)sizeof(T);
+        r.a = load16<char, true>(reinterpret_cast<const char*>(out_grad + base) + lo);
         r.h = u32x4{0u, 0u, 0u, 0u};
-        if constexpr (LAYER != 2 && !REMAKE) r.h = load16<T, true>(h_saved + base + lo);
+        if constexpr (LAYER != 2 && !REMAKE) r.h = load16<char, true>(reinterpret_cast<const char*>(h_saved + base) + lo);
         const T* __restrict__ hsrc = LAYER == 2 ? out_grad : h_saved;
         // h just before the tile (h[-1] at the start of the row): one address for the whole wave
-        const T* src = tw > 0 ? hsrc + (base - 1) : (h0 != nullptr ? h0 + row : hsrc + base);
+        const T* src = p.k > 0 ? hsrc + (base - 1) : (h0 != nullptr ? h0 + (p.row0 + jc) : hsrc + base);
         r.hb = load_by_wave(src, vzero);
         r.h_first = T(0);
         // (no new cache line except in the first tile)
-        if constexpr (REMAKE) r.h_first = load_by_wave(hsrc + (tw > 0 ? base - 1 : base), vzero);
+        if constexpr (REMAKE) r.h_first = load_by_wave(hsrc + (p.k > 0 ? base - 1 : base), vzero);
     };
     auto fetch_slot = [&](Slot& s, int32_t k, int32_t mi) {
         const int64_t tw = (int64_t)k * TILE;
@@ -216,8 +229,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     Slot slot_a, slot_b;
     int32_t kf = ntiles - 1, mf = 0;  // the step after the one at work: where the loads that run ahead are
     fetch_slot(slot_a, kf, mf);
+    Place place_next = place_of(kf, mf), place_now = place_next;
 #pragma unroll
-    for (int j = 0; j < RING; ++j) fetch_row(rows[j], kf, mf, j);
+    for (int j = 0; j < RING; ++j) fetch_row(rows[j], place_next, j);
 
     int parity = 0;
     if constexpr (kSharedX || kSharedY) {
@@ -241,10 +255,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         }
         auto slot_step = [&](const Slot& cur, Slot& next_slot, int32_t mi) __attribute__((always_inline)) {
             ahead(kf, mf);
+            place_now = place_next;
+            place_next = place_of(kf, mf);
             fetch_slot(next_slot, kf, mf);
             if (mi >= mcount) {  // the padding step of an odd count
 #pragma unroll
-                for (int j = 0; j < RING; ++j) fetch_row(rows[j], kf, mf, j);
+                for (int j = 0; j < RING; ++j) fetch_row(rows[j], place_next, j);
                 return;
             }
             [[maybe_unused]] Rms rms_now;
@@ -306,9 +322,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     } else if constexpr (!REMAKE) {
                         Elem<T>::unpack(held.h, h);
                     }
-                    if (j + RING < J) fetch_row(held, k, mi, j + RING);  // further on in this slot
-                    else fetch_row(held, kf, mf, j + RING - J);         // the first rows of the step after
-                    if (d0 + j >= D) continue;  // the whole wave: a row past the last d adds nothing
+                    if (j + RING < J) fetch_row(held, place_now, j + RING);  // further on in this slot
+                    else fetch_row(held, place_next, j + RING - J);         // the first rows of the step after
+                    // the whole wave: a row past the last d adds nothing. (The count goes through an empty asm so
+                    // that the comparison is made here, one scalar compare, and not kept from before the loops as
+                    // a lane mask per row: sixteen scalar registers the kernel does not have.)
+                    int32_t rows_valid = rows_here;
+                    asm volatile("" : "+s"(rows_valid));
+                    if (j >= rows_valid) continue;
 
                     float carry = carry_of[j];
                     if constexpr (LAYER != 0) {
