@@ -73,9 +73,12 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
         const int32_t rem = left < TILE ? (int32_t)left : TILE;
         return (uint32_t)(lane_off < rem ? lane_off : rem - E);
     };
+    // Token tiles in flight: RING of them (a row's tile is loaded RING rows ahead of its use: the first
+    // rows of the next tile while the last rows of this one are worked on).
+    constexpr int RING = J >= 8 ? J / 2 : J;
     struct Loads {
         u32x4 g;
-        u32x4 x[J];
+        u32x4 x[RING];
     };
     // k beyond the last tile: the last tile again (not used)
     auto fetch_gates = [&](Loads& q, int32_t k) {
@@ -84,16 +87,16 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     };
     auto fetch_tokens = [&](Loads& q, int32_t k, int j) {
         k = k < ntiles ? k : ntiles - 1;
-        q.x[j] = load16<T, false>(tokens + (b * D + d_of(j)) * L + (int64_t)k * TILE + lane_elems(k));
+        q.x[j % RING] = load16<T, false>(tokens + (b * D + d_of(j)) * L + (int64_t)k * TILE + lane_elems(k));
     };
 
-    // The loads run a tile ahead, each into the registers it was just unpacked from: a second set
-    // of registers handed over at the end of a tile would make that hand-over wait for the
-    // tile's stores as well.
+    // The loads run ahead (the gates a tile, the tokens RING rows), each into the registers it was
+    // just unpacked from: a second set of registers handed over at the end of a tile would make that
+    // hand-over wait for the tile's stores as well.
     Loads q;
     fetch_gates(q, 0);
 #pragma unroll
-    for (int j = 0; j < J; ++j) fetch_tokens(q, 0, j);
+    for (int j = 0; j < RING; ++j) fetch_tokens(q, 0, j);
     int parity = 0;
     wait_for_loads();
     // One tile. `whole`: it lies wholly inside the row and nothing is tested per lane, so that
@@ -124,8 +127,9 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
 #pragma unroll
         for (int j = 0; j < J; ++j) {
             float u[E];
-            Elem<T>::unpack(q.x[j], u);
-            fetch_tokens(q, k + 1, j);
+            Elem<T>::unpack(q.x[j % RING], u);
+            if (j + RING < J) fetch_tokens(q, k, j + RING);
+            else fetch_tokens(q, k + 1, j + RING - J);
 #pragma unroll
             for (int i = 0; i < E; ++i) u[i] = __builtin_fmaf(-g[i], u[i], u[i]);  // (1 - g) x, one rounding
             float bb = u[0];
