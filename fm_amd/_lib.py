@@ -91,11 +91,21 @@ def load() -> ctypes.CDLL:
     lib.fmscan_backward_reduced.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     lib.fmscan_backward_layer.restype = c_int
     lib.fmscan_backward_layer.argtypes = [c_void_p] * 13 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
+    lib.fmscan_reduced_split.restype = c_int64
+    lib.fmscan_reduced_split.argtypes = [c_int64] * 3
+    lib.fmscan_reduced_pays.restype = c_int
+    lib.fmscan_reduced_pays.argtypes = [c_int64] * 3
+    lib.fmscan_backward_reduced_split.restype = c_int
+    lib.fmscan_backward_reduced_split.argtypes = [c_void_p] * 9 + [c_int64] * 5 + [c_int, c_uint, c_void_p]
+    lib.fmscan_backward_layer_split.restype = c_int
+    lib.fmscan_backward_layer_split.argtypes = [c_void_p] * 13 + [c_int64] * 5 + [c_int, c_uint, c_void_p]
     dims = [c_int64] * 4
     lib.fmscan_readout_inv_rms.restype = c_int
     lib.fmscan_readout_inv_rms.argtypes = [c_void_p] * 2 + dims + [c_int, c_float, c_void_p]
     lib.fmscan_forward_normed_max_d.restype = c_int64
     lib.fmscan_forward_normed_max_d.argtypes = []
+    lib.fmscan_forward_normed_pays.restype = c_int
+    lib.fmscan_forward_normed_pays.argtypes = [c_int64] * 3
     lib.fmscan_forward_normed.restype = c_int
     lib.fmscan_forward_normed.argtypes = [c_void_p] * 5 + dims + [c_int, c_float, c_void_p]
     lib.fmscan_sumsq_groups.restype = c_int64

@@ -26,6 +26,16 @@ extern "C" {
 
 int64_t fmscan_forward_normed_max_d(void) { return kNormedMaxD; }
 
+int fmscan_forward_normed_pays(int64_t B, int64_t M, int64_t D) {
+    if (B < 1 || M < 1 || D < 1) return 0;
+    // A block of these kernels is a slot (or 128 rows of one) for the whole length of the sequence: below 64
+    // blocks three quarters of the GPU stand idle, and fmscan_forward (a block per four rows, rows cut into
+    // segments when there are few) followed by the norm's and the read-out's own kernels is faster although
+    // it moves twice the bytes (measured: (B,L,M,D) = (1,32768,32,128) 0.43 against 0.28 ms, (1,65536,16,64)
+    // 0.46 against 0.18; (2,16384,32,128) 0.28 either way; (4,8192,32,128) 0.20 against 0.27).
+    return (__int128)B * M * ((D + kNormedMaxD - 1) / kNormedMaxD) >= 64 ? 1 : 0;
+}
+
 int fmscan_forward_normed(const void* gates, const void* tokens, const void* initial_state, void* states_n,
                           float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, float eps,
                           void* stream) {

@@ -49,6 +49,13 @@ namespace fmscan {
 // (h_saved is NULL) but taken back from the normalised ones, h = out_grad * rms, so that
 // the layer has to keep nothing of size (B, M, D, L) besides the states it returns.
 // coef_out, coef_self and rms are float32.
+//
+// split > 1, for problems with too few (b, group of d) pairs to fill the GPU: the M slots of a batch
+// element are dealt to `split` blocks instead of one. The caller states it as a problem of B * split
+// batch elements of M / split slots each, which is the same memory for everything indexed by (b, m);
+// the kernel only has to find the token rows (and the layer's output-gradient rows) of its batch element
+// at b / split, and to leave its token gradient, a sum over its own slots only, as float32 in
+// token_partial[b / split, d, b % split, :] for a sum over the blocks of a batch element that rounds once.
 template <typename T, int J, int NW, bool PLAIN, int LAYER>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) void scan_backward_reduced_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
@@ -56,7 +63,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     const T* __restrict__ tokens, float* __restrict__ gate_partial /* (B, M, NG, L) */,
     const T* __restrict__ h0, T* __restrict__ h0_grad, const float* __restrict__ coef_out /* (B, M, L) */,
     const float* __restrict__ coef_self /* (B, M, L) */, const T* __restrict__ layer_out_grad /* (B, D, L) */,
-    const float* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L, int32_t Mw) {
+    const float* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L, int32_t Mw,
+    float* __restrict__ token_partial /* (B / split, D, split, L), or NULL */, int32_t split) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     extern __shared__ float lds[];
@@ -83,6 +91,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int32_t lane_off = (63 - lane) * E;  // lane l owns the chunk l chunks before the end of the tile
     float* mycarry = carries + w * Mw * J;
     const int32_t rows_here = uniform(D - d0 < J ? D - d0 : J);  // rows of this block that exist (the last group may be short)
+    const int64_t b_tok = split > 1 ? uniform((int)((uint32_t)b / (uint32_t)split)) : b;  // whose tokens these are
 
     // (the trip count is the same for all lanes and only the access is predicated: a loop that
     // some lanes skip would leave the values it shares with the code below in vector registers,
@@ -203,7 +212,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         for (int s = 0; s < SH; ++s) {
             const int32_t jj = w * SH + s < J ? w * SH + s : J - 1;  // (a wave beyond the J rows loads the last again, unused)
             const int32_t d = d0 + jj < D ? d0 + jj : D - 1;
-            const int64_t off = (b * D + d) * L + tw + lo;
+            const int64_t off = (b_tok * D + d) * L + tw + lo;
             ts.x[s] = ts.y[s] = u32x4{0u, 0u, 0u, 0u};
             if constexpr (kSharedX) ts.x[s] = load16<T, false>(tokens + off);
             if constexpr (kSharedY) ts.y[s] = load16<T, false>(layer_out_grad + off);
@@ -459,8 +468,20 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                             *cell = make_float4(dtok[j][4 * q4], dtok[j][4 * q4 + 1], dtok[j][4 * q4 + 2],
                                                 dtok[j][4 * q4 + 3]);
                     }
-                    if (ww == NW - 1 && d0 + j < D)
-                        store_chunk<T, true>(token_grad + (b * D + d0 + j) * L, tw + lane_off, L, Elem<T>::pack(dtok[j]));
+                    if (ww == NW - 1 && d0 + j < D) {
+                        if (token_partial == nullptr) {
+                            store_chunk<T, true>(token_grad + (b * D + d0 + j) * L, tw + lane_off, L, Elem<T>::pack(dtok[j]));
+                        } else if (tw + lane_off < L) {  // (tiles are whole chunks)
+                            float* __restrict__ dst =
+                                token_partial + ((b_tok * D + d0 + j) * split + (b - b_tok * split)) * L + tw + lane_off;
+#pragma unroll
+                            for (int q4 = 0; q4 < E / 4; ++q4) {
+                                const u32x4 v = {f2u(dtok[j][4 * q4]), f2u(dtok[j][4 * q4 + 1]), f2u(dtok[j][4 * q4 + 2]),
+                                                 f2u(dtok[j][4 * q4 + 3])};
+                                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst + 4 * q4));
+                            }
+                        }
+                    }
                 }
             }
             if (ww < NW - 1) __syncthreads();

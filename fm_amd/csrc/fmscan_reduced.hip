@@ -14,6 +14,22 @@ constexpr int kReducedWaves = 4;  // waves of a block: they split the M memory s
 // partials and the work per slot that does not depend on the row; 4 otherwise, for twice the blocks.
 int reduced_group(int64_t B, int64_t D) { return (__int128)B * ((D + 7) / 8) >= 512 ? 8 : 4; }
 
+// Into how many blocks the M slots of a batch element are dealt (1: not at all) so that the (b, group of
+// 4 d) pairs, times that number, reach the 512 blocks that fill the GPU: the smallest divisor of M that
+// does, among those that leave each of a block's waves a slot (M / split >= kReducedWaves).
+int64_t reduced_split(int64_t B, int64_t M, int64_t D) {
+    const __int128 pairs = (__int128)B * ((D + 3) / 4);
+    if (pairs >= 512 || M < 2 * kReducedWaves) return 1;
+    const int64_t want = (int64_t)((512 + pairs - 1) / pairs);
+    int64_t best = 1;
+    for (int64_t s = 2; s <= M / kReducedWaves; ++s) {
+        if (M % s != 0) continue;
+        best = s;
+        if (s >= want) break;
+    }
+    return best;
+}
+
 }  // namespace
 
 extern "C" {
@@ -26,19 +42,26 @@ int64_t fmscan_reduced_groups(int64_t B, int64_t D) {
 
 // Shared by fmscan_backward_reduced and fmscan_backward_layer (coef_out != NULL): in the second
 // form `out_grad` carries the normalised states and the gradient of the states is made in the kernel.
+// split > 1: the slots of a batch element dealt to `split` blocks; the token gradient then goes to
+// token_partial (float32) and token_grad is not written.
 static int backward_reduced(const char* who, const void* gates, const void* out_grad, const void* first_prop_grad,
                             void* token_grad, const void* cached_output, const void* input_tokens,
                             float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
                             const float* coef_out, const float* coef_self, const void* layer_out_grad,
                             const float* rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
-                            unsigned flags, void* stream) {
+                            unsigned flags, void* stream, float* token_partial = nullptr, int64_t split = 1) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
     if (flags & ~FMSCAN_FLAG_PLAIN)
         return fail(FMSCAN_E_FLAGS, "%s: only FMSCAN_FLAG_PLAIN is understood here", who);
+    if (split < 1 || M % split != 0 || split > INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: split = %lld must be >= 1 and divide M = %lld", who, (long long)split,
+                    (long long)M);
+    if ((split > 1) != (token_partial != nullptr))
+        return fail(FMSCAN_E_NULL, "%s: token_partial goes with split > 1, token_grad with split == 1", who);
     const bool layer = coef_out != nullptr;
     const bool recover = layer && !cached_output;  // the states come back from states_n * rms
-    if (!gates || !out_grad || !token_grad || (!cached_output && !recover) || !gate_grad_partial)
+    if (!gates || !out_grad || (!token_grad && split == 1) || (!cached_output && !recover) || !gate_grad_partial)
         return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
                     "be NULL", who, coef_out ? "states_n" : "out_grad");
     if (recover && !rms)
@@ -48,11 +71,14 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
         return fail(FMSCAN_E_NULL, "%s: coef_self and out_grad must not be NULL", who);
     if (!pb.plain && !input_tokens)
         return fail(FMSCAN_E_NULL, "%s: input_tokens must not be NULL without FMSCAN_FLAG_PLAIN", who);
-    const int group = reduced_group(B, D);
-    const int64_t groups = fmscan_reduced_groups(B, D);
-    if (B > INT32_MAX / groups) return fail(FMSCAN_E_SHAPE, "%s: B * ceil(D/%d) must be < 2^31", who, group);
+    // what the kernel is told: B * split batch elements of M / split slots (the same memory)
+    const int64_t Bk = B * split, Mk = M / split;
+    const int group = reduced_group(Bk, D);
+    const int64_t groups = fmscan_reduced_groups(Bk, D);
+    if (Bk > INT32_MAX / groups) return fail(FMSCAN_E_SHAPE, "%s: B * split * ceil(D/%d) must be < 2^31", who, group);
     const int64_t full = pb.rows * L * pb.esize;
-    const Range outs[] = {{"token_grad", token_grad, B * D * L * pb.esize},
+    const Range outs[] = {split > 1 ? Range{"token_partial", token_partial, B * D * split * L * 4}
+                                    : Range{"token_grad", token_grad, B * D * L * pb.esize},
                           {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
                           {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
     const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
@@ -73,13 +99,14 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
             if (overlap(outs[i], outs[j]))
                 return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, outs[i].name, outs[j].name);
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
-                     aligned16(token_grad) && aligned16(cached_output) && (!recover || aligned16(rms)) &&
+                     aligned16(token_grad) && aligned16(token_partial) && aligned16(cached_output) &&
+                     (!recover || aligned16(rms)) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial) &&
                      (!layer || (aligned16(coef_out) && aligned16(coef_self) && aligned16(layer_out_grad)));
     if (!vec)
         return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
     const size_t tile = (size_t)(16 / pb.esize) * 64;
-    const int64_t Mw = (M + kReducedWaves - 1) / kReducedWaves;  // slots per wave
+    const int64_t Mw = (Mk + kReducedWaves - 1) / kReducedWaves;  // slots per wave
     const size_t lds = (2 * group * tile + 2 * (size_t)group * 2 * 64 * 4 +
                         (size_t)kReducedWaves * (size_t)Mw * group + (size_t)kReducedWaves * tile) * sizeof(float);
     if (lds > kMaxDynamicLds)
@@ -88,7 +115,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     if ((L + (int64_t)tile - 1) / (int64_t)tile > INT32_MAX)
         return fail(FMSCAN_E_SHAPE, "%s: ceil(L / %zu) must be < 2^31", who, tile);
     const void* h_init = initial_state ? initial_state : first_prop_grad;
-    const unsigned grid = (unsigned)(B * groups);
+    const unsigned grid = (unsigned)(Bk * groups);
     int rc = 0;
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
@@ -101,7 +128,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                 (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
                 (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
                 (T*)initial_state_grad, coef_out, coef_self, (const T*)layer_out_grad,
-                recover ? rms : nullptr, (int32_t)M, (int32_t)D, L, (int32_t)Mw);
+                recover ? rms : nullptr, (int32_t)Mk, (int32_t)D, L, (int32_t)Mw, token_partial, (int32_t)split);
         };
         auto with_plain = [&](auto lt) {
             if (group == 8) {
@@ -139,6 +166,41 @@ int fmscan_backward_layer(const void* gates, const void* states_n, const float* 
     return backward_reduced("fmscan_backward_layer", gates, states_n, first_prop_grad, token_grad, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
                             out_grad, rms, B, M, D, L, dtype, flags, stream);
+}
+
+int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D) {
+    if (B < 1 || M < 1 || D < 1) return 0;
+    return reduced_split(B, M, D);
+}
+
+int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D) {
+    if (B < 1 || M < 2 || D < 2) return 0;
+    // Measured against fmscan_backward followed by the two sums (bf16, ms): 512 blocks after the split
+    // (2,32,128,16384) 0.24 against 0.27, (4,32,128,8192) 0.18 against 0.27; 256 blocks (1,32,128,32768)
+    // 0.35 against 0.33; 64 blocks (1,16,64,65536) 0.56 against 0.16, (2,8,64,32768) 0.29 against 0.09.
+    return (__int128)B * ((D + 3) / 4) * reduced_split(B, M, D) >= 256 ? 1 : 0;
+}
+
+int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,
+                                  float* token_grad_partial, const void* cached_output, const void* input_tokens,
+                                  float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                                  int64_t B, int64_t M, int64_t D, int64_t L, int64_t split, int dtype,
+                                  unsigned flags, void* stream) {
+    return backward_reduced("fmscan_backward_reduced_split", gates, out_grad, first_prop_grad, nullptr, cached_output,
+                            input_tokens, gate_grad_partial, initial_state, initial_state_grad, nullptr, nullptr,
+                            nullptr, nullptr, B, M, D, L, dtype, flags, stream, token_grad_partial, split);
+}
+
+int fmscan_backward_layer_split(const void* gates, const void* states_n, const float* coef_out,
+                                const float* coef_self, const void* out_grad, const void* first_prop_grad,
+                                float* token_grad_partial, const void* cached_output, const float* rms,
+                                const void* input_tokens, float* gate_grad_partial, const void* initial_state,
+                                void* initial_state_grad, int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
+                                int dtype, unsigned flags, void* stream) {
+    if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer_split: coef_out must not be NULL");
+    return backward_reduced("fmscan_backward_layer_split", gates, states_n, first_prop_grad, nullptr, cached_output,
+                            input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
+                            out_grad, rms, B, M, D, L, dtype, flags, stream, token_grad_partial, split);
 }
 
 int fmscan_sum_groups(const float* partial, int64_t G, void* out, int64_t rows, int64_t L, int dtype,

@@ -225,24 +225,33 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
         if t is not None:
             _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
     code = _dtype_code(gates)
-    groups = _raw.fmscan_reduced_groups(B, D)
-    d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
+    # few batch elements: the slots of each are dealt to `split` blocks, whose token gradients are summed after
+    split = max(1, _raw.fmscan_reduced_split(B, M, D))
+    groups = _raw.fmscan_reduced_groups(B * split, D)
     partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
+    flags = _lib.FLAG_PLAIN if plain else 0
+    common = (cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state),
+              _ptr(initial_state_grad), B, M, D, L)
+    if split > 1:
+        token_partial = torch.empty((B, D, split, L), dtype=torch.float32, device=dev)
+        with _on_device(dev):
+            _lib.check(_raw.fmscan_backward_reduced_split(
+                gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), token_partial.data_ptr(), *common,
+                split, code, flags, torch.cuda.current_stream(dev).cuda_stream))
+        return _sum_groups(partial, gates.dtype), _sum_groups(token_partial, gates.dtype)
+    d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
     if cached_output.numel():
         with _on_device(dev):
-            stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(_raw.fmscan_backward_reduced(
-                gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), d_tokens.data_ptr(),
-                cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(),
-                None if initial_state is None else initial_state.data_ptr(),
-                None if initial_state_grad is None else initial_state_grad.data_ptr(),
-                B, M, D, L, code, _lib.FLAG_PLAIN if plain else 0, stream))
+                gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), d_tokens.data_ptr(), *common,
+                code, flags, torch.cuda.current_stream(dev).cuda_stream))
     return _sum_groups(partial, gates.dtype), d_tokens
 
 
 def _sum_groups(partial, dtype):
     """(B, M, L) of `dtype` from the float32 (B, M, G, L) partials of the gates' gradient: their sum over
-    G (what the reference does with torch.sum over a (B, M, D, L) tensor, fm_scan.py:76), rounded once."""
+    G (what the reference does with torch.sum over a (B, M, D, L) tensor, fm_scan.py:76), rounded once.
+    The same for the (B, D, split, L) partials of the token gradient."""
     B, M, G, L = partial.shape
     if G == 1 and dtype == torch.float32:
         return partial.squeeze(2)
@@ -306,8 +315,9 @@ def _scan_gradients(gates, tokens, states, initial_state, grad_output, want_init
     # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
     d_initial_state = torch.empty_like(first_prop_grad) if want_initial_state_grad else None
 
-    if _reduced_ok(gates, tokens, states, grad_output):
-        # both sums are real: one kernel produces d_gates and d_tokens directly
+    if _reduced_ok(gates, tokens, states, grad_output) and _raw.fmscan_reduced_pays(B, M, D):
+        # both sums are real: one kernel produces d_gates and d_tokens directly (unless the shape leaves
+        # it too few blocks: very few batch elements, slots and channels, very long rows)
         d_gates, d_tokens = fm_scan_backward_reduced(
             gates, grad_output, first_prop_grad, states, tokens,
             initial_state=initial_state, initial_state_grad=d_initial_state)
@@ -480,7 +490,10 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
     code = _dtype_code(gates)
     states = torch.empty((B, M, D, L), device=dev, dtype=gates.dtype)
     kept_state = initial_state if given_state else None
-    if mem_norm and states.numel() and (L * states.element_size()) % 16 == 0 and _aligned(gates, tokens, states, read):
+    # (few batch elements with few slots: the kernels below, a block per slot for the whole sequence,
+    # would leave most of the GPU idle; the separate kernels further down do not)
+    if (mem_norm and states.numel() and (L * states.element_size()) % 16 == 0
+            and _aligned(gates, tokens, states, read) and _raw.fmscan_forward_normed_pays(B, M, D)):
         inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
@@ -539,21 +552,31 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         coef_out, coef_self = torch.empty_like(q), torch.empty_like(q)  # float32, like q
         rms = torch.empty_like(q) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
-        groups = _raw.fmscan_reduced_groups(B, D)
-        d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
+        # few batch elements: the slots of each are dealt to `split` blocks, whose token gradients are summed after
+        split = max(1, _raw.fmscan_reduced_split(B, M, D))
+        groups = _raw.fmscan_reduced_groups(B * split, D)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
         d_h0 = torch.empty((B, M, D), dtype=dtype, device=dev) if want_initial_state_grad else None
+        if split > 1:
+            token_partial = torch.empty((B, D, split, L), dtype=torch.float32, device=dev)
+        else:
+            d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             _lib.check(_raw.fmscan_readout_dot(
                 states_n.data_ptr(), out_grad.data_ptr(), None, q.data_ptr(), None, _ptr(inv_rms),
                 read.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(), _ptr(rms), B, M, D, L, code, stream))
-            _lib.check(_raw.fmscan_backward_layer(
-                gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
-                out_grad.data_ptr(), None, d_tokens.data_ptr(),  # nothing arrives from beyond the last step
-                None if mem_norm else states.data_ptr(),  # with the norm: states = states_n * rms
-                _ptr(rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0),
-                B, M, D, L, code, 0, stream))
+            head = (gates.data_ptr(), states_n.data_ptr(), coef_out.data_ptr(), coef_self.data_ptr(),
+                    out_grad.data_ptr(), None)  # nothing arrives from beyond the last step
+            tail = (None if mem_norm else states.data_ptr(),  # with the norm: states = states_n * rms
+                    _ptr(rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0), B, M, D, L)
+            if split > 1:
+                _lib.check(_raw.fmscan_backward_layer_split(*head, token_partial.data_ptr(), *tail, split, code, 0,
+                                                              stream))
+            else:
+                _lib.check(_raw.fmscan_backward_layer(*head, d_tokens.data_ptr(), *tail, code, 0, stream))
+        if split > 1:
+            d_tokens = _sum_groups(token_partial, dtype)
         return partial, d_tokens, d_h0, q
 
     if out_grad is None:

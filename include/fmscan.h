@@ -237,6 +237,43 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
                           int dtype, unsigned flags, void* stream);
 
 /*
+ * fmscan_backward_reduced and fmscan_backward_layer for problems with few batch elements and
+ * long rows. Their kernel gives a block to every (b, group of 4 or 8 consecutive d) and walks
+ * the row from its end to its start, so B * ceil(D / 4) blocks are all the parallelism it has;
+ * below 512 of them part of the GPU stands idle (the reference's kernel has a block per row,
+ * fm/scan/fm_scan.cuh:221-342, and does not know the situation). With split > 1 (a divisor of
+ * M, M / split >= 4) the M slots of a batch element are dealt to `split` blocks; the token
+ * gradient, a sum over all slots, is then left as float32 partial sums
+ *   token_grad_partial  (B, D, split, L)  out, float32
+ * for fmscan_sum_groups (rows = B * D, G = split), which adds them in their order and rounds
+ * once: deterministic like the rest. gate_grad_partial is (B, M, G, L) with
+ * G = fmscan_reduced_groups(B * split, D). fmscan_reduced_split(B, M, D): the split these
+ * calls should be given for a shape (1: use the calls above; 0 for a shape that is none).
+ * No counterpart in the reference; everything else as the two calls above.
+ */
+int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D);
+/* 1 when fmscan_backward_reduced (with the split above) is expected to be at least as fast as
+ * fmscan_backward followed by the two sums, 0 when even the split leaves too few blocks (very few
+ * batch elements with few slots and channels, very long rows: fmscan_backward cuts such rows into
+ * segments, this kernel cannot). */
+int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D);
+int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,
+                                  float* token_grad_partial,
+                                  const void* cached_output, const void* input_tokens,
+                                  float* gate_grad_partial,
+                                  const void* initial_state, void* initial_state_grad,
+                                  int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
+                                  int dtype, unsigned flags, void* stream);
+int fmscan_backward_layer_split(const void* gates, const void* states_n,
+                                const float* coef_out, const float* coef_self, const void* out_grad,
+                                const void* first_prop_grad, float* token_grad_partial,
+                                const void* cached_output, const float* rms,
+                                const void* input_tokens, float* gate_grad_partial,
+                                const void* initial_state, void* initial_state_grad,
+                                int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
+                                int dtype, unsigned flags, void* stream);
+
+/*
  * The read-out of the Factorization-Memory layer (reference fm/scan/fm_scan.py:124-131,
  * inside fm_memory): RMS norm of the scanned states over the D axis of every memory slot
  *   inv_rms[b,m,t] = rsqrt(mean_d states[b,m,d,t]^2 + eps)            (:126)
@@ -304,6 +341,11 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
  * The read-out over the slots is then fmscan_readout_forward(states_n, NULL, read, NULL, output).
  */
 int64_t fmscan_forward_normed_max_d(void);
+/* 1 when this call (or fmscan_forward_sumsq below, for larger D) is expected to be the faster way to
+ * the normalised states for a shape, 0 when the three calls are: a block of these kernels is a slot
+ * (or 128 rows of one) for the whole length of the sequence, and few batch elements with few slots
+ * leave most of the GPU idle. No counterpart in the reference. */
+int fmscan_forward_normed_pays(int64_t B, int64_t M, int64_t D);
 int fmscan_forward_normed(const void* gates, const void* tokens, const void* initial_state,
                           void* states_n, float* inv_rms,
                           int64_t B, int64_t M, int64_t D, int64_t L,

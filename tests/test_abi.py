@@ -24,12 +24,15 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
-                                    "fmscan_backward_reduced", "fmscan_build_id",
+                                    "fmscan_backward_layer_split", "fmscan_backward_reduced",
+                                    "fmscan_backward_reduced_split", "fmscan_build_id",
                                     "fmscan_forward", "fmscan_forward_normed", "fmscan_forward_normed_max_d",
+                                    "fmscan_forward_normed_pays",
                                     "fmscan_forward_static", "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
                                     "fmscan_layer_prepare", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
-                                    "fmscan_reduced_groups", "fmscan_sum_groups", "fmscan_sumsq_finish", "fmscan_sumsq_groups",
+                                    "fmscan_reduced_groups", "fmscan_reduced_pays", "fmscan_reduced_split", "fmscan_sum_groups", "fmscan_sumsq_finish",
+                                    "fmscan_sumsq_groups",
                                     "fmscan_swap_last_two",
                                     "fmscan_workspace_bytes"]
 
@@ -112,6 +115,31 @@ def test_rejected_arguments(lib):
     assert lay(h=None) == E_NULL                      # no saved states and no inv_rms to take them back with
     assert lay(h=None, r=3 * P) == E_ALIAS            # inv_rms under token_grad
     assert lay(dx=9 * P) == E_ALIAS                   # token_grad on top of the layer's out_grad
+    # the same two with the slots of a batch element dealt to `split` blocks
+    reds = lambda **k: lib.fmscan_backward_reduced_split(
+        P, 2 * P, None, k.get("tp", 3 * P), 4 * P, 5 * P, 6 * P, None, None, 2, 8, 2, 8, k.get("split", 2), 0, 0, None)
+    assert reds(split=3) == E_SHAPE                   # 3 does not divide M = 8
+    assert reds(split=0) == E_SHAPE
+    assert reds(tp=None) == E_NULL                    # the split token gradient has nowhere to go
+    assert reds(split=1) == E_NULL                    # and without a split it is not what is written
+    assert reds(tp=4 * P) == E_ALIAS                  # token_grad_partial on top of cached_output
+    lays = lambda **k: lib.fmscan_backward_layer_split(
+        P, 2 * P, k.get("co", 7 * P), 8 * P, 9 * P, None, k.get("tp", 3 * P), 4 * P, None, 5 * P, 6 * P, None, None,
+        2, 8, 2, 8, k.get("split", 4), 0, 0, None)
+    assert lays(co=None) == E_NULL
+    assert lays(split=5) == E_SHAPE
+    assert lays(tp=9 * P) == E_ALIAS                  # token_grad_partial on top of the layer's out_grad
+    # which split the library asks for: none where (b, group of 4 d) pairs fill the GPU or the slots are few,
+    # else the smallest divisor of M that brings the pairs to 512 blocks, every wave of a block keeping a slot
+    split = lib.fmscan_reduced_split
+    assert split(32, 32, 128) == 1 and split(1, 7, 64) == 1 and split(0, 32, 128) == 0
+    assert split(1, 32, 128) == 8 and split(2, 32, 128) == 8 and split(4, 32, 128) == 4 and split(8, 32, 128) == 2
+    assert split(1, 16, 64) == 4 and split(3, 12, 20) == 3
+    # whether the kernels with the sums inside, or scan and norm in one kernel, are expected to pay
+    assert lib.fmscan_reduced_pays(32, 32, 128) == 1 and lib.fmscan_reduced_pays(2, 32, 128) == 1
+    assert lib.fmscan_reduced_pays(1, 16, 64) == 0 and lib.fmscan_reduced_pays(4, 1, 64) == 0
+    assert lib.fmscan_forward_normed_pays(32, 32, 128) == 1 and lib.fmscan_forward_normed_pays(2, 32, 128) == 1
+    assert lib.fmscan_forward_normed_pays(1, 32, 128) == 0 and lib.fmscan_forward_normed_pays(1, 8, 2048) == 1
     # groups of 8 rows where B * ceil(D / 8) fills the GPU twice over, of 4 otherwise
     assert lib.fmscan_reduced_groups(32, 128) == 16 and lib.fmscan_reduced_groups(1, 128) == 32
     assert lib.fmscan_reduced_groups(2, 9) == 3 and lib.fmscan_reduced_groups(512, 9) == 2 and lib.fmscan_reduced_groups(0, 9) == 0

@@ -25,7 +25,8 @@ per returned quantity. Tolerances, with what they pay for:
 The shapes take every branch of the layer's backward: both sums inside one kernel (M > 1, D > 1,
 16-byte rows), M = 1, D = 1, D not a multiple of the 8 rows a block sums over, rows that are not
 16-byte multiples (element access), rows shorter than a tile, a loss on the output alone and on
-both results, with and without an initial state. D = 1 with the norm is run with eps of the order
+both results, with and without an initial state, and the routes that depend on how many blocks a
+shape gives (scan and norm in one kernel or apart; the slots of a batch element in one block or several). D = 1 with the norm is run with eps of the order
 of the squared states: for eps << h^2 that gradient is pure cancellation and no implementation
 that stores the normalised states can deliver it (tests/test_oracle.py::
 test_norm_gradient_with_one_channel_is_all_cancellation).
@@ -84,6 +85,8 @@ LAYER_SHAPES = [
     ((1, 2048, 2, 130), 1e-4, "D beyond one block of the read-out"),
     ((64, 40, 3, 60), 1e-4, "enough blocks for groups of 8 rows in backward, the last group ragged"),
     ((16, 520, 5, 256), 1e-4, "groups of 8 rows, a ragged last tile, waves with one slot or none"),
+    ((16, 264, 4, 24), 1e-4, "64 slots: scan and norm in one kernel, 8 waves of 4 rows"),
+    ((1, 1032, 16, 20), 1e-4, "one batch element: separate kernels forward, slots dealt to four blocks backward"),
 ]
 
 
@@ -249,9 +252,11 @@ def test_layer_rejects_a_misplaced_initial_state(scan):
 
 def test_layer_with_more_than_2_31_state_elements(scan):
     """(B, L, M, D) = (9, 65536, 32, 128): 2^31 + 2^28 elements of the states, which the reference's
-    32-bit indices could not address (fm_scan.cuh:76-82). Batch elements are independent and every
-    kernel of the layer sums in a fixed order, so the last batch element, all of it beyond element
-    2^31, must come out bit for bit as a layer call on that batch element alone does."""
+    32-bit indices could not address (fm_scan.cuh:76-82). Batch elements are independent, so the last
+    batch element, all of it beyond element 2^31, must come out as a layer call on that batch element
+    alone does: to rounding, not bit for bit, since a single batch element takes other routes (scan and
+    norm in separate kernels, its slots dealt to several blocks in backward) whose float32 sums run in
+    another order. A wrong index would be an error of order one."""
     B, L, M, D, dt = 9, 65536, 32, 128, torch.bfloat16
     gen = torch.Generator(device=DEV).manual_seed(5)
     rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
@@ -275,7 +280,11 @@ def test_layer_with_more_than_2_31_state_elements(scan):
     alone = run(slice(B - 1, B))
     for name, a, b in zip(("output", "memory_states", "d_alpha", "d_update_scale", "d_output_scale", "d_inputs"),
                           last, alone):
-        assert torch.equal(a, b), name
+        a, b = a.float(), b.float()
+        differing = float((a != b).float().mean())
+        err = float((a - b).norm() / b.norm())
+        print(f"{name}: {differing:.2%} of the entries differ, {err:.1e} normwise")
+        assert err < 1e-3, (name, err)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
