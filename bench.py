@@ -378,6 +378,84 @@ def layer_step(torch, dev):
     return step, B * M * D * L, f"fm_memory (B,L,M,D)=({B},{L},{M},{D}) {dtn}, mem_norm, fwd+bwd via autograd"
 
 
+# (B, L, M, D) of the layer off its benchmark shape: the same count of state elements, or half of it, with
+# fewer batch elements and longer rows, where the fused kernels' blocks (one per batch element and group of
+# channels, or per slot, for the whole sequence) become few
+LAYER_SHAPES = [(32, 2048, 32, 128), (8, 8192, 32, 128), (4, 8192, 32, 128), (2, 16384, 32, 128), (1, 32768, 32, 128),
+                (1, 65536, 16, 64), (1, 8192, 32, 2048), (64, 1024, 16, 64)]
+
+
+def run_layer_shapes(torch, args) -> int:
+    """`--layer-shapes`: the layer's step (fm_memory forward + backward, bfloat16, loss on the output) over
+    LAYER_SHAPES, with the routes the library names for each shape. A table on stderr, one JSON line on stdout."""
+    import fm.scan.fm_scan as S
+
+    dev = torch.device("cuda", 0)
+    dt = torch.bfloat16
+    lib = S.module
+    rows = []
+    for (B, L, M, D) in LAYER_SHAPES:
+        gen = torch.Generator(device=dev).manual_seed(0)
+        rn = lambda *sh: torch.randn(*sh, device=dev, generator=gen)
+        alpha = torch.softmax(rn(B, L, M), -1).to(dt).requires_grad_()
+        us = torch.rand(B, L, 1, device=dev, generator=gen).to(dt).requires_grad_()
+        osc = torch.rand(B, L, 1, device=dev, generator=gen).to(dt).requires_grad_()
+        inp = rn(B, L, D).to(dt).requires_grad_()
+        w_out = rn(B, L, D).to(dt)
+        leaves = (alpha, us, osc, inp)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+
+        def step(record=False):
+            if record:
+                ev[0].record()
+            out, _ = S.fm_memory(alpha, us, osc, inp)
+            if record:
+                ev[1].record()
+            out.backward(w_out)
+            if record:
+                ev[2].record()
+            for t in leaves:
+                t.grad = None
+
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(20):
+                step()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / 20
+            best = ms if best is None else min(best, ms)
+        fwd = bwd = None
+        for _ in range(5):
+            step(True)
+            torch.cuda.synchronize()
+            f, b = ev[0].elapsed_time(ev[1]), ev[1].elapsed_time(ev[2])
+            fwd, bwd = (f if fwd is None else min(fwd, f)), (b if bwd is None else min(bwd, b))
+        n = B * M * D * L
+        rows.append({"shape": [B, L, M, D], "elements": n, "ms_per_step": round(best, 4), "fwd_ms": round(fwd, 4),
+                     "bwd_ms": round(bwd, 4), "Gelem_per_s": round(n / best / 1e6, 1),
+                     "scan_and_norm_in_one_kernel": bool(lib.fmscan_forward_normed_pays(B, M, D)),
+                     "slots_dealt_to_blocks": int(lib.fmscan_reduced_split(B, M, D)),
+                     "groups_of_d": int(lib.fmscan_reduced_groups(B * max(1, lib.fmscan_reduced_split(B, M, D)), D))})
+        del alpha, us, osc, inp, w_out
+        torch.cuda.empty_cache()
+    print(f"{'(B, L, M, D)':>24s} {'elements':>11s} {'step ms':>8s} {'fwd':>7s} {'bwd':>7s} {'Gelem/s':>8s}  routes",
+          file=sys.stderr)
+    for r in rows:
+        print(f"{str(tuple(r['shape'])):>24s} {r['elements']:11d} {r['ms_per_step']:8.3f} {r['fwd_ms']:7.3f} "
+              f"{r['bwd_ms']:7.3f} {r['Gelem_per_s']:8.1f}  "
+              f"{'scan + norm in one kernel' if r['scan_and_norm_in_one_kernel'] else 'scan, norm, read-out apart'}; "
+              f"slots of a batch element in {r['slots_dealt_to_blocks']} block(s), {r['groups_of_d']} groups of d",
+              file=sys.stderr)
+    print(json.dumps({"metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
+                      "unit": "Gelem/s", "dtype": "f32", "storage_dtype": "bf16", "data": "synthetic",
+                      "shapes": rows}), flush=True)
+    return 0
+
+
 def run_layer(torch, args) -> int:
     import fm.scan.fm_scan as S
 
@@ -629,6 +707,9 @@ def main() -> int:
                     help="no benchmark line: a text table of the library's choice of kernel variant against "
                          "every override, over a grid of shapes off the benchmark configurations")
     ap.add_argument("--grid-raw", default="", help="with --grid: also write every timing, one JSON object a line, to this file")
+    ap.add_argument("--layer-shapes", action="store_true",
+                    help="the layer's step over shapes with fewer batch elements and longer rows than the "
+                         "benchmark's, with the routes the library takes for each; a table on stderr")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replays (what a launch-bound "
                          "caller, e.g. the small configuration 1, gets without the per-call Python cost)")
@@ -651,6 +732,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.grid:
         return run_grid(torch, args)
+    if args.layer_shapes:
+        return run_layer_shapes(torch, args)
     if args.workload == "layer":
         return run_layer(torch, args)
     B, Cn, T, dtn = WORKLOADS[args.workload]
