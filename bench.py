@@ -437,7 +437,9 @@ def run_layer_shapes(torch, args) -> int:
         n = B * M * D * L
         rows.append({"shape": [B, L, M, D], "elements": n, "ms_per_step": round(best, 4), "fwd_ms": round(fwd, 4),
                      "bwd_ms": round(bwd, 4), "Gelem_per_s": round(n / best / 1e6, 1),
-                     "scan_and_norm_in_one_kernel": bool(lib.fmscan_forward_normed_pays(B, M, D)),
+                     "sequence_cut_into": int(lib.fmscan_forward_normed_segments(B, M, D, L, 2)),  # 0: D beyond one block
+                     "scan_and_norm_in_one_kernel": bool(lib.fmscan_forward_normed_segments(B, M, D, L, 2) > 1
+                                                         or lib.fmscan_forward_normed_pays(B, M, D)),
                      "slots_dealt_to_blocks": int(lib.fmscan_reduced_split(B, M, D)),
                      "groups_of_d": int(lib.fmscan_reduced_groups(B * max(1, lib.fmscan_reduced_split(B, M, D)), D))})
         del alpha, us, osc, inp, w_out
@@ -447,7 +449,8 @@ def run_layer_shapes(torch, args) -> int:
     for r in rows:
         print(f"{str(tuple(r['shape'])):>24s} {r['elements']:11d} {r['ms_per_step']:8.3f} {r['fwd_ms']:7.3f} "
               f"{r['bwd_ms']:7.3f} {r['Gelem_per_s']:8.1f}  "
-              f"{'scan + norm in one kernel' if r['scan_and_norm_in_one_kernel'] else 'scan, norm, read-out apart'}; "
+              f"{'scan + norm in one kernel' if r['scan_and_norm_in_one_kernel'] else 'scan, norm, read-out apart'}"
+              f"{', sequence cut in %d' % r['sequence_cut_into'] if r['sequence_cut_into'] > 1 else ''}; "
               f"slots of a batch element in {r['slots_dealt_to_blocks']} block(s), {r['groups_of_d']} groups of d",
               file=sys.stderr)
     print(json.dumps({"metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",

@@ -106,6 +106,11 @@ def load() -> ctypes.CDLL:
     lib.fmscan_forward_normed_max_d.argtypes = []
     lib.fmscan_forward_normed_pays.restype = c_int
     lib.fmscan_forward_normed_pays.argtypes = [c_int64] * 3
+    lib.fmscan_forward_normed_segments.restype = c_int64
+    lib.fmscan_forward_normed_segments.argtypes = [c_int64] * 4 + [c_int]
+    lib.fmscan_forward_normed_cut.restype = c_int
+    lib.fmscan_forward_normed_cut.argtypes = [c_void_p] * 5 + dims + [c_int, c_float, c_int64, c_void_p, c_size_t,
+                                              c_void_p]
     lib.fmscan_forward_normed.restype = c_int
     lib.fmscan_forward_normed.argtypes = [c_void_p] * 5 + dims + [c_int, c_float, c_void_p]
     lib.fmscan_sumsq_groups.restype = c_int64

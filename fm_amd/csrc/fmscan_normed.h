@@ -27,11 +27,17 @@ namespace fmscan {
 // as they are and, in place of inv_rms, the sum of squares over its rows,
 // inv_rms[(b * M + m) * DB + db][t]: (B, M, DB, L) partial sums that sumsq_finish_kernel turns
 // into inv_rms. One barrier per tile. The sum of squares then costs no pass over the states.
+//
+// nseg > 1, for few slots and long rows: the sequence is cut into nseg segments of seg_tiles tiles and a
+// block is one segment of a slot (blockIdx = slot * nseg + segment). The state that enters a segment comes
+// from the step pairs of the segments before it, which scan_aggregate_kernel has left in seg_pairs (the
+// first pass of the segmented scan kernels: it reads only the gates and tokens, which are small here).
 template <typename T, int J, int NW, bool WHOLE = true>
 __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     const T* __restrict__ gates, const T* __restrict__ tokens, const T* __restrict__ h0,
     T* __restrict__ states_n /* (B, M, D, L) */, float* __restrict__ inv_rms /* (B, M, L) */, int32_t M,
-    int32_t D, int64_t L, float eps, int32_t DB) {
+    int32_t D, int64_t L, float eps, int32_t DB, int32_t nseg, int32_t seg_tiles,
+    const float2* __restrict__ seg_pairs /* (B * M * D, nseg): scan_aggregate_kernel's, or NULL */) {
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     constexpr int SLICE = TILE / NW;  // elements of a tile's sum of squares each wave finishes
@@ -45,6 +51,11 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     // the same tokens, so they are renumbered to share an XCD.
     uint32_t id = blockIdx.x;
     if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+    int32_t seg = 0;
+    if (nseg > 1) {
+        seg = uniform((int)(id % (uint32_t)nseg));
+        id /= (uint32_t)nseg;
+    }
     int64_t bm, b;  // bm = b * M + m
     int32_t db = 0;
     if constexpr (WHOLE) {
@@ -63,9 +74,21 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     auto d_of = [&](int j) { return d0 + j < D ? d0 + j : D - 1; };  // a row past D is loaded as D - 1 and dropped
     auto counted = [&](int j) { return d0 + j < D; };                // the same for the whole wave
 
+    // the tiles of this block: all of them, or those of its segment
+    const int32_t k_lo = seg * seg_tiles;
+    const int32_t k_hi = nseg > 1 && k_lo + seg_tiles < ntiles ? k_lo + seg_tiles : ntiles;
+    if (k_lo >= ntiles) return;  // the whole block (the host cuts so that this does not happen)
+
     float carry[J];
 #pragma unroll
-    for (int j = 0; j < J; ++j) carry[j] = h0 ? Elem<T>::widen(h0[bm * D + d_of(j)]) : 0.0f;
+    for (int j = 0; j < J; ++j) {
+        const int64_t row = bm * D + d_of(j);
+        carry[j] = h0 ? Elem<T>::widen(h0[row]) : 0.0f;
+        for (int32_t sg = 0; sg < seg; ++sg) {  // the segments before this one, oldest first
+            const float2 p = seg_pairs[row * nseg + sg];
+            carry[j] = __builtin_fmaf(p.x, carry[j], p.y);
+        }
+    }
 
     // lane offset (elements) inside tile k, clamped into the row (a chunk past the end reads the last one)
     auto lane_elems = [&](int32_t k) {
@@ -94,9 +117,9 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     // just unpacked from: a second set of registers handed over at the end of a tile would make that
     // hand-over wait for the tile's stores as well.
     Loads q;
-    fetch_gates(q, 0);
+    fetch_gates(q, k_lo);
 #pragma unroll
-    for (int j = 0; j < RING; ++j) fetch_tokens(q, 0, j);
+    for (int j = 0; j < RING; ++j) fetch_tokens(q, k_lo, j);
     int parity = 0;
     wait_for_loads();
     // One tile. `whole`: it lies wholly inside the row and nothing is tested per lane, so that
@@ -205,8 +228,9 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
         parity ^= 1;
     };
     const int32_t whole_tiles = (int32_t)(L / TILE);
-    for (int32_t k = 0; k < whole_tiles; ++k) tile(k, std::true_type{});
-    if (whole_tiles < ntiles) tile(whole_tiles, std::false_type{});
+    const int32_t k_whole = k_hi < whole_tiles ? k_hi : whole_tiles;
+    for (int32_t k = k_lo; k < k_whole; ++k) tile(k, std::true_type{});
+    if (whole_tiles < k_hi) tile(whole_tiles, std::false_type{});  // (k_hi == ntiles: the row's last, short tile)
 }
 
 // inv_rms[r][t] = rsqrt(sum_g partial[r][g][t] / D + eps) for the (B, M, G, L) partial sums of

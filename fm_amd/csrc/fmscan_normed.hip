@@ -10,11 +10,40 @@ namespace {
 
 constexpr int64_t kNormedMaxD = 128;  // rows of one slot a block can hold in registers (16 waves x 8 rows)
 
+// How a slot's sequence is cut (nseg == 1: not at all).
+struct Cut {
+    int32_t nseg, seg_tiles;
+    float2* pairs;
+};
+
 template <typename T, int J, int NW>
 void launch_normed(const void* g, const void* x, const void* h0, void* out, float* inv_rms, int64_t B, int64_t M,
-                   int64_t D, int64_t L, float eps, hipStream_t s) {
-    fmscan::scan_forward_normed_kernel<T, J, NW><<<(unsigned)(B * M), 64 * NW, 0, s>>>(
-        (const T*)g, (const T*)x, (const T*)h0, (T*)out, inv_rms, (int32_t)M, (int32_t)D, L, eps, 1);
+                   int64_t D, int64_t L, float eps, Cut cut, hipStream_t s) {
+    if (cut.nseg > 1) {  // pass one: every segment of every row to its step pair, a wave per segment
+        constexpr int R = 4, P = 3;
+        const int64_t slots = B * M * D * cut.nseg;
+        fmscan::scan_aggregate_kernel<T, R, P, false, true, false><<<(unsigned)((slots + R - 1) / R), 64 * R, 0, s>>>(
+            (const T*)g, (const T*)x, cut.pairs, B * M * D, (int32_t)M, (int32_t)D, L, cut.nseg, (int64_t)cut.seg_tiles);
+    }
+    fmscan::scan_forward_normed_kernel<T, J, NW><<<(unsigned)(B * M * cut.nseg), 64 * NW, 0, s>>>(
+        (const T*)g, (const T*)x, (const T*)h0, (T*)out, inv_rms, (int32_t)M, (int32_t)D, L, eps, 1, cut.nseg,
+        cut.seg_tiles, cut.pairs);
+}
+
+// Segments for a slot's sequence so that B * M * segments blocks reach one per compute unit, none shorter
+// than four tiles; 1 when the slots alone do, or the rows are too short to cut.
+Cut plan_cut(int64_t B, int64_t M, int64_t L, int esize) {
+    const int64_t tile = (16 / esize) * 64, ntiles = (L + tile - 1) / tile;
+    Cut c{1, (int32_t)(ntiles < INT32_MAX ? ntiles : INT32_MAX), nullptr};
+    const __int128 slots = (__int128)B * M;
+    if (slots >= 256 || ntiles < 8 || ntiles >= INT32_MAX) return c;
+    int64_t want = (int64_t)((256 + slots - 1) / slots);
+    if (want > ntiles / 4) want = ntiles / 4;
+    if (want > 64) want = 64;
+    const int64_t seg_tiles = (ntiles + want - 1) / want;
+    c.seg_tiles = (int32_t)seg_tiles;
+    c.nseg = (int32_t)((ntiles + seg_tiles - 1) / seg_tiles);
+    return c;
 }
 
 constexpr int kSumsqRows = 8, kSumsqWaves = 16;  // rows per wave and waves per block of the partial-sum form
@@ -36,10 +65,10 @@ int fmscan_forward_normed_pays(int64_t B, int64_t M, int64_t D) {
     return (__int128)B * M * ((D + kNormedMaxD - 1) / kNormedMaxD) >= 64 ? 1 : 0;
 }
 
-int fmscan_forward_normed(const void* gates, const void* tokens, const void* initial_state, void* states_n,
-                          float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, float eps,
-                          void* stream) {
-    const char* who = "fmscan_forward_normed";
+// fmscan_forward_normed (segments == 1) and fmscan_forward_normed_cut.
+static int forward_normed(const char* who, const void* gates, const void* tokens, const void* initial_state,
+                          void* states_n, float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                          float eps, int64_t segments, void* workspace, size_t workspace_bytes, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, 0, &pb)) return rc;
     if (!gates || !tokens || !states_n || !inv_rms)
@@ -59,14 +88,60 @@ int fmscan_forward_normed(const void* gates, const void* tokens, const void* ini
     if (overlap(outs[0], outs[1])) return fail(FMSCAN_E_ALIAS, "%s: states_n overlaps inv_rms", who);
     if ((L * pb.esize) % 16 != 0 || !aligned16(gates) || !aligned16(tokens) || !aligned16(states_n))
         return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
+    // the cut: as many segments as asked for, each a whole number of tiles, none empty
+    const int64_t tile = (16 / pb.esize) * 64, ntiles = (L + tile - 1) / tile;
+    if (segments < 1 || segments > 255 || segments > ntiles || ntiles >= INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: segments = %lld must be between 1 and min(255, ceil(L / %lld) = %lld)", who,
+                    (long long)segments, (long long)tile, (long long)ntiles);
+    Cut cut{1, (int32_t)ntiles, nullptr};
+    if (segments > 1) {
+        cut.seg_tiles = (int32_t)((ntiles + segments - 1) / segments);
+        cut.nseg = (int32_t)((ntiles + cut.seg_tiles - 1) / cut.seg_tiles);
+        const __int128 need = (__int128)pb.rows * cut.nseg * (int64_t)sizeof(float2);
+        if (!workspace || ((uintptr_t)workspace & 7u) || (__int128)workspace_bytes < need)
+            return fail(FMSCAN_E_WORKSPACE, "%s: %d segments need an 8-byte aligned workspace of %lld bytes (got %zu)",
+                        who, cut.nseg, (long long)need, workspace_bytes);
+        if ((__int128)B * M * cut.nseg > (__int128)INT32_MAX || (__int128)pb.rows * cut.nseg > ((__int128)1 << 33))
+            return fail(FMSCAN_E_SHAPE, "%s: B * M * D * segments is too large for one launch", who);
+        const Range ws{"workspace", workspace, (int64_t)need};
+        for (const Range& r : outs)
+            if (overlap(ws, r)) return fail(FMSCAN_E_ALIAS, "%s: workspace overlaps %s", who, r.name);
+        for (const Range& r : ins)
+            if (overlap(ws, r)) return fail(FMSCAN_E_ALIAS, "%s: workspace overlaps %s", who, r.name);
+        cut.pairs = (float2*)workspace;
+    }
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
         hipStream_t s = (hipStream_t)stream;
-        if (D <= 32) launch_normed<T, 4, 8>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, s);
-        else if (D <= 64) launch_normed<T, 4, 16>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, s);
-        else launch_normed<T, 8, 16>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, s);
+        if (D <= 32) launch_normed<T, 4, 8>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, cut, s);
+        else if (D <= 64) launch_normed<T, 4, 16>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, cut, s);
+        else launch_normed<T, 8, 16>(gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, eps, cut, s);
     });
     return launched(who);
+}
+
+}  // extern "C"
+
+extern "C" {
+
+int fmscan_forward_normed(const void* gates, const void* tokens, const void* initial_state, void* states_n,
+                          float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, float eps,
+                          void* stream) {
+    return forward_normed("fmscan_forward_normed", gates, tokens, initial_state, states_n, inv_rms, B, M, D, L, dtype,
+                          eps, 1, nullptr, 0, stream);
+}
+
+int64_t fmscan_forward_normed_segments(int64_t B, int64_t M, int64_t D, int64_t L, int dtype) {
+    if (B < 1 || M < 1 || D < 1 || L < 1 || D > kNormedMaxD) return 0;
+    if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16) return 0;
+    return plan_cut(B, M, L, dtype == FMSCAN_DTYPE_F32 ? 4 : 2).nseg;
+}
+
+int fmscan_forward_normed_cut(const void* gates, const void* tokens, const void* initial_state, void* states_n,
+                              float* inv_rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype, float eps,
+                              int64_t segments, void* workspace, size_t workspace_bytes, void* stream) {
+    return forward_normed("fmscan_forward_normed_cut", gates, tokens, initial_state, states_n, inv_rms, B, M, D, L,
+                          dtype, eps, segments, workspace, workspace_bytes, stream);
 }
 
 int64_t fmscan_sumsq_groups(int64_t D) {
@@ -100,7 +175,7 @@ int fmscan_forward_sumsq(const void* gates, const void* tokens, const void* init
         fmscan::scan_forward_normed_kernel<T, kSumsqRows, kSumsqWaves, false>
             <<<(unsigned)(B * M * groups), 64 * kSumsqWaves, 0, (hipStream_t)stream>>>(
                 (const T*)gates, (const T*)tokens, (const T*)initial_state, (T*)states, sumsq_partial, (int32_t)M,
-                (int32_t)D, L, 0.0f, (int32_t)groups);
+                (int32_t)D, L, 0.0f, (int32_t)groups, 1, 0, nullptr);
     });
     return launched(who);
 }

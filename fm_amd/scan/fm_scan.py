@@ -490,19 +490,25 @@ def _layer_forward(gates, tokens, initial_state, read, mem_norm, norm_eps):
     code = _dtype_code(gates)
     states = torch.empty((B, M, D, L), device=dev, dtype=gates.dtype)
     kept_state = initial_state if given_state else None
-    # (few batch elements with few slots: the kernels below, a block per slot for the whole sequence,
-    # would leave most of the GPU idle; the separate kernels further down do not)
-    if (mem_norm and states.numel() and (L * states.element_size()) % 16 == 0
-            and _aligned(gates, tokens, states, read) and _raw.fmscan_forward_normed_pays(B, M, D)):
+    # (few batch elements with few slots: the kernels below, a block per slot for the whole sequence, would
+    # leave most of the GPU idle; the sequence is then cut into segments, or, where it is too short for
+    # that or D too large, the separate kernels further down are taken)
+    fused = mem_norm and states.numel() and (L * states.element_size()) % 16 == 0 and _aligned(gates, tokens, states, read)
+    segments = _raw.fmscan_forward_normed_segments(B, M, D, L, code) if fused else 0  # 0: D beyond one block
+    if fused and (segments > 1 or _raw.fmscan_forward_normed_pays(B, M, D)):
         inv_rms = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         with _on_device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            if D <= _raw.fmscan_forward_normed_max_d():
+            if segments >= 1:
                 # scan and norm in one kernel: the scanned states never reach memory
                 # (no initial state: NULL, which the library reads as zeros; no fill kernel)
-                _lib.check(_raw.fmscan_forward_normed(gates.data_ptr(), tokens.data_ptr(), _ptr(kept_state),
-                                                        states.data_ptr(), inv_rms.data_ptr(), B, M, D, L, code,
-                                                        float(norm_eps), stream))
+                head = (gates.data_ptr(), tokens.data_ptr(), _ptr(kept_state), states.data_ptr(), inv_rms.data_ptr(),
+                        B, M, D, L, code, float(norm_eps))
+                if segments > 1:
+                    pairs = torch.empty(B * M * D * segments * 8, dtype=torch.uint8, device=dev)
+                    _lib.check(_raw.fmscan_forward_normed_cut(*head, segments, pairs.data_ptr(), pairs.numel(), stream))
+                else:
+                    _lib.check(_raw.fmscan_forward_normed(*head, stream))
                 output, _, _ = fm_readout_forward(states, read, mem_norm=False)  # the read-out alone
                 return output, None, states, inv_rms, kept_state
             # too many rows per slot for one block: the scan leaves the sums of squares of blocks of rows,

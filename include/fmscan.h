@@ -350,6 +350,21 @@ int fmscan_forward_normed(const void* gates, const void* tokens, const void* ini
                           void* states_n, float* inv_rms,
                           int64_t B, int64_t M, int64_t D, int64_t L,
                           int dtype, float eps, void* stream);
+/* The same with every slot's sequence cut into `segments` pieces (1 <= segments <= 255, at most one per
+ * tile of 256 float32 / 512 16-bit elements), each piece a block of its own: for few slots and long rows,
+ * where a block per slot leaves most of the GPU idle. Two passes, like fmscan_forward's cut rows: the
+ * first reduces every segment of every row to its step pair (it reads only gates and tokens) into
+ *   workspace  B * M * D * segments * 8 bytes, 8-byte aligned (FMSCAN_E_WORKSPACE otherwise),
+ * the second is the kernel of fmscan_forward_normed started inside the row with the state those pairs
+ * give. Results agree with the uncut call to rounding. fmscan_forward_normed_segments: the number of
+ * segments the library would cut a shape into (1: call fmscan_forward_normed; 0: a shape this kernel
+ * does not take). No counterpart in the reference. */
+int64_t fmscan_forward_normed_segments(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
+int fmscan_forward_normed_cut(const void* gates, const void* tokens, const void* initial_state,
+                              void* states_n, float* inv_rms,
+                              int64_t B, int64_t M, int64_t D, int64_t L,
+                              int dtype, float eps,
+                              int64_t segments, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The same for any D, in two steps: fmscan_forward_sumsq is fmscan_forward (16-byte aligned rows only,

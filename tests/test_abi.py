@@ -26,8 +26,9 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
                                     "fmscan_backward_layer_split", "fmscan_backward_reduced",
                                     "fmscan_backward_reduced_split", "fmscan_build_id",
-                                    "fmscan_forward", "fmscan_forward_normed", "fmscan_forward_normed_max_d",
-                                    "fmscan_forward_normed_pays",
+                                    "fmscan_forward", "fmscan_forward_normed", "fmscan_forward_normed_cut",
+                                    "fmscan_forward_normed_max_d", "fmscan_forward_normed_pays",
+                                    "fmscan_forward_normed_segments",
                                     "fmscan_forward_static", "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
                                     "fmscan_layer_prepare", "fmscan_readout_backward",
                                     "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
@@ -140,6 +141,21 @@ def test_rejected_arguments(lib):
     assert lib.fmscan_reduced_pays(1, 16, 64) == 0 and lib.fmscan_reduced_pays(4, 1, 64) == 0
     assert lib.fmscan_forward_normed_pays(32, 32, 128) == 1 and lib.fmscan_forward_normed_pays(2, 32, 128) == 1
     assert lib.fmscan_forward_normed_pays(1, 32, 128) == 0 and lib.fmscan_forward_normed_pays(1, 8, 2048) == 1
+    # scan and norm in one kernel with the sequence cut: no cut without a workspace, no more segments than tiles
+    cutn = lambda **k: lib.fmscan_forward_normed_cut(
+        P, 2 * P, None, 3 * P, 4 * P, 1, 2, 8, k.get("L", 4096), 0, 1e-6, k.get("segments", 4), k.get("ws", 5 * P),
+        k.get("ws_bytes", 1 << 20), None)
+    assert cutn(ws=None) == E_WORKSPACE
+    assert cutn(ws_bytes=8) == E_WORKSPACE
+    assert cutn(ws=5 * P + 4) == E_WORKSPACE
+    assert cutn(segments=0) == E_SHAPE and cutn(segments=256) == E_SHAPE
+    assert cutn(L=512, segments=3) == E_SHAPE         # two tiles of float32
+    assert cutn(ws=3 * P) == E_ALIAS                  # the workspace on top of states_n
+    segs = lib.fmscan_forward_normed_segments
+    assert segs(32, 32, 128, 2048, 2) == 1 and segs(1, 32, 128, 32768, 2) == 8 and segs(2, 32, 128, 16384, 2) == 4
+    assert segs(1, 8, 24, 2048, 2) == 1               # four tiles: too short to cut
+    assert segs(1, 8, 24, 4104, 2) == 2 and segs(1, 8, 24, 4104, 0) == 4
+    assert segs(1, 8, 200, 4104, 2) == 0 and segs(1, 8, 24, 4104, 7) == 0
     # groups of 8 rows where B * ceil(D / 8) fills the GPU twice over, of 4 otherwise
     assert lib.fmscan_reduced_groups(32, 128) == 16 and lib.fmscan_reduced_groups(1, 128) == 32
     assert lib.fmscan_reduced_groups(2, 9) == 3 and lib.fmscan_reduced_groups(512, 9) == 2 and lib.fmscan_reduced_groups(0, 9) == 0

@@ -87,6 +87,7 @@ LAYER_SHAPES = [
     ((16, 520, 5, 256), 1e-4, "groups of 8 rows, a ragged last tile, waves with one slot or none"),
     ((16, 264, 4, 24), 1e-4, "64 slots: scan and norm in one kernel, 8 waves of 4 rows"),
     ((1, 1032, 16, 20), 1e-4, "one batch element: separate kernels forward, slots dealt to four blocks backward"),
+    ((1, 4104, 8, 24), 1e-4, "few slots, long rows: scan and norm in one kernel with the sequence cut in 2 (4 in float32)"),
 ]
 
 
@@ -321,6 +322,22 @@ def test_forward_scan_and_norm_in_one_kernel(scan, dtype):
         check_all(tag + " vs three calls", {"normalised states": normed, "inv_rms": inv},
                   {"normalised states": n3.double().cpu().numpy(), "inv_rms": r3.double().cpu().numpy()},
                   {"normalised states": tol, "inv_rms": 1e-5})
+        # the sequence cut into segments (two passes): every number of segments the tiles allow up to 5,
+        # against the oracle and against the uncut call (the state that enters a segment is composed from
+        # step pairs instead of carried along: equal to float32 rounding before the states are stored)
+        tile = 256 if dtype == torch.float32 else 512
+        for segments in range(2, min(5, (L + tile - 1) // tile) + 1):
+            ws = torch.empty(B * M * D * segments * 8, dtype=torch.uint8, device=DEV)
+            cut_n, cut_inv = torch.full_like(normed, float("nan")), torch.full_like(inv, float("nan"))
+            rc = lib.fmscan_forward_normed_cut(g.data_ptr(), x.data_ptr(), None if h0 is None else h0.data_ptr(),
+                                               cut_n.data_ptr(), cut_inv.data_ptr(), B, M, D, L, code, eps, segments,
+                                               ws.data_ptr(), ws.numel(), st)
+            assert rc == 0, lib.fmscan_last_error()
+            check_all(f"{tag} cut into {segments}", {"normalised states": cut_n, "inv_rms": cut_inv},
+                      {"normalised states": o_normed, "inv_rms": o_inv}, {"normalised states": tol, "inv_rms": tol})
+            check_all(f"{tag} cut into {segments} vs uncut", {"normalised states": cut_n, "inv_rms": cut_inv},
+                      {"normalised states": normed.double().cpu().numpy(), "inv_rms": inv.double().cpu().numpy()},
+                      {"normalised states": tol, "inv_rms": 1e-5})
     # beyond the limit and unaligned: rejected, nothing launched
     D = limit + 1
     g = torch.rand(1, 1, 64, device=DEV); x = torch.rand(1, D, 64, device=DEV)
