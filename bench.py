@@ -435,13 +435,15 @@ def run_layer_shapes(torch, args) -> int:
             f, b = ev[0].elapsed_time(ev[1]), ev[1].elapsed_time(ev[2])
             fwd, bwd = (f if fwd is None else min(fwd, f)), (b if bwd is None else min(bwd, b))
         n = B * M * D * L
+        from fm_amd.scan.fm_scan import _layer_backward_plan
+        plan = _layer_backward_plan(B, M, D, L, 2)  # (split, segments) of the layer's backward kernel
         rows.append({"shape": [B, L, M, D], "elements": n, "ms_per_step": round(best, 4), "fwd_ms": round(fwd, 4),
                      "bwd_ms": round(bwd, 4), "Gelem_per_s": round(n / best / 1e6, 1),
                      "sequence_cut_into": int(lib.fmscan_forward_normed_segments(B, M, D, L, 2)),  # 0: D beyond one block
                      "scan_and_norm_in_one_kernel": bool(lib.fmscan_forward_normed_segments(B, M, D, L, 2) > 1
                                                          or lib.fmscan_forward_normed_pays(B, M, D)),
-                     "slots_dealt_to_blocks": int(lib.fmscan_reduced_split(B, M, D)),
-                     "groups_of_d": int(lib.fmscan_reduced_groups(B * max(1, lib.fmscan_reduced_split(B, M, D)), D))})
+                     "slots_dealt_to_blocks": plan[0], "backward_cut_into": plan[1],
+                     "groups_of_d": int(lib.fmscan_reduced_groups(B * plan[0], D))})
         del alpha, us, osc, inp, w_out
         torch.cuda.empty_cache()
     print(f"{'(B, L, M, D)':>24s} {'elements':>11s} {'step ms':>8s} {'fwd':>7s} {'bwd':>7s} {'Gelem/s':>8s}  routes",
@@ -451,7 +453,8 @@ def run_layer_shapes(torch, args) -> int:
               f"{r['bwd_ms']:7.3f} {r['Gelem_per_s']:8.1f}  "
               f"{'scan + norm in one kernel' if r['scan_and_norm_in_one_kernel'] else 'scan, norm, read-out apart'}"
               f"{', sequence cut in %d' % r['sequence_cut_into'] if r['sequence_cut_into'] > 1 else ''}; "
-              f"slots of a batch element in {r['slots_dealt_to_blocks']} block(s), {r['groups_of_d']} groups of d",
+              f"backward: slots of a batch element in {r['slots_dealt_to_blocks']} block(s), "
+              f"{'rows cut in %d, ' % r['backward_cut_into'] if r['backward_cut_into'] > 1 else ''}{r['groups_of_d']} groups of d",
               file=sys.stderr)
     print(json.dumps({"metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
                       "unit": "Gelem/s", "dtype": "f32", "storage_dtype": "bf16", "data": "synthetic",

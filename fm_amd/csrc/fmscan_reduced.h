@@ -56,7 +56,13 @@ namespace fmscan {
 // the kernel only has to find the token rows (and the layer's output-gradient rows) of its batch element
 // at b / split, and to leave its token gradient, a sum over its own slots only, as float32 in
 // token_partial[b / split, d, b % split, :] for a sum over the blocks of a batch element that rounds once.
-template <typename T, int J, int NW, bool PLAIN, int LAYER>
+//
+// MODE 1 and 2, for few blocks and long rows (layer forms only): the sequence is cut into nseg segments of
+// seg_tiles tiles and a block takes one segment of its rows (blockIdx = ((b, group), segment)). What arrives
+// at a segment from the steps after it comes from the step pairs of the later segments: MODE 2 is the pass
+// that makes them (for every row and segment but the first: the segment's gate product and what leaves it
+// when nothing enters; no gradient is accumulated or stored), MODE 1 the kernel proper started inside the row.
+template <typename T, int J, int NW, bool PLAIN, int LAYER, int MODE = 0>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) void scan_backward_reduced_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved,
@@ -64,7 +70,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     const T* __restrict__ h0, T* __restrict__ h0_grad, const float* __restrict__ coef_out /* (B, M, L) */,
     const float* __restrict__ coef_self /* (B, M, L) */, const T* __restrict__ layer_out_grad /* (B, D, L) */,
     const float* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L, int32_t Mw,
-    float* __restrict__ token_partial /* (B / split, D, split, L), or NULL */, int32_t split) {
+    float* __restrict__ token_partial /* (B / split, D, split, L), or NULL */, int32_t split,
+    int32_t nseg, int32_t seg_tiles, float2* __restrict__ seg_pairs /* (B * M * D, nseg); MODE 1: read, 2: written */) {
+    static_assert(MODE == 0 || LAYER != 0, "rows are cut in the layer forms only");
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     extern __shared__ float lds[];
@@ -73,6 +81,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     u32x4* shared_xy = reinterpret_cast<u32x4*>(lds + 2 * J * TILE);  // [2][J][2][64]: tokens and layer_out_grad of a tile
     float* carries = lds + 2 * J * TILE + 2 * J * 2 * 64 * 4;         // [NW][Mw * J]
     float* staging = carries + NW * Mw * J;                          // [NW][TILE], 8-element chunks only: see the partials' stores
+    [[maybe_unused]] float* gate_products = staging + NW * TILE;     // [NW][Mw] (MODE 2): a segment's gate product, per slot
 
     const int lane = threadIdx.x & 63;
     const int w = uniform((int)(threadIdx.x >> 6));
@@ -82,12 +91,26 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // takes the x-th eighth of the (b, group) pairs.
     uint32_t id = blockIdx.x;
     if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+    [[maybe_unused]] int32_t seg = 0;
+    if constexpr (MODE != 0) {
+        seg = uniform((int)(id % (uint32_t)nseg));
+        id /= (uint32_t)nseg;
+    }
     const int64_t b = uniform((int)(id / (uint32_t)NG));
     const int32_t grp = uniform((int)id - (int32_t)b * NG);
     const int32_t d0 = grp * J;
     const int32_t m0 = w * Mw;
     const int32_t mcount = uniform(M - m0 < 0 ? 0 : (M - m0 < Mw ? M - m0 : Mw));  // slots of this wave
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
+    // the tiles of this block: all of them, or those of its segment
+    const int32_t k_lo = MODE != 0 ? seg * seg_tiles : 0;
+    const int32_t k_hi = MODE != 0 && k_lo + seg_tiles < ntiles ? k_lo + seg_tiles : ntiles;
+    if constexpr (MODE != 0) {
+        if (k_lo >= ntiles) return;  // the whole block (the host cuts so that this does not happen)
+    }
+    if constexpr (MODE == 2) {
+        if (seg == 0) return;  // nothing lies before the first segment: its pair is never asked for
+    }
     const int32_t lane_off = (63 - lane) * E;  // lane l owns the chunk l chunks before the end of the tile
     float* mycarry = carries + w * Mw * J;
     const int32_t rows_here = uniform(D - d0 < J ? D - d0 : J);  // rows of this block that exist (the last group may be short)
@@ -100,8 +123,23 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         const int32_t idx = base + lane;
         const int32_t mi = idx / J, j = idx - mi * J;
         const int32_t d = d0 + j < D ? d0 + j : D - 1;
-        if (idx < mcount * J)
-            mycarry[idx] = first_prop_grad ? Elem<T>::widen(first_prop_grad[((b * M + m0 + mi) * D + d)]) : 0.0f;
+        if (idx < mcount * J) {
+            const int64_t row = (b * M + m0 + mi) * D + d;
+            float c = 0.0f;
+            if constexpr (MODE != 2) {
+                c = first_prop_grad ? Elem<T>::widen(first_prop_grad[row]) : 0.0f;
+                if constexpr (MODE == 1) {
+                    for (int32_t sg = nseg - 1; sg > seg; --sg) {  // the segments after this one, from the row's end
+                        const float2 p = seg_pairs[row * nseg + sg];
+                        c = __builtin_fmaf(p.x, c, p.y);
+                    }
+                }
+            }
+            mycarry[idx] = c;
+        }
+    }
+    if constexpr (MODE == 2) {
+        for (int32_t mi = lane; mi < mcount; mi += 64) gate_products[w * Mw + mi] = 1.0f;
     }
     // Everything here is wave-uniform. A row j of the block's group past the last d (last group) is
     // loaded like any other (as row D - 1), never accumulated or stored.
@@ -117,7 +155,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // Where the saved states are at hand (LAYER != 2) and there are tokens (!PLAIN), the states
     // of a tile are not read but made again from its gates and tokens and the one saved state
     // before the tile, as scan_backward_kernel does.
-    constexpr bool REMAKE = LAYER != 2 && !PLAIN;
+    constexpr bool REMAKE = LAYER != 2 && !PLAIN && MODE != 2;  // (pass one has no use for the states)
     const uint32_t vzero = opaque_zero();
     struct Row {
         u32x4 a;   // out_grad, or the normalised states (LAYER)
@@ -192,7 +230,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     auto ahead = [&](int32_t& k, int32_t& mi) {
         if (mi + 1 < mpad) {
             ++mi;
-        } else if (k > 0) {
+        } else if (k > k_lo) {
             --k;
             mi = 0;
         }
@@ -201,7 +239,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // The J token rows of the block (and the J rows of the layer's output gradient) are the same
     // for every slot and every wave: each tile of them is loaded once per block, about J / NW rows
     // per wave, and passed through LDS, a tile ahead of its use.
-    constexpr bool kSharedX = !PLAIN, kSharedY = LAYER != 0;
+    constexpr bool kSharedX = !PLAIN && MODE != 2, kSharedY = LAYER != 0;
     struct TokenShare {
         u32x4 x[SH], y[SH];
     };
@@ -236,7 +274,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // two sets of registers that swap roles from step to step: handing one set over to the other
     // at the end of a step would have to wait for every load and store in flight.
     Slot slot_a, slot_b;
-    int32_t kf = ntiles - 1, mf = 0;  // the step after the one at work: where the loads that run ahead are
+    int32_t kf = k_hi - 1, mf = 0;  // the step after the one at work: where the loads that run ahead are
     fetch_slot(slot_a, kf, mf);
     Place place_next = place_of(kf, mf), place_now = place_next;
 #pragma unroll
@@ -245,15 +283,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     int parity = 0;
     if constexpr (kSharedX || kSharedY) {
         TokenShare first;
-        fetch_share(first, ntiles - 1);
+        fetch_share(first, k_hi - 1);
         publish_share(first, parity);
     }
     __syncthreads();  // carries and the first tile of the shared rows are in place
 
-    for (int32_t k = ntiles - 1; k >= 0; --k) {
+    for (int32_t k = k_hi - 1; k >= k_lo; --k) {
         const int64_t tw = (int64_t)k * TILE;
         TokenShare upcoming;  // the tile before this one, on its way to LDS
-        if constexpr (kSharedX || kSharedY) fetch_share(upcoming, k > 0 ? k - 1 : 0);
+        if constexpr (kSharedX || kSharedY) fetch_share(upcoming, k > k_lo ? k - 1 : k_lo);
         const bool inside = tw + lane_off < L;  // this lane's chunk lies in the row (tiles are whole chunks)
         const bool ragged = tw + TILE > L;      // the whole wave: only the row's last tile can end early
         float dtok[J][E];
@@ -273,7 +311,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                 return;
             }
             [[maybe_unused]] Rms rms_now;
-            if constexpr (LAYER == 2) fetch_rms(rms_now, k, mi);
+            if constexpr (LAYER == 2 && MODE != 2) fetch_rms(rms_now, k, mi);
 
             // per slot: gates (1 where there is no step: identity), coefficients (0 there: no gradient)
             float g[E], co[E], cs[E];
@@ -299,6 +337,9 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
             for (int i = E - 2; i >= 0; --i) a *= g[i];
             const GateLevels levels = scan_gates(a);
+            if constexpr (MODE == 2) {  // the segment's gate product so far (one value for the whole wave)
+                if (lane == 0) gate_products[w * Mw + mi] *= levels.ta;
+            }
             // (first tile: the chain of remade states starts at the saved h[0], whatever enters: the
             // first step of lane 63, which owns the start of the row, counts as gate 0, token h[0])
             const bool first_step = k == 0 && lane == 63;
@@ -350,7 +391,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
                         for (int i = 0; i < E; ++i) G[i] = inside ? G[i] : 0.0f;
                     }
-                    if constexpr (!PLAIN) Elem<T>::unpack(shared_xy[((parity * J + j) * 2 + 0) * 64 + lane], x);
+                    if constexpr (kSharedX) Elem<T>::unpack(shared_xy[((parity * J + j) * 2 + 0) * 64 + lane], x);
                     float hprev[E];  // the state before each of the chunk's steps
                     if constexpr (REMAKE) {
                         float u[E];
@@ -382,18 +423,21 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
                     float c = __builtin_fmaf(levels.ea, carry, eb);
                     carry = __builtin_fmaf(levels.ta, carry, tb);
                     if (lane == 0) carry_of[j] = carry;
+                    if constexpr (MODE != 2) {
 #pragma unroll
-                    for (int i = E - 1; i >= 0; --i) {
-                        const float delta = G[i] + c;
-                        c = g[i] * delta;
-                        // token gradient (1 - g) * delta
-                        if constexpr (PLAIN) dtok[j][i] += delta;
-                        else dtok[j][i] = __builtin_fmaf(one_minus_g[i], delta, dtok[j][i]);
-                        with_state[i] = __builtin_fmaf(hprev[i], delta, with_state[i]);
-                        if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
+                        for (int i = E - 1; i >= 0; --i) {
+                            const float delta = G[i] + c;
+                            c = g[i] * delta;
+                            // token gradient (1 - g) * delta
+                            if constexpr (PLAIN) dtok[j][i] += delta;
+                            else dtok[j][i] = __builtin_fmaf(one_minus_g[i], delta, dtok[j][i]);
+                            with_state[i] = __builtin_fmaf(hprev[i], delta, with_state[i]);
+                            if constexpr (!PLAIN) with_token[i] = __builtin_fmaf(x[i], delta, with_token[i]);
+                        }
                     }
                 }
             }
+            if constexpr (MODE == 2) return;  // pass one: the carries are all it is after
 
             // the slot's gate gradient, summed over this group of d
             float dgate[E];
@@ -449,6 +493,11 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         // (its buffer was last read two tiles ago)
         if constexpr (kSharedX || kSharedY) publish_share(upcoming, parity ^ 1);
 
+        if constexpr (MODE == 2) {  // pass one has no token gradient to hand on: the barrier of the shared rows only
+            __syncthreads();
+            parity ^= 1;
+            continue;
+        }
         // the token gradients of the tile go down the waves; the last wave stores the sums
         float* buf = handover + parity * (J * TILE);
 #pragma unroll
@@ -489,7 +538,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
         parity ^= 1;
     }
 
-    if (h0_grad) {
+    if constexpr (MODE == 2) {
+        // the segment's step pair for every row of this wave: (gate product of the slot, what left the segment)
+        __builtin_amdgcn_wave_barrier();  // lane 0's writes of the carries and products precede the reads below
+        for (int32_t base = 0; base < mcount * J; base += 64) {
+            const int32_t idx = base + lane;
+            const int32_t mi = idx / J, j = idx - mi * J;
+            if (idx >= mcount * J || d0 + j >= D) continue;
+            const int64_t row = (b * M + m0 + mi) * D + d0 + j;
+            seg_pairs[row * nseg + seg] = make_float2(gate_products[w * Mw + mi], mycarry[idx]);
+        }
+        return;
+    }
+    if (h0_grad && k_lo == 0) {  // (a cut row: the block of its first segment)
         __builtin_amdgcn_wave_barrier();  // lane 0's carry writes precede the reads below
         for (int32_t base = 0; base < mcount * J; base += 64) {
             const int32_t idx = base + lane;

@@ -49,7 +49,9 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                             float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
                             const float* coef_out, const float* coef_self, const void* layer_out_grad,
                             const float* rms, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
-                            unsigned flags, void* stream, float* token_partial = nullptr, int64_t split = 1) {
+                            unsigned flags, void* stream, float* token_partial = nullptr, int64_t split = 1,
+                            bool split_call = false, int64_t segments = 1, void* workspace = nullptr,
+                            size_t workspace_bytes = 0) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
     if (flags & ~FMSCAN_FLAG_PLAIN)
@@ -57,11 +59,11 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     if (split < 1 || M % split != 0 || split > INT32_MAX)
         return fail(FMSCAN_E_SHAPE, "%s: split = %lld must be >= 1 and divide M = %lld", who, (long long)split,
                     (long long)M);
-    if ((split > 1) != (token_partial != nullptr))
-        return fail(FMSCAN_E_NULL, "%s: token_partial goes with split > 1, token_grad with split == 1", who);
+    if ((split > 1 || split_call) != (token_partial != nullptr))
+        return fail(FMSCAN_E_NULL, "%s: token_grad_partial must not be NULL", who);
     const bool layer = coef_out != nullptr;
     const bool recover = layer && !cached_output;  // the states come back from states_n * rms
-    if (!gates || !out_grad || (!token_grad && split == 1) || (!cached_output && !recover) || !gate_grad_partial)
+    if (!gates || !out_grad || (!token_grad && !token_partial) || (!cached_output && !recover) || !gate_grad_partial)
         return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
                     "be NULL", who, coef_out ? "states_n" : "out_grad");
     if (recover && !rms)
@@ -77,7 +79,7 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     const int64_t groups = fmscan_reduced_groups(Bk, D);
     if (Bk > INT32_MAX / groups) return fail(FMSCAN_E_SHAPE, "%s: B * split * ceil(D/%d) must be < 2^31", who, group);
     const int64_t full = pb.rows * L * pb.esize;
-    const Range outs[] = {split > 1 ? Range{"token_partial", token_partial, B * D * split * L * 4}
+    const Range outs[] = {token_partial ? Range{"token_grad_partial", token_partial, B * D * split * L * 4}
                                     : Range{"token_grad", token_grad, B * D * L * pb.esize},
                           {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
                           {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
@@ -107,36 +109,76 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
         return fail(FMSCAN_E_UNALIGNED, "%s: pointers and L * sizeof(element) must be multiples of 16 bytes", who);
     const size_t tile = (size_t)(16 / pb.esize) * 64;
     const int64_t Mw = (Mk + kReducedWaves - 1) / kReducedWaves;  // slots per wave
-    const size_t lds = (2 * group * tile + 2 * (size_t)group * 2 * 64 * 4 +
-                        (size_t)kReducedWaves * (size_t)Mw * group + (size_t)kReducedWaves * tile) * sizeof(float);
+    const size_t lds = (2 * group * tile + 2 * (size_t)group * 2 * 64 * 4 + (size_t)kReducedWaves * (size_t)Mw * group +
+                        (size_t)kReducedWaves * tile + (size_t)kReducedWaves * (size_t)Mw) * sizeof(float);
     if (lds > kMaxDynamicLds)
         return fail(FMSCAN_E_SHAPE, "%s: M = %lld needs %zu bytes of LDS (limit %u)", who, (long long)M, lds,
                     kMaxDynamicLds);
     if ((L + (int64_t)tile - 1) / (int64_t)tile > INT32_MAX)
         return fail(FMSCAN_E_SHAPE, "%s: ceil(L / %zu) must be < 2^31", who, tile);
     const void* h_init = initial_state ? initial_state : first_prop_grad;
-    const unsigned grid = (unsigned)(Bk * groups);
+    // the cut: as many segments as asked for, each a whole number of tiles, none empty (layer forms,
+    // Factorization-Memory form only); two passes, the segments' step pairs between them in the workspace
+    const int64_t ntiles = (L + (int64_t)tile - 1) / (int64_t)tile;
+    if (segments < 1 || segments > 255 || segments > ntiles)
+        return fail(FMSCAN_E_SHAPE, "%s: segments = %lld must be between 1 and min(255, ceil(L / %zu) = %lld)", who,
+                    (long long)segments, tile, (long long)ntiles);
+    int32_t nseg = 1, seg_tiles = (int32_t)ntiles;
+    float2* pairs = nullptr;
+    if (segments > 1) {
+        if (!layer || pb.plain)
+            return fail(FMSCAN_E_FLAGS, "%s: rows are cut in the layer form without FMSCAN_FLAG_PLAIN only", who);
+        seg_tiles = (int32_t)((ntiles + segments - 1) / segments);
+        nseg = (int32_t)((ntiles + seg_tiles - 1) / seg_tiles);
+        const __int128 need = (__int128)pb.rows * nseg * (int64_t)sizeof(float2);
+        if (!workspace || ((uintptr_t)workspace & 7u) || (__int128)workspace_bytes < need)
+            return fail(FMSCAN_E_WORKSPACE, "%s: %d segments need an 8-byte aligned workspace of %lld bytes (got %zu)",
+                        who, nseg, (long long)need, workspace_bytes);
+        if ((__int128)Bk * groups * nseg > (__int128)INT32_MAX)
+            return fail(FMSCAN_E_SHAPE, "%s: B * split * ceil(D/%d) * segments must be < 2^31", who, group);
+        const Range ws{"workspace", workspace, (int64_t)need};
+        for (const Range& o : outs)
+            if (overlap(ws, o)) return fail(FMSCAN_E_ALIAS, "%s: workspace overlaps %s", who, o.name);
+        for (const Range& in : ins)
+            if (overlap(ws, in)) return fail(FMSCAN_E_ALIAS, "%s: workspace overlaps %s", who, in.name);
+        pairs = (float2*)workspace;
+    }
+    const unsigned grid = (unsigned)(Bk * groups * nseg);
     int rc = 0;
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
-        auto go = [&](auto jt, auto pt, auto lt) {
+        auto go = [&](auto jt, auto pt, auto lt, auto mode) {
             auto kern = fmscan::scan_backward_reduced_kernel<T, decltype(jt)::value, kReducedWaves, decltype(pt)::value,
-                                                             decltype(lt)::value>;  // lt: 0 plain call, 1 layer, 2 layer + recovered states
+                                                             decltype(lt)::value,  // lt: 0 plain call, 1 layer, 2 layer + recovered states
+                                                             decltype(mode)::value>;  // 0 whole rows, 1 a segment, 2 the segments' step pairs
             static std::atomic<uint64_t> armed{0};
             if ((rc = raise_lds_limit((const void*)kern, armed, who)) != 0) return;
             kern<<<grid, 64 * kReducedWaves, lds, (hipStream_t)stream>>>(
                 (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
                 (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
                 (T*)initial_state_grad, coef_out, coef_self, (const T*)layer_out_grad,
-                recover ? rms : nullptr, (int32_t)Mk, (int32_t)D, L, (int32_t)Mw, token_partial, (int32_t)split);
+                recover ? rms : nullptr, (int32_t)Mk, (int32_t)D, L, (int32_t)Mw, token_partial, (int32_t)split, nseg,
+                seg_tiles, pairs);
         };
         auto with_plain = [&](auto lt) {
+            if constexpr (decltype(lt)::value != 0) {
+                if (nseg > 1) {  // (not plain: checked above)
+                    if (group == 8) {
+                        go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<2>{});
+                        if (!rc) go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<1>{});
+                    } else {
+                        go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<2>{});
+                        if (!rc) go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<1>{});
+                    }
+                    return;
+                }
+            }
             if (group == 8) {
-                if (pb.plain) go(IntTag<8>{}, BoolTag<true>{}, lt);
-                else go(IntTag<8>{}, BoolTag<false>{}, lt);
+                if (pb.plain) go(IntTag<8>{}, BoolTag<true>{}, lt, IntTag<0>{});
+                else go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<0>{});
             } else {
-                if (pb.plain) go(IntTag<4>{}, BoolTag<true>{}, lt);
-                else go(IntTag<4>{}, BoolTag<false>{}, lt);
+                if (pb.plain) go(IntTag<4>{}, BoolTag<true>{}, lt, IntTag<0>{});
+                else go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<0>{});
             }
         };
         if (recover) with_plain(IntTag<2>{});
@@ -173,6 +215,37 @@ int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D) {
     return reduced_split(B, M, D);
 }
 
+int fmscan_backward_layer_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, int64_t* split,
+                               int64_t* segments) {
+    if (!split || !segments) return fail(FMSCAN_E_NULL, "fmscan_backward_layer_plan: split and segments must not be NULL");
+    *split = *segments = 0;
+    if (B < 1 || M < 1 || D < 1 || L < 1)
+        return fail(FMSCAN_E_SHAPE, "fmscan_backward_layer_plan: B, M, D, L must be >= 1");
+    if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16)
+        return fail(FMSCAN_E_DTYPE, "fmscan_backward_layer_plan: unknown dtype %d", dtype);
+    *split = reduced_split(B, M, D);
+    *segments = 1;
+    // From 64 (b, group of 4 d) pairs on, dealing the slots out reaches the 512 blocks without a second
+    // read of the states, and was as fast or faster than any cut (bf16, us, split x segments:
+    // (2,32,128,16384) 8x1 194, 1x8 184; (4,32,128,8192) 4x1 135, 1x8 180). Below, rows are cut first, into
+    // up to 16 segments of four tiles or more, and the slots dealt out for what is still missing:
+    // (1,32,128,32768) 8x1 287, 1x16 186; (1,16,64,65536) 4x1 514, 1x16 144, 2x16 121.
+    const __int128 pairs = (__int128)B * ((D + 3) / 4);
+    const int64_t tile = dtype == FMSCAN_DTYPE_F32 ? 256 : 512, ntiles = (L + tile - 1) / tile;
+    const int64_t most = ntiles / 4 < 16 ? ntiles / 4 : 16;
+    if (pairs >= 64 || most < 2) return 0;
+    const int64_t want = (int64_t)((512 + pairs - 1) / pairs);
+    *segments = want < most ? want : most;
+    const int64_t rest = (int64_t)((512 + pairs * *segments - 1) / (pairs * *segments));
+    *split = 1;
+    for (int64_t s = 2; rest > 1 && s <= M / kReducedWaves; ++s) {
+        if (M % s != 0) continue;
+        *split = s;
+        if (s >= rest) break;
+    }
+    return 0;
+}
+
 int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D) {
     if (B < 1 || M < 2 || D < 2) return 0;
     // Measured against fmscan_backward followed by the two sums (bf16, ms): 512 blocks after the split
@@ -188,7 +261,7 @@ int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const
                                   unsigned flags, void* stream) {
     return backward_reduced("fmscan_backward_reduced_split", gates, out_grad, first_prop_grad, nullptr, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, nullptr, nullptr,
-                            nullptr, nullptr, B, M, D, L, dtype, flags, stream, token_grad_partial, split);
+                            nullptr, nullptr, B, M, D, L, dtype, flags, stream, token_grad_partial, split, true);
 }
 
 int fmscan_backward_layer_split(const void* gates, const void* states_n, const float* coef_out,
@@ -196,11 +269,13 @@ int fmscan_backward_layer_split(const void* gates, const void* states_n, const f
                                 float* token_grad_partial, const void* cached_output, const float* rms,
                                 const void* input_tokens, float* gate_grad_partial, const void* initial_state,
                                 void* initial_state_grad, int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
-                                int dtype, unsigned flags, void* stream) {
+                                int64_t segments, void* workspace, size_t workspace_bytes, int dtype, unsigned flags,
+                                void* stream) {
     if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer_split: coef_out must not be NULL");
     return backward_reduced("fmscan_backward_layer_split", gates, states_n, first_prop_grad, nullptr, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
-                            out_grad, rms, B, M, D, L, dtype, flags, stream, token_grad_partial, split);
+                            out_grad, rms, B, M, D, L, dtype, flags, stream, token_grad_partial, split, true, segments,
+                            workspace, workspace_bytes);
 }
 
 int fmscan_sum_groups(const float* partial, int64_t G, void* out, int64_t rows, int64_t L, int dtype,

@@ -355,6 +355,15 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def _layer_backward_plan(B, M, D, L, code):
+    """(split, segments) the library would use for the layer's backward kernel at this shape."""
+    import ctypes
+
+    split, segments = ctypes.c_int64(0), ctypes.c_int64(0)
+    _lib.check(_raw.fmscan_backward_layer_plan(B, M, D, L, code, ctypes.byref(split), ctypes.byref(segments)))
+    return max(1, split.value), max(1, segments.value)
+
+
 def fm_readout_forward(states, read, mem_norm=True, norm_eps=1e-6, *, in_place=False):
     """RMS norm over D and read-out over M of scanned states (reference fm_scan.py:124-131).
 
@@ -558,13 +567,16 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         q = torch.empty((B, M, L), dtype=torch.float32, device=dev)
         coef_out, coef_self = torch.empty_like(q), torch.empty_like(q)  # float32, like q
         rms = torch.empty_like(q) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
-        # few batch elements: the slots of each are dealt to `split` blocks, whose token gradients are summed after
-        split = max(1, _raw.fmscan_reduced_split(B, M, D))
+        # few batch elements: the rows are cut into segments and the slots of a batch element dealt to
+        # `split` blocks, as the library plans it; the token gradients of those blocks are summed after
+        split, segments = _layer_backward_plan(B, M, D, L, code)
+        divided = split > 1 or segments > 1
         groups = _raw.fmscan_reduced_groups(B * split, D)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
         d_h0 = torch.empty((B, M, D), dtype=dtype, device=dev) if want_initial_state_grad else None
-        if split > 1:
+        if divided:
             token_partial = torch.empty((B, D, split, L), dtype=torch.float32, device=dev)
+            pairs = torch.empty(B * M * D * segments * 8 if segments > 1 else 0, dtype=torch.uint8, device=dev)
         else:
             d_tokens = torch.empty((B, D, L), dtype=dtype, device=dev)
         with _on_device(dev):
@@ -576,12 +588,13 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
                     out_grad.data_ptr(), None)  # nothing arrives from beyond the last step
             tail = (None if mem_norm else states.data_ptr(),  # with the norm: states = states_n * rms
                     _ptr(rms), tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state), _ptr(d_h0), B, M, D, L)
-            if split > 1:
-                _lib.check(_raw.fmscan_backward_layer_split(*head, token_partial.data_ptr(), *tail, split, code, 0,
-                                                              stream))
+            if divided:
+                _lib.check(_raw.fmscan_backward_layer_split(
+                    *head, token_partial.data_ptr(), *tail, split, segments,
+                    pairs.data_ptr() if segments > 1 else None, pairs.numel(), code, 0, stream))
             else:
                 _lib.check(_raw.fmscan_backward_layer(*head, d_tokens.data_ptr(), *tail, code, 0, stream))
-        if split > 1:
+        if divided:
             d_tokens = _sum_groups(token_partial, dtype)
         return partial, d_tokens, d_h0, q
 

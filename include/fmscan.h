@@ -246,9 +246,18 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
  * gradient, a sum over all slots, is then left as float32 partial sums
  *   token_grad_partial  (B, D, split, L)  out, float32
  * for fmscan_sum_groups (rows = B * D, G = split), which adds them in their order and rounds
- * once: deterministic like the rest. gate_grad_partial is (B, M, G, L) with
- * G = fmscan_reduced_groups(B * split, D). fmscan_reduced_split(B, M, D): the split these
- * calls should be given for a shape (1: use the calls above; 0 for a shape that is none).
+ * once: deterministic like the rest (these two calls write it for split = 1 as well). gate_grad_partial
+ * is (B, M, G, L) with G = fmscan_reduced_groups(B * split, D). fmscan_reduced_split(B, M, D): the split
+ * these calls should be given for a shape (1: use the calls above; 0 for a shape that is none).
+ * fmscan_backward_layer_split can also cut the rows into `segments` pieces (1 <= segments <= 255, at
+ * most one per tile of 256 float32 / 512 16-bit elements; without FMSCAN_FLAG_PLAIN only), each piece a
+ * block of its own, in two passes: the first runs the kernel without accumulating or storing any gradient
+ * and leaves every segment's step pair (its gate product and what leaves it when nothing enters) in
+ *   workspace  B * M * D * segments * 8 bytes, 8-byte aligned (FMSCAN_E_WORKSPACE otherwise),
+ * the second is the kernel proper, started inside the row with what those pairs give. It reads states_n
+ * twice, which pays where the blocks are few. fmscan_backward_layer_plan(B, M, D, L, dtype, &split,
+ * &segments): the split and the number of segments the library would use for a shape (1 and 1: call
+ * fmscan_backward_layer); returns 0, or an error code with both left 0.
  * No counterpart in the reference; everything else as the two calls above.
  */
 int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D);
@@ -271,7 +280,10 @@ int fmscan_backward_layer_split(const void* gates, const void* states_n,
                                 const void* input_tokens, float* gate_grad_partial,
                                 const void* initial_state, void* initial_state_grad,
                                 int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
+                                int64_t segments, void* workspace, size_t workspace_bytes,
                                 int dtype, unsigned flags, void* stream);
+int fmscan_backward_layer_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                               int64_t* split, int64_t* segments);
 
 /*
  * The read-out of the Factorization-Memory layer (reference fm/scan/fm_scan.py:124-131,

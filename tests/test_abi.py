@@ -24,7 +24,7 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
-                                    "fmscan_backward_layer_split", "fmscan_backward_reduced",
+                                    "fmscan_backward_layer_plan", "fmscan_backward_layer_split", "fmscan_backward_reduced",
                                     "fmscan_backward_reduced_split", "fmscan_build_id",
                                     "fmscan_forward", "fmscan_forward_normed", "fmscan_forward_normed_cut",
                                     "fmscan_forward_normed_max_d", "fmscan_forward_normed_pays",
@@ -122,14 +122,29 @@ def test_rejected_arguments(lib):
     assert reds(split=3) == E_SHAPE                   # 3 does not divide M = 8
     assert reds(split=0) == E_SHAPE
     assert reds(tp=None) == E_NULL                    # the split token gradient has nowhere to go
-    assert reds(split=1) == E_NULL                    # and without a split it is not what is written
     assert reds(tp=4 * P) == E_ALIAS                  # token_grad_partial on top of cached_output
     lays = lambda **k: lib.fmscan_backward_layer_split(
         P, 2 * P, k.get("co", 7 * P), 8 * P, 9 * P, None, k.get("tp", 3 * P), 4 * P, None, 5 * P, 6 * P, None, None,
-        2, 8, 2, 8, k.get("split", 4), 0, 0, None)
+        2, 8, 2, k.get("L", 8), k.get("split", 4), k.get("segments", 1), k.get("ws", None), k.get("ws_bytes", 0), 0,
+        k.get("flags", 0), None)
     assert lays(co=None) == E_NULL
     assert lays(split=5) == E_SHAPE
     assert lays(tp=9 * P) == E_ALIAS                  # token_grad_partial on top of the layer's out_grad
+    assert lays(segments=2) == E_SHAPE                # one tile of float32: nothing to cut
+    assert lays(L=4096, segments=0) == E_SHAPE and lays(L=4096, segments=256) == E_SHAPE
+    assert lays(L=4096, segments=4) == E_WORKSPACE    # the segments' step pairs need a workspace
+    assert lays(L=4096, segments=4, ws=10 * P, ws_bytes=64) == E_WORKSPACE
+    assert lays(L=4096, segments=4, ws=10 * P, ws_bytes=1 << 20, flags=1) == E_FLAGS   # not in the plain form
+    assert lays(L=4096, segments=4, ws=3 * P, ws_bytes=1 << 20) == E_ALIAS            # on top of token_grad_partial
+    import ctypes
+    def plan(*shape):
+        sp, sg = ctypes.c_int64(-1), ctypes.c_int64(-1)
+        return lib.fmscan_backward_layer_plan(*shape, ctypes.byref(sp), ctypes.byref(sg)), sp.value, sg.value
+    assert plan(32, 32, 128, 2048, 2) == (0, 1, 1) and plan(4, 32, 128, 8192, 2) == (0, 4, 1)
+    assert plan(2, 32, 128, 16384, 2) == (0, 8, 1)    # 64 pairs of (b, 4 d): the slots dealt out, no second read
+    assert plan(1, 32, 128, 32768, 2) == (0, 1, 16) and plan(1, 16, 64, 65536, 2) == (0, 2, 16)
+    assert plan(1, 32, 128, 2048, 2) == (0, 8, 1)     # four tiles: too short to cut
+    assert plan(1, 32, 128, 2048, 9)[0] == E_DTYPE and plan(0, 32, 128, 2048, 2) == (E_SHAPE, 0, 0)
     # which split the library asks for: none where (b, group of 4 d) pairs fill the GPU or the slots are few,
     # else the smallest divisor of M that brings the pairs to 512 blocks, every wave of a block keeping a slot
     split = lib.fmscan_reduced_split

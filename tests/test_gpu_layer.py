@@ -87,7 +87,7 @@ LAYER_SHAPES = [
     ((16, 520, 5, 256), 1e-4, "groups of 8 rows, a ragged last tile, waves with one slot or none"),
     ((16, 264, 4, 24), 1e-4, "64 slots: scan and norm in one kernel, 8 waves of 4 rows"),
     ((1, 1032, 16, 20), 1e-4, "one batch element: separate kernels forward, slots dealt to four blocks backward"),
-    ((1, 4104, 8, 24), 1e-4, "few slots, long rows: scan and norm in one kernel with the sequence cut in 2 (4 in float32)"),
+    ((1, 4104, 8, 24), 1e-4, "few slots, long rows: the sequence cut in 2 (4 in float32), in scan + norm and in backward"),
 ]
 
 

@@ -933,7 +933,10 @@ def test_slots_dealt_to_several_blocks(scan, dtype):
     each dealt to `split` blocks, the token gradient left as float32 partial sums) against the unsplit
     calls on the same inputs: the gate-gradient partials and the initial state's gradient are the same
     numbers (equal bits where both calls form groups of the same size), the token gradient is the
-    unsplit one before its rounding. Every divisor of M that leaves a wave a slot, and one that does not."""
+    unsplit one before its rounding. Every divisor of M that leaves a wave a slot, and one that does not.
+    The layer form also with its rows cut into segments (two passes: what arrives at a segment from the
+    steps after it is composed from step pairs instead of carried along), 2 to 5 of them and no split at
+    all: the same to float32 rounding."""
     lib = scan.module
     st = torch.cuda.current_stream().cuda_stream
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
@@ -968,8 +971,8 @@ def test_slots_dealt_to_several_blocks(scan, dtype):
             assert lib.fmscan_backward_reduced_split(P(g), P(G), P(fpg), P(tp[0]), P(states), P(x), P(ps[0]), P(h0),
                                                      P(ds[0]), B, M, D, L, split, code, 0, st) == 0, lib.fmscan_last_error()
             assert lib.fmscan_backward_layer_split(P(g), P(states_n), P(co), P(cs), P(og), P(fpg), P(tp[1]), None, P(rms),
-                                                   P(x), P(ps[1]), P(h0), P(ds[1]), B, M, D, L, split, code, 0,
-                                                   st) == 0, lib.fmscan_last_error()
+                                                   P(x), P(ps[1]), P(h0), P(ds[1]), B, M, D, L, split, 1, None, 0, code,
+                                                   0, st) == 0, lib.fmscan_last_error()
             for k, form in enumerate(("plain call", "layer form")):
                 tag = f"{(B, M, D, L)} {dtype} split={split} {form}"
                 assert torch.equal(ds[k], dh0[k]), tag + " d_initial_state"
@@ -982,6 +985,28 @@ def test_slots_dealt_to_several_blocks(scan, dtype):
                 # the unsplit call rounds the same float32 sum, made in another order
                 check(tag + " d_tokens", summed, tok[k].double().cpu().numpy(), TOL[dtype])
                 check(tag + " d_tokens, before the rounding", tp[k].sum(dim=2), tok[k].double().cpu().numpy(), TOL[dtype])
+        tile = 256 if dtype == torch.float32 else 512
+        for split, segments in [(1, s) for s in range(2, min(5, (L + tile - 1) // tile) + 1)] + [(splits[0], 2)]:
+            if segments > (L + tile - 1) // tile:
+                continue
+            gs = lib.fmscan_reduced_groups(B * split, D)
+            tp1, ps1, ds1 = torch.empty(B, D, split, L, device=DEV), torch.empty(B, M, gs, L, device=DEV), torch.empty_like(h0)
+            ws = torch.empty(B * M * D * segments * 8, dtype=torch.uint8, device=DEV)
+            for saved, r in ((states, None), (None, rms)):  # the states at hand, or taken back from states_n * rms
+                for t in (tp1, ps1):
+                    t.fill_(float("nan"))
+                assert lib.fmscan_backward_layer_split(P(g), P(states_n), P(co), P(cs), P(og), P(fpg), P(tp1), P(saved),
+                                                       P(r), P(x), P(ps1), P(h0), P(ds1), B, M, D, L, split, segments,
+                                                       P(ws), ws.numel(), code, 0, st) == 0, lib.fmscan_last_error()
+                whole_tok, whole_part, whole_dh0 = torch.empty_like(tok[1]), torch.empty_like(part[1]), torch.empty_like(h0)
+                assert lib.fmscan_backward_layer(P(g), P(states_n), P(co), P(cs), P(og), P(fpg), P(whole_tok), P(saved),
+                                                 P(r), P(x), P(whole_part), P(h0), P(whole_dh0), B, M, D, L, code, 0,
+                                                 st) == 0, lib.fmscan_last_error()
+                tag = f"{(B, M, D, L)} {dtype} split={split} segments={segments} saved states {saved is not None}"
+                check(tag + " d_tokens", tp1.sum(dim=2), whole_tok.double().cpu().numpy(), TOL[dtype])
+                check(tag + " gate gradient", ps1.sum(dim=2), whole_part.sum(dim=2).double().cpu().numpy(),
+                      1e-5 if dtype == torch.float32 else 1e-4)
+                check(tag + " d_initial_state", ds1, whole_dh0.double().cpu().numpy(), TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
