@@ -559,7 +559,7 @@ def run_layer(torch, args) -> int:
         kernels[name] = {"ms": round(ms, 4), "algorithmic_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1)}
     dom = kernels["scan_backward_reduced_kernel (layer form)"]
     traffic, traffic_from = profiled_traffic(f"layer_kernels_B{B}_L{L}_M{M}_D{D}_{STORAGE[dtn]}",
-                                             "scan_backward_reduced_kernel*, 2>", s * N)
+                                             "scan_backward_reduced_kernel*, 2, 0>", s * N)
     result = {
         "metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
         "value": round(N / (ms_per_step * 1e-3) / 1e9, 2), "unit": "Gelem/s", "n_gpus": 1, "steps": args.steps,
