@@ -20,6 +20,8 @@ pointers and the current HIP stream; there is no CPU implementation behind them.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from .. import _lib
@@ -357,8 +359,6 @@ def _ptr(t):
 
 def _layer_backward_plan(B, M, D, L, code):
     """(split, segments) the library would use for the layer's backward kernel at this shape."""
-    import ctypes
-
     split, segments = ctypes.c_int64(0), ctypes.c_int64(0)
     _lib.check(_raw.fmscan_backward_layer_plan(B, M, D, L, code, ctypes.byref(split), ctypes.byref(segments)))
     return max(1, split.value), max(1, segments.value)
