@@ -332,16 +332,19 @@ def per_config(torch, dev, skip, steps, warmup):
             out[name]["fwd_kernel_over_copy"] = copy["forward_kernel_over_copy"]
             out[name]["bwd_kernel_over_copy"] = copy["backward_kernel_over_copy"]
         torch.cuda.empty_cache()
+    # the layer: ten launches and PyTorch's allocator per step, so the steps and warm-up of `--workload layer`
     step, N, name = layer_step(torch, dev)
-    for _ in range(warmup):
+    layer_warmup, layer_steps = max(warmup, 10), max(steps, 50)
+    for _ in range(layer_warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for _ in range(layer_steps):
         step()
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
-    out["layer"] = {"workload": name, "ms_per_step": round(ms, 4), "Gelem_per_s": round(N / ms / 1e6, 2)}
+    ms = (time.perf_counter() - t0) * 1e3 / layer_steps
+    out["layer"] = {"workload": name, "steps": layer_steps, "warmup": layer_warmup, "ms_per_step": round(ms, 4),
+                    "Gelem_per_s": round(N / ms / 1e6, 2)}
     return out
 
 
