@@ -14,10 +14,18 @@ constexpr int kReducedWaves = 4;  // waves of a block: they split the M memory s
 // partials and the work per slot that does not depend on the row; 4 otherwise, for twice the blocks.
 int reduced_group(int64_t B, int64_t D) { return (__int128)B * ((D + 7) / 8) >= 512 ? 8 : 4; }
 
-// Into how many blocks the M slots of a batch element are dealt (1: not at all) so that the (b, group of
-// 4 d) pairs, times that number, reach the 512 blocks that fill the GPU: the smallest divisor of M that
-// does, among those that leave each of a block's waves a slot (M / split >= kReducedWaves).
+// Into how many blocks the M slots of a batch element are dealt (1: not at all) so that the blocks reach
+// the 512 that fill the GPU. First choice: with groups of 8 rows, the smallest divisor of M that brings the
+// (b, group of 8 d) pairs there and leaves every wave two slots (M / split >= 2 * kReducedWaves); measured
+// in the layer form (bf16, us, unsplit -> split): (16,32,128,2048) 127 -> 101 (2), (8,32,128,8192) 298 -> 212
+// (4), (4,64,128,4096) 261 -> 108 (8), (8,16,256,4096) 122 -> 108 (2). Else with groups of 4 rows: the
+// smallest divisor that brings the (b, group of 4 d) pairs there, every wave keeping a slot.
 int64_t reduced_split(int64_t B, int64_t M, int64_t D) {
+    const __int128 pairs8 = (__int128)B * ((D + 7) / 8);
+    if (pairs8 >= 512) return 1;
+    const int64_t want8 = (int64_t)((512 + pairs8 - 1) / pairs8);
+    for (int64_t s = 2; s <= M / (2 * kReducedWaves); ++s)
+        if (M % s == 0 && s >= want8) return s;
     const __int128 pairs = (__int128)B * ((D + 3) / 4);
     if (pairs >= 512 || M < 2 * kReducedWaves) return 1;
     const int64_t want = (int64_t)((512 + pairs - 1) / pairs);

@@ -149,7 +149,7 @@ def test_rejected_arguments(lib):
     # else the smallest divisor of M that brings the pairs to 512 blocks, every wave of a block keeping a slot
     split = lib.fmscan_reduced_split
     assert split(32, 32, 128) == 1 and split(1, 7, 64) == 1 and split(0, 32, 128) == 0
-    assert split(1, 32, 128) == 8 and split(2, 32, 128) == 8 and split(4, 32, 128) == 4 and split(8, 32, 128) == 2
+    assert split(1, 32, 128) == 8 and split(2, 32, 128) == 8 and split(4, 32, 128) == 4 and split(8, 32, 128) == 4 and split(16, 32, 128) == 2
     assert split(1, 16, 64) == 4 and split(3, 12, 20) == 3
     # whether the kernels with the sums inside, or scan and norm in one kernel, are expected to pay
     assert lib.fmscan_reduced_pays(32, 32, 128) == 1 and lib.fmscan_reduced_pays(2, 32, 128) == 1
