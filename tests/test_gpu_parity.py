@@ -390,11 +390,10 @@ def test_more_than_2_31_elements(scan):
     scan.fm_scan_forward(g[-1:].contiguous(), x[-1:].contiguous(), z[-1:], s1)
     assert torch.equal(states[-1:], s1)
     dg1, dt1 = scan.fm_scan_backward_reduced(g[-1:].contiguous(), G[-1:].contiguous(), z[-1:], s1, x[-1:].contiguous())
-    # the gate gradient's partial sums are the same numbers added in the same order; a single batch
-    # element has its slots dealt to more blocks than nine have, so the token gradient's float32 sum
-    # over the slots runs in another order: equal to one bfloat16 rounding of the largest entry, 2^-8 (a
-    # wrong index would be an error of order one)
-    assert torch.equal(d_gates[-1:], dg1)
+    # a single batch element has its slots dealt to more blocks than nine have, and its rows summed in
+    # groups of 4 instead of 8, so both gradients' float32 sums run in another order: equal to one
+    # bfloat16 rounding of the largest entry, 2^-8 (a wrong index would be an error of order one)
+    check("gate gradient of the last batch element", d_gates[-1:], dg1.double().cpu().numpy(), 4e-3)
     check("token gradient of the last batch element", d_tokens[-1:], dt1.double().cpu().numpy(), 4e-3)
 
 
