@@ -397,7 +397,8 @@ def run_layer_shapes(torch, args) -> int:
     dt = torch.bfloat16
     lib = S.module
     rows = []
-    for (B, L, M, D) in LAYER_SHAPES:
+    shapes = [tuple(int(v) for v in args.layer_shape.split(","))] if args.layer_shape else LAYER_SHAPES
+    for (B, L, M, D) in shapes:
         gen = torch.Generator(device=dev).manual_seed(0)
         rn = lambda *sh: torch.randn(*sh, device=dev, generator=gen)
         alpha = torch.softmax(rn(B, L, M), -1).to(dt).requires_grad_()
@@ -716,6 +717,8 @@ def main() -> int:
                     help="no benchmark line: a text table of the library's choice of kernel variant against "
                          "every override, over a grid of shapes off the benchmark configurations")
     ap.add_argument("--grid-raw", default="", help="with --grid: also write every timing, one JSON object a line, to this file")
+    ap.add_argument("--layer-shape", default="", metavar="B,L,M,D",
+                    help="with --layer-shapes: this one shape instead of the list")
     ap.add_argument("--layer-shapes", action="store_true",
                     help="the layer's step over shapes with fewer batch elements and longer rows than the "
                          "benchmark's, with the routes the library takes for each; a table on stderr")
