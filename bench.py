@@ -439,8 +439,8 @@ def run_layer_shapes(torch, args) -> int:
             f, b = ev[0].elapsed_time(ev[1]), ev[1].elapsed_time(ev[2])
             fwd, bwd = (f if fwd is None else min(fwd, f)), (b if bwd is None else min(bwd, b))
         n = B * M * D * L
-        from fm_amd.scan.fm_scan import _layer_backward_plan
-        plan = _layer_backward_plan(B, M, D, L, 2)  # (split, segments) of the layer's backward kernel
+        from fm_amd.scan.fm_scan import _reduced_plan
+        plan = _reduced_plan(B, M, D, L, 2)  # (split, segments) of the layer's backward kernel
         rows.append({"shape": [B, L, M, D], "elements": n, "ms_per_step": round(best, 4), "fwd_ms": round(fwd, 4),
                      "bwd_ms": round(bwd, 4), "Gelem_per_s": round(n / best / 1e6, 1),
                      "sequence_cut_into": int(lib.fmscan_forward_normed_segments(B, M, D, L, 2)),  # 0: D beyond one block

@@ -94,14 +94,15 @@ def load() -> ctypes.CDLL:
     lib.fmscan_reduced_split.restype = c_int64
     lib.fmscan_reduced_split.argtypes = [c_int64] * 3
     lib.fmscan_reduced_pays.restype = c_int
-    lib.fmscan_reduced_pays.argtypes = [c_int64] * 3
+    lib.fmscan_reduced_pays.argtypes = [c_int64] * 4 + [c_int]
     lib.fmscan_backward_reduced_split.restype = c_int
-    lib.fmscan_backward_reduced_split.argtypes = [c_void_p] * 9 + [c_int64] * 5 + [c_int, c_uint, c_void_p]
+    lib.fmscan_backward_reduced_split.argtypes = ([c_void_p] * 9 + [c_int64] * 6 + [c_void_p, c_size_t]
+                                                  + [c_int, c_uint, c_void_p])
     lib.fmscan_backward_layer_split.restype = c_int
     lib.fmscan_backward_layer_split.argtypes = ([c_void_p] * 13 + [c_int64] * 6 + [c_void_p, c_size_t]
                                                 + [c_int, c_uint, c_void_p])
-    lib.fmscan_backward_layer_plan.restype = c_int
-    lib.fmscan_backward_layer_plan.argtypes = [c_int64] * 4 + [c_int, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64)]
+    lib.fmscan_reduced_plan.restype = c_int
+    lib.fmscan_reduced_plan.argtypes = [c_int64] * 4 + [c_int, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64)]
     dims = [c_int64] * 4
     lib.fmscan_readout_inv_rms.restype = c_int
     lib.fmscan_readout_inv_rms.argtypes = [c_void_p] * 2 + dims + [c_int, c_float, c_void_p]

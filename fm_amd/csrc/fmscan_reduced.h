@@ -57,7 +57,7 @@ namespace fmscan {
 // at b / split, and to leave its token gradient, a sum over its own slots only, as float32 in
 // token_partial[b / split, d, b % split, :] for a sum over the blocks of a batch element that rounds once.
 //
-// MODE 1 and 2, for few blocks and long rows (layer forms only): the sequence is cut into nseg segments of
+// MODE 1 and 2, for few blocks and long rows (not PLAIN): the sequence is cut into nseg segments of
 // seg_tiles tiles and a block takes one segment of its rows (blockIdx = ((b, group), segment)). What arrives
 // at a segment from the steps after it comes from the step pairs of the later segments: MODE 2 is the pass
 // that makes them (for every row and segment but the first: the segment's gate product and what leaves it
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     const float* __restrict__ rms /* (B, M, L): 1 / inv_rms */, int32_t M, int32_t D, int64_t L, int32_t Mw,
     float* __restrict__ token_partial /* (B / split, D, split, L), or NULL */, int32_t split,
     int32_t nseg, int32_t seg_tiles, float2* __restrict__ seg_pairs /* (B * M * D, nseg); MODE 1: read, 2: written */) {
-    static_assert(MODE == 0 || LAYER != 0, "rows are cut in the layer forms only");
+    static_assert(MODE == 0 || !PLAIN, "rows are cut in the Factorization-Memory form only");
     constexpr int E = Elem<T>::E;
     constexpr int TILE = E * 64;
     extern __shared__ float lds[];

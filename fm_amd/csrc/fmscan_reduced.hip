@@ -134,8 +134,8 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
     int32_t nseg = 1, seg_tiles = (int32_t)ntiles;
     float2* pairs = nullptr;
     if (segments > 1) {
-        if (!layer || pb.plain)
-            return fail(FMSCAN_E_FLAGS, "%s: rows are cut in the layer form without FMSCAN_FLAG_PLAIN only", who);
+        if (pb.plain)
+            return fail(FMSCAN_E_FLAGS, "%s: rows are cut without FMSCAN_FLAG_PLAIN only", who);
         seg_tiles = (int32_t)((ntiles + segments - 1) / segments);
         nseg = (int32_t)((ntiles + seg_tiles - 1) / seg_tiles);
         const __int128 need = (__int128)pb.rows * nseg * (int64_t)sizeof(float2);
@@ -169,17 +169,15 @@ static int backward_reduced(const char* who, const void* gates, const void* out_
                 seg_tiles, pairs);
         };
         auto with_plain = [&](auto lt) {
-            if constexpr (decltype(lt)::value != 0) {
-                if (nseg > 1) {  // (not plain: checked above)
-                    if (group == 8) {
-                        go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<2>{});
-                        if (!rc) go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<1>{});
-                    } else {
-                        go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<2>{});
-                        if (!rc) go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<1>{});
-                    }
-                    return;
+            if (nseg > 1) {  // (not plain: checked above)
+                if (group == 8) {
+                    go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<2>{});
+                    if (!rc) go(IntTag<8>{}, BoolTag<false>{}, lt, IntTag<1>{});
+                } else {
+                    go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<2>{});
+                    if (!rc) go(IntTag<4>{}, BoolTag<false>{}, lt, IntTag<1>{});
                 }
+                return;
             }
             if (group == 8) {
                 if (pb.plain) go(IntTag<8>{}, BoolTag<true>{}, lt, IntTag<0>{});
@@ -223,14 +221,14 @@ int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D) {
     return reduced_split(B, M, D);
 }
 
-int fmscan_backward_layer_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, int64_t* split,
+int fmscan_reduced_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, int64_t* split,
                                int64_t* segments) {
-    if (!split || !segments) return fail(FMSCAN_E_NULL, "fmscan_backward_layer_plan: split and segments must not be NULL");
+    if (!split || !segments) return fail(FMSCAN_E_NULL, "fmscan_reduced_plan: split and segments must not be NULL");
     *split = *segments = 0;
     if (B < 1 || M < 1 || D < 1 || L < 1)
-        return fail(FMSCAN_E_SHAPE, "fmscan_backward_layer_plan: B, M, D, L must be >= 1");
+        return fail(FMSCAN_E_SHAPE, "fmscan_reduced_plan: B, M, D, L must be >= 1");
     if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16)
-        return fail(FMSCAN_E_DTYPE, "fmscan_backward_layer_plan: unknown dtype %d", dtype);
+        return fail(FMSCAN_E_DTYPE, "fmscan_reduced_plan: unknown dtype %d", dtype);
     *split = reduced_split(B, M, D);
     *segments = 1;
     // From 64 (b, group of 4 d) pairs on, dealing the slots out reaches the 512 blocks without a second
@@ -254,22 +252,25 @@ int fmscan_backward_layer_plan(int64_t B, int64_t M, int64_t D, int64_t L, int d
     return 0;
 }
 
-int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D) {
-    if (B < 1 || M < 2 || D < 2) return 0;
-    // Measured against fmscan_backward followed by the two sums (bf16, ms): 512 blocks after the split
+int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype) {
+    if (B < 1 || M < 2 || D < 2 || L < 1) return 0;
+    int64_t split = 0, segments = 0;
+    if (fmscan_reduced_plan(B, M, D, L, dtype, &split, &segments) != 0) return 0;
+    // Measured against fmscan_backward followed by the two sums (bf16, ms): 512 blocks after split and cut
     // (2,32,128,16384) 0.24 against 0.27, (4,32,128,8192) 0.18 against 0.27; 256 blocks (1,32,128,32768)
     // 0.35 against 0.33; 64 blocks (1,16,64,65536) 0.56 against 0.16, (2,8,64,32768) 0.29 against 0.09.
-    return (__int128)B * ((D + 3) / 4) * reduced_split(B, M, D) >= 256 ? 1 : 0;
+    return (__int128)B * ((D + 3) / 4) * split * segments >= 256 ? 1 : 0;
 }
 
 int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,
                                   float* token_grad_partial, const void* cached_output, const void* input_tokens,
                                   float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
-                                  int64_t B, int64_t M, int64_t D, int64_t L, int64_t split, int dtype,
-                                  unsigned flags, void* stream) {
+                                  int64_t B, int64_t M, int64_t D, int64_t L, int64_t split, int64_t segments,
+                                  void* workspace, size_t workspace_bytes, int dtype, unsigned flags, void* stream) {
     return backward_reduced("fmscan_backward_reduced_split", gates, out_grad, first_prop_grad, nullptr, cached_output,
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, nullptr, nullptr,
-                            nullptr, nullptr, B, M, D, L, dtype, flags, stream, token_grad_partial, split, true);
+                            nullptr, nullptr, B, M, D, L, dtype, flags, stream, token_grad_partial, split, true, segments,
+                            workspace, workspace_bytes);
 }
 
 int fmscan_backward_layer_split(const void* gates, const void* states_n, const float* coef_out,

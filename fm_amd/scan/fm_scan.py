@@ -227,19 +227,24 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
         if t is not None:
             _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
     code = _dtype_code(gates)
-    # few batch elements: the slots of each are dealt to `split` blocks, whose token gradients are summed after
-    split = max(1, _raw.fmscan_reduced_split(B, M, D))
+    # few batch elements: the rows are cut into segments (not in the plain form) and the slots of a batch
+    # element dealt to `split` blocks, as the library plans it; those blocks' token gradients are summed after
+    split, segments = _reduced_plan(B, M, D, L, code) if cached_output.numel() else (1, 1)
+    if plain and segments > 1:
+        split, segments = max(1, _raw.fmscan_reduced_split(B, M, D)), 1
     groups = _raw.fmscan_reduced_groups(B * split, D)
     partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
     flags = _lib.FLAG_PLAIN if plain else 0
     common = (cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state),
               _ptr(initial_state_grad), B, M, D, L)
-    if split > 1:
+    if split > 1 or segments > 1:
         token_partial = torch.empty((B, D, split, L), dtype=torch.float32, device=dev)
+        pairs = torch.empty(B * M * D * segments * 8 if segments > 1 else 0, dtype=torch.uint8, device=dev)
         with _on_device(dev):
             _lib.check(_raw.fmscan_backward_reduced_split(
                 gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), token_partial.data_ptr(), *common,
-                split, code, flags, torch.cuda.current_stream(dev).cuda_stream))
+                split, segments, pairs.data_ptr() if segments > 1 else None, pairs.numel(), code, flags,
+                torch.cuda.current_stream(dev).cuda_stream))
         return _sum_groups(partial, gates.dtype), _sum_groups(token_partial, gates.dtype)
     d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
     if cached_output.numel():
@@ -317,9 +322,9 @@ def _scan_gradients(gates, tokens, states, initial_state, grad_output, want_init
     # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
     d_initial_state = torch.empty_like(first_prop_grad) if want_initial_state_grad else None
 
-    if _reduced_ok(gates, tokens, states, grad_output) and _raw.fmscan_reduced_pays(B, M, D):
+    if _reduced_ok(gates, tokens, states, grad_output) and _raw.fmscan_reduced_pays(B, M, D, L, _dtype_code(gates)):
         # both sums are real: one kernel produces d_gates and d_tokens directly (unless the shape leaves
-        # it too few blocks: very few batch elements, slots and channels, very long rows)
+        # it too few blocks: very few batch elements, slots and channels, rows too short to cut)
         d_gates, d_tokens = fm_scan_backward_reduced(
             gates, grad_output, first_prop_grad, states, tokens,
             initial_state=initial_state, initial_state_grad=d_initial_state)
@@ -357,10 +362,10 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
-def _layer_backward_plan(B, M, D, L, code):
-    """(split, segments) the library would use for the layer's backward kernel at this shape."""
+def _reduced_plan(B, M, D, L, code):
+    """(split, segments) the library would use for the backward kernels with the sums inside at this shape."""
     split, segments = ctypes.c_int64(0), ctypes.c_int64(0)
-    _lib.check(_raw.fmscan_backward_layer_plan(B, M, D, L, code, ctypes.byref(split), ctypes.byref(segments)))
+    _lib.check(_raw.fmscan_reduced_plan(B, M, D, L, code, ctypes.byref(split), ctypes.byref(segments)))
     return max(1, split.value), max(1, segments.value)
 
 
@@ -569,7 +574,7 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         rms = torch.empty_like(q) if mem_norm else None  # 1 / inv_rms: takes the scanned states back
         # few batch elements: the rows are cut into segments and the slots of a batch element dealt to
         # `split` blocks, as the library plans it; the token gradients of those blocks are summed after
-        split, segments = _layer_backward_plan(B, M, D, L, code)
+        split, segments = _reduced_plan(B, M, D, L, code)
         divided = split > 1 or segments > 1
         groups = _raw.fmscan_reduced_groups(B * split, D)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)

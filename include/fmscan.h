@@ -249,29 +249,29 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
  * once: deterministic like the rest (these two calls write it for split = 1 as well). gate_grad_partial
  * is (B, M, G, L) with G = fmscan_reduced_groups(B * split, D). fmscan_reduced_split(B, M, D): the split
  * these calls should be given for a shape (1: use the calls above; 0 for a shape that is none).
- * fmscan_backward_layer_split can also cut the rows into `segments` pieces (1 <= segments <= 255, at
+ * Both can also cut the rows into `segments` pieces (1 <= segments <= 255, at
  * most one per tile of 256 float32 / 512 16-bit elements; without FMSCAN_FLAG_PLAIN only), each piece a
  * block of its own, in two passes: the first runs the kernel without accumulating or storing any gradient
  * and leaves every segment's step pair (its gate product and what leaves it when nothing enters) in
  *   workspace  B * M * D * segments * 8 bytes, 8-byte aligned (FMSCAN_E_WORKSPACE otherwise),
  * the second is the kernel proper, started inside the row with what those pairs give. It reads states_n
- * twice, which pays where the blocks are few. fmscan_backward_layer_plan(B, M, D, L, dtype, &split,
+ * (out_grad) twice, which pays where the blocks are few. fmscan_reduced_plan(B, M, D, L, dtype, &split,
  * &segments): the split and the number of segments the library would use for a shape (1 and 1: call
- * fmscan_backward_layer); returns 0, or an error code with both left 0.
+ * fmscan_backward_layer or fmscan_backward_reduced); returns 0, or an error code with both left 0.
  * No counterpart in the reference; everything else as the two calls above.
  */
 int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D);
-/* 1 when fmscan_backward_reduced (with the split above) is expected to be at least as fast as
- * fmscan_backward followed by the two sums, 0 when even the split leaves too few blocks (very few
- * batch elements with few slots and channels, very long rows: fmscan_backward cuts such rows into
- * segments, this kernel cannot). */
-int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D);
+/* 1 when fmscan_backward_reduced (split and cut as fmscan_reduced_plan below says) is expected to be at
+ * least as fast as fmscan_backward followed by the two sums, 0 when even that leaves too few blocks
+ * (very few batch elements with few slots and channels, rows too short to cut). */
+int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
 int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,
                                   float* token_grad_partial,
                                   const void* cached_output, const void* input_tokens,
                                   float* gate_grad_partial,
                                   const void* initial_state, void* initial_state_grad,
                                   int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
+                                  int64_t segments, void* workspace, size_t workspace_bytes,
                                   int dtype, unsigned flags, void* stream);
 int fmscan_backward_layer_split(const void* gates, const void* states_n,
                                 const float* coef_out, const float* coef_self, const void* out_grad,
@@ -282,7 +282,7 @@ int fmscan_backward_layer_split(const void* gates, const void* states_n,
                                 int64_t B, int64_t M, int64_t D, int64_t L, int64_t split,
                                 int64_t segments, void* workspace, size_t workspace_bytes,
                                 int dtype, unsigned flags, void* stream);
-int fmscan_backward_layer_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+int fmscan_reduced_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
                                int64_t* split, int64_t* segments);
 
 /*

@@ -24,18 +24,17 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
-                                    "fmscan_backward_layer_plan", "fmscan_backward_layer_split", "fmscan_backward_reduced",
-                                    "fmscan_backward_reduced_split", "fmscan_build_id",
-                                    "fmscan_forward", "fmscan_forward_normed", "fmscan_forward_normed_cut",
+                                    "fmscan_backward_layer_split", "fmscan_backward_reduced",
+                                    "fmscan_backward_reduced_split", "fmscan_build_id", "fmscan_forward",
+                                    "fmscan_forward_normed", "fmscan_forward_normed_cut",
                                     "fmscan_forward_normed_max_d", "fmscan_forward_normed_pays",
-                                    "fmscan_forward_normed_segments",
-                                    "fmscan_forward_static", "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
-                                    "fmscan_layer_prepare", "fmscan_readout_backward",
-                                    "fmscan_readout_dot", "fmscan_readout_forward", "fmscan_readout_inv_rms",
-                                    "fmscan_reduced_groups", "fmscan_reduced_pays", "fmscan_reduced_split", "fmscan_sum_groups", "fmscan_sumsq_finish",
-                                    "fmscan_sumsq_groups",
-                                    "fmscan_swap_last_two",
-                                    "fmscan_workspace_bytes"]
+                                    "fmscan_forward_normed_segments", "fmscan_forward_static",
+                                    "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
+                                    "fmscan_layer_prepare", "fmscan_readout_backward", "fmscan_readout_dot",
+                                    "fmscan_readout_forward", "fmscan_readout_inv_rms", "fmscan_reduced_groups",
+                                    "fmscan_reduced_pays", "fmscan_reduced_plan", "fmscan_reduced_split",
+                                    "fmscan_sum_groups", "fmscan_sumsq_finish", "fmscan_sumsq_groups",
+                                    "fmscan_swap_last_two", "fmscan_workspace_bytes"]
 
 
 def test_every_declared_symbol_is_exported(lib):
@@ -118,11 +117,13 @@ def test_rejected_arguments(lib):
     assert lay(dx=9 * P) == E_ALIAS                   # token_grad on top of the layer's out_grad
     # the same two with the slots of a batch element dealt to `split` blocks
     reds = lambda **k: lib.fmscan_backward_reduced_split(
-        P, 2 * P, None, k.get("tp", 3 * P), 4 * P, 5 * P, 6 * P, None, None, 2, 8, 2, 8, k.get("split", 2), 0, 0, None)
+        P, 2 * P, None, k.get("tp", 3 * P), 4 * P, 5 * P, 6 * P, None, None, 2, 8, 2, k.get("L", 8), k.get("split", 2),
+        k.get("segments", 1), k.get("ws", None), k.get("ws_bytes", 0), 0, k.get("flags", 0), None)
     assert reds(split=3) == E_SHAPE                   # 3 does not divide M = 8
     assert reds(split=0) == E_SHAPE
     assert reds(tp=None) == E_NULL                    # the split token gradient has nowhere to go
     assert reds(tp=4 * P) == E_ALIAS                  # token_grad_partial on top of cached_output
+    assert reds(L=4096, segments=4) == E_WORKSPACE and reds(L=4096, segments=4, ws=10 * P, ws_bytes=1 << 20, flags=1) == E_FLAGS
     lays = lambda **k: lib.fmscan_backward_layer_split(
         P, 2 * P, k.get("co", 7 * P), 8 * P, 9 * P, None, k.get("tp", 3 * P), 4 * P, None, 5 * P, 6 * P, None, None,
         2, 8, 2, k.get("L", 8), k.get("split", 4), k.get("segments", 1), k.get("ws", None), k.get("ws_bytes", 0), 0,
@@ -139,7 +140,7 @@ def test_rejected_arguments(lib):
     import ctypes
     def plan(*shape):
         sp, sg = ctypes.c_int64(-1), ctypes.c_int64(-1)
-        return lib.fmscan_backward_layer_plan(*shape, ctypes.byref(sp), ctypes.byref(sg)), sp.value, sg.value
+        return lib.fmscan_reduced_plan(*shape, ctypes.byref(sp), ctypes.byref(sg)), sp.value, sg.value
     assert plan(32, 32, 128, 2048, 2) == (0, 1, 1) and plan(4, 32, 128, 8192, 2) == (0, 4, 1)
     assert plan(2, 32, 128, 16384, 2) == (0, 8, 1)    # 64 pairs of (b, 4 d): the slots dealt out, no second read
     assert plan(1, 32, 128, 32768, 2) == (0, 1, 16) and plan(1, 16, 64, 65536, 2) == (0, 2, 16)
@@ -152,8 +153,9 @@ def test_rejected_arguments(lib):
     assert split(1, 32, 128) == 8 and split(2, 32, 128) == 8 and split(4, 32, 128) == 4 and split(8, 32, 128) == 4 and split(16, 32, 128) == 2
     assert split(1, 16, 64) == 4 and split(3, 12, 20) == 3
     # whether the kernels with the sums inside, or scan and norm in one kernel, are expected to pay
-    assert lib.fmscan_reduced_pays(32, 32, 128) == 1 and lib.fmscan_reduced_pays(2, 32, 128) == 1
-    assert lib.fmscan_reduced_pays(1, 16, 64) == 0 and lib.fmscan_reduced_pays(4, 1, 64) == 0
+    pays = lib.fmscan_reduced_pays
+    assert pays(32, 32, 128, 2048, 2) == 1 and pays(2, 32, 128, 16384, 2) == 1
+    assert pays(1, 16, 64, 65536, 2) == 1 and pays(1, 16, 64, 2048, 2) == 0 and pays(4, 1, 64, 2048, 2) == 0
     assert lib.fmscan_forward_normed_pays(32, 32, 128) == 1 and lib.fmscan_forward_normed_pays(2, 32, 128) == 1
     assert lib.fmscan_forward_normed_pays(1, 32, 128) == 0 and lib.fmscan_forward_normed_pays(1, 8, 2048) == 1
     # scan and norm in one kernel with the sequence cut: no cut without a workspace, no more segments than tiles

@@ -968,7 +968,8 @@ def test_slots_dealt_to_several_blocks(scan, dtype):
             ps = [torch.empty(B, M, gs, L, device=DEV) for _ in range(2)]
             ds = [torch.empty_like(h0) for _ in range(2)]
             assert lib.fmscan_backward_reduced_split(P(g), P(G), P(fpg), P(tp[0]), P(states), P(x), P(ps[0]), P(h0),
-                                                     P(ds[0]), B, M, D, L, split, code, 0, st) == 0, lib.fmscan_last_error()
+                                                     P(ds[0]), B, M, D, L, split, 1, None, 0, code, 0,
+                                                     st) == 0, lib.fmscan_last_error()
             assert lib.fmscan_backward_layer_split(P(g), P(states_n), P(co), P(cs), P(og), P(fpg), P(tp[1]), None, P(rms),
                                                    P(x), P(ps[1]), P(h0), P(ds[1]), B, M, D, L, split, 1, None, 0, code,
                                                    0, st) == 0, lib.fmscan_last_error()
@@ -1006,6 +1007,17 @@ def test_slots_dealt_to_several_blocks(scan, dtype):
                 check(tag + " gate gradient", ps1.sum(dim=2), whole_part.sum(dim=2).double().cpu().numpy(),
                       1e-5 if dtype == torch.float32 else 1e-4)
                 check(tag + " d_initial_state", ds1, whole_dh0.double().cpu().numpy(), TOL[dtype])
+            # the call that is given the states' gradient as a tensor, cut the same way
+            for t in (tp1, ps1):
+                t.fill_(float("nan"))
+            assert lib.fmscan_backward_reduced_split(P(g), P(G), P(fpg), P(tp1), P(states), P(x), P(ps1), P(h0), P(ds1),
+                                                     B, M, D, L, split, segments, P(ws), ws.numel(), code, 0,
+                                                     st) == 0, lib.fmscan_last_error()
+            tag = f"{(B, M, D, L)} {dtype} split={split} segments={segments} plain call"
+            check(tag + " d_tokens", tp1.sum(dim=2), tok[0].double().cpu().numpy(), TOL[dtype])
+            check(tag + " gate gradient", ps1.sum(dim=2), part[0].sum(dim=2).double().cpu().numpy(),
+                  1e-5 if dtype == torch.float32 else 1e-4)
+            check(tag + " d_initial_state", ds1, dh0[0].double().cpu().numpy(), TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
