@@ -29,7 +29,7 @@ namespace fmscan {
 // into inv_rms. One barrier per tile. The sum of squares then costs no pass over the states.
 //
 // nseg > 1, for few slots and long rows: the sequence is cut into nseg segments of seg_tiles tiles and a
-// block is one segment of a slot (blockIdx = slot * nseg + segment). The state that enters a segment comes
+// block is one segment of a slot (blockIdx = (b, segment, m)). The state that enters a segment comes
 // from the step pairs of the segments before it, which scan_aggregate_kernel has left in seg_pairs (the
 // first pass of the segmented scan kernels: it reads only the gates and tokens, which are small here).
 template <typename T, int J, int NW, bool WHOLE = true>
@@ -51,23 +51,21 @@ __global__ __launch_bounds__(64 * NW) void scan_forward_normed_kernel(
     // the same tokens, so they are renumbered to share an XCD.
     uint32_t id = blockIdx.x;
     if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+    // the slot runs fastest, then the segment: the M blocks of one stretch of b's tokens follow each other
+    const uint32_t m_of = id % (uint32_t)M;
+    uint32_t rest = id / (uint32_t)M;
     int32_t seg = 0;
     if (nseg > 1) {
-        seg = uniform((int)(id % (uint32_t)nseg));
-        id /= (uint32_t)nseg;
+        seg = uniform((int)(rest % (uint32_t)nseg));
+        rest /= (uint32_t)nseg;
     }
-    int64_t bm, b;  // bm = b * M + m
     int32_t db = 0;
-    if constexpr (WHOLE) {
-        bm = (int64_t)uniform((int)id);
-        b = uniform((int)(id / (uint32_t)M));
-    } else {
-        const uint32_t per_b = (uint32_t)M * (uint32_t)DB;
-        const uint32_t bb = id / per_b, rest = id - bb * per_b;
-        db = uniform((int)(rest / (uint32_t)M));
-        b = uniform((int)bb);
-        bm = (int64_t)uniform((int)(bb * (uint32_t)M + (rest - (uint32_t)db * (uint32_t)M)));
+    if constexpr (!WHOLE) {
+        db = uniform((int)(rest % (uint32_t)DB));
+        rest /= (uint32_t)DB;
     }
+    const int64_t b = uniform((int)rest);
+    const int64_t bm = (int64_t)uniform((int)(rest * (uint32_t)M + m_of));  // b * M + m
     const int32_t d0 = (db * NW + w) * J;
     const int32_t ntiles = (int32_t)((L + TILE - 1) / TILE);
     const int32_t lane_off = lane * E;

@@ -58,7 +58,7 @@ namespace fmscan {
 // token_partial[b / split, d, b % split, :] for a sum over the blocks of a batch element that rounds once.
 //
 // MODE 1 and 2, for few blocks and long rows (not PLAIN): the sequence is cut into nseg segments of
-// seg_tiles tiles and a block takes one segment of its rows (blockIdx = ((b, group), segment)). What arrives
+// seg_tiles tiles and a block takes one segment of its rows (blockIdx = ((b, segment), group)). What arrives
 // at a segment from the steps after it comes from the step pairs of the later segments: MODE 2 is the pass
 // that makes them (for every row and segment but the first: the segment's gate product and what leaves it
 // when nothing enters; no gradient is accumulated or stored), MODE 1 the kernel proper started inside the row.
@@ -91,10 +91,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2))) vo
     // takes the x-th eighth of the (b, group) pairs.
     uint32_t id = blockIdx.x;
     if (gridDim.x % 8u == 0u) id = (id % 8u) * (gridDim.x / 8u) + id / 8u;
+    // Cut rows: the groups of one (b, segment) follow each other (they read the same stretch of the gates
+    // and coefficient vectors), then the blocks that share b's tokens, then the segments.
     [[maybe_unused]] int32_t seg = 0;
     if constexpr (MODE != 0) {
-        seg = uniform((int)(id % (uint32_t)nseg));
-        id /= (uint32_t)nseg;
+        const uint32_t g = id % (uint32_t)NG, r = id / (uint32_t)NG;
+        const uint32_t s = r % (uint32_t)split, r2 = r / (uint32_t)split;
+        seg = uniform((int)(r2 % (uint32_t)nseg));
+        id = ((r2 / (uint32_t)nseg) * (uint32_t)split + s) * (uint32_t)NG + g;
     }
     const int64_t b = uniform((int)(id / (uint32_t)NG));
     const int32_t grp = uniform((int)id - (int32_t)b * NG);
