@@ -27,7 +27,7 @@ CSRC = PKG / "csrc"
 UNITS = ["fmscan_core.hip", "fmscan_forward.hip", "fmscan_backward.hip", "fmscan_reduced.hip",
          "fmscan_readout.hip", "fmscan_normed.hip"]
 HEADERS = ["fmscan_host.h", "fmscan_device.h", "fmscan_kernels.h", "fmscan_reduced.h", "fmscan_readout.h",
-           "fmscan_normed.h"]
+           "fmscan_normed.h", "fmscan_packed.h"]
 DEPS = [CSRC / n for n in UNITS + HEADERS] + [PKG.parent / "include" / "fmscan.h"]
 LIB = PKG / "lib" / "libfmscan_hip.so"
 HIPCC_FLAGS = [

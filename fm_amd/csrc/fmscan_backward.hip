@@ -2,6 +2,7 @@
 // Contract: include/fmscan.h.
 #include "fmscan_host.h"
 #include "fmscan_kernels.h"
+#include "fmscan_packed.h"
 
 using namespace fmscan::host;
 
@@ -80,6 +81,23 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(out_grad) &&
                      aligned16(token_grad_out) && aligned16(cached_output) &&
                      (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_out);
+    const bool fold = M == 1 && D == 1;
+    if (packs_rows(pb, vec, true)) {  // short rows: several per wave
+        const int32_t lanes_log2 = packed_lanes_log2(pb);
+        with_dtype(dtype, [&](auto tt) {
+            using T = typename decltype(tt)::type;
+            with_bool(pb.plain, [&](auto pt) {
+                with_bool(fold, [&](auto ft) {
+                    fmscan::scan_backward_packed_kernel<T, decltype(pt)::value, decltype(ft)::value>
+                        <<<packed_blocks(pb, lanes_log2), 256, 0, (hipStream_t)stream>>>(
+                            (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad_out,
+                            (const T*)cached_output, (const T*)input_tokens, (T*)gate_grad_out, (const T*)h_init,
+                            (T*)initial_state_grad, pb.rows, (int32_t)pb.M, (int32_t)pb.D, (int32_t)pb.L, lanes_log2);
+                });
+            });
+        });
+        return launched("backward");
+    }
     Tuning tune;
     if (int rc = settle(pb, true, workspace, workspace_bytes, "fmscan_backward", &tune)) return rc;
     float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
@@ -87,7 +105,6 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
         launch_aggregate(dtype, pb, tune, vec, gates, out_grad, pairs, (hipStream_t)stream);
         if (int rc = launched("backward (segment pass)")) return rc;
     }
-    const bool fold = M == 1 && D == 1;
     int rc = 0;
     dispatch<true>(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;

@@ -2,6 +2,7 @@
 // Contract: include/fmscan.h.
 #include "fmscan_host.h"
 #include "fmscan_kernels.h"
+#include "fmscan_packed.h"
 
 using namespace fmscan::host;
 
@@ -90,6 +91,22 @@ int forward(const char* who, const void* gates, const void* tokens, const void* 
             return fail(FMSCAN_E_ALIAS, "%s: out overlaps %s", who, in.name);
 
     const bool vec = (L * pb.esize) % 16 == 0 && aligned16(gates) && aligned16(tokens) && aligned16(out);
+    const bool fold = M == 1 && D == 1;
+    if (packs_rows(pb, vec, false)) {  // short rows: several per wave
+        const int32_t lanes_log2 = packed_lanes_log2(pb);
+        with_dtype(dtype, [&](auto tt) {
+            using T = typename decltype(tt)::type;
+            with_bool(pb.plain, [&](auto pt) {
+                with_bool(fold, [&](auto ft) {
+                    fmscan::scan_forward_packed_kernel<T, decltype(pt)::value, decltype(ft)::value>
+                        <<<packed_blocks(pb, lanes_log2), 256, 0, (hipStream_t)stream>>>(
+                            (const T*)gates, (const T*)tokens, (const T*)initial_state, (T*)out, pb.rows,
+                            (int32_t)pb.M, (int32_t)pb.D, (int32_t)pb.L, lanes_log2);
+                });
+            });
+        });
+        return launched("forward");
+    }
     Tuning tune;
     if (int rc = settle(pb, false, workspace, workspace_bytes, who, &tune)) return rc;
     float2* pairs = tune.nseg > 1 ? (float2*)workspace : nullptr;
@@ -97,7 +114,6 @@ int forward(const char* who, const void* gates, const void* tokens, const void* 
         launch_aggregate(dtype, pb, tune, vec, gates, tokens, pairs, (hipStream_t)stream);
         if (int rc = launched("forward (segment pass)")) return rc;
     }
-    const bool fold = M == 1 && D == 1;
     int rc = 0;
     dispatch<false>(dtype, tune, pb.plain, vec, fold, [&](auto tt, auto wt, auto rt, auto dt, auto pt, auto vt, auto ft) {
         using T = typename decltype(tt)::type;

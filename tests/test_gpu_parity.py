@@ -565,6 +565,81 @@ def test_few_long_rows_are_cut_into_segments(scan, dtype, plain):
         check(tag + " cut vs uncut", out, out1.double().cpu().numpy(), TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_short_rows_several_per_wave(scan, dtype):
+    """Rows of at most 64 chunks of 16 bytes take the kernels that put several rows into a wave: every
+    number of chunks from 1 to 64, row counts that leave the last wave part empty, fold mapping and shared
+    gates / tokens, both forms, non-zero initial state and first_prop_grad, the initial-state gradient;
+    against the oracle, and against the one-row-per-wave kernels (asked for by flag) to rounding."""
+    E = 4 if dtype == torch.float32 else 8
+    shapes = [(37, 1, 1), (2, 3, 5), (1, 4, 33), (130, 1, 1)]
+    n = 0
+    for chunks in range(1, 65):
+        L = chunks * E
+        B, M, D = shapes[chunks % len(shapes)]
+        for plain in ((False, True) if chunks % 5 == 0 else (chunks % 2 == 1,)):
+            gen = torch.Generator().manual_seed(1000 + chunks)
+            g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+            x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+            G = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+            h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+            fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+            out = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+            dx, dg, dh0 = torch.empty_like(out), torch.empty_like(out), torch.empty_like(h0)
+            scan.fm_scan_forward(g, x, h0, out, plain=plain)
+            scan.fm_scan_backward(g, G, fpg, dx, out, x, dg, initial_state=h0, initial_state_grad=dh0, plain=plain)
+            tag = f"{(B, M, D, L)} {dtype} plain={plain}"
+            check(tag + " states", out, C.forward_f64(g, x, h0, plain), TOL[dtype])
+            tg, gg, delta = O.backward_per_row(g, G, out, x, fpg, h0, plain)
+            check(tag + " token grad", dx, tg, TOL[dtype])
+            check(tag + " gate grad", dg, gg, TOL[dtype])
+            check(tag + " initial state grad", dh0, O.to_f64(g)[:, :, 0][:, :, None] * delta[..., 0], TOL[dtype])
+            # the general kernels on the same problem
+            out1 = torch.empty_like(out)
+            dx1, dg1, dh1 = torch.empty_like(out), torch.empty_like(out), torch.empty_like(h0)
+            scan.fm_scan_forward(g, x, h0, out1, plain=plain, waves_per_row=1)
+            scan.fm_scan_backward(g, G, fpg, dx1, out, x, dg1, initial_state=h0, initial_state_grad=dh1,
+                                  plain=plain, waves_per_row=1)
+            for name, a, b in (("states", out, out1), ("token grad", dx, dx1), ("gate grad", dg, dg1),
+                               ("initial state grad", dh0, dh1)):
+                check(tag + f" {name} vs a row per wave", a, b.double().cpu().numpy(), 2 * TOL[dtype])
+            # no initial state given: the reference's first_prop_grad stands in for it in the gate gradient
+            dx2, dg2 = torch.empty_like(out), torch.empty_like(out)
+            scan.fm_scan_backward(g, G, fpg, dx2, out, x, dg2, plain=plain)
+            tg2, gg2 = C.backward_f64(g, G, out, x, fpg, None, plain)
+            check(tag + " token grad (reference call)", dx2, tg2, TOL[dtype])
+            check(tag + " gate grad (reference call)", dg2, gg2, TOL[dtype])
+            n += 1
+    assert n == 64 + 12
+
+
+def test_short_rows_do_not_see_their_neighbours(scan):
+    """Several rows share a wave, and the wave scan runs across all of its lanes: a row's results must be
+    the same bits wherever it sits and whatever its neighbours hold, NaN and infinity included."""
+    dt = torch.bfloat16
+    for L in (8, 24, 64, 136, 256, 392, 512):
+        rows = 203
+        gen = gpu_gen(L)
+        g = torch.rand(rows, 1, L, device=DEV, generator=gen).to(dt)
+        x = torch.randn(rows, 1, L, device=DEV, generator=gen).to(dt)
+        G = torch.randn(rows, 1, 1, L, device=DEV, generator=gen).to(dt)
+        a = run_fwd_bwd(scan, g, x, G)
+        perm = torch.randperm(rows, device=DEV, generator=gen)
+        b = run_fwd_bwd(scan, g[perm].contiguous(), x[perm].contiguous(), G[perm].contiguous())
+        for ta, tb in zip(a, b):
+            assert torch.equal(ta[perm], tb), L
+        # every third row poisoned
+        bad = torch.arange(rows, device=DEV) % 3 == 1
+        g2, x2, G2 = g.clone(), x.clone(), G.clone()
+        x2[bad] = float("nan")
+        g2[bad] = float("inf")
+        G2[bad] = float("-inf")
+        c = run_fwd_bwd(scan, g2, x2, G2)
+        for ta, tc in zip(a, c):
+            assert torch.equal(ta[~bad], tc[~bad]), L
+            assert not torch.isfinite(tc[bad].float()).all()
+
+
 def test_segment_requests_without_room_fail_loudly(scan):
     g = torch.rand(2, 1, 65536, device=DEV)
     x = torch.rand(2, 1, 65536, device=DEV)
