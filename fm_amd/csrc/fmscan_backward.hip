@@ -87,13 +87,13 @@ int fmscan_backward(const void* gates, const void* out_grad, const void* first_p
         with_dtype(dtype, [&](auto tt) {
             using T = typename decltype(tt)::type;
             with_bool(pb.plain, [&](auto pt) {
-                with_bool(fold, [&](auto ft) {
-                    fmscan::scan_backward_packed_kernel<T, decltype(pt)::value, decltype(ft)::value>
+                with_bool(vec, [&](auto vt) { with_bool(fold, [&](auto ft) {
+                    fmscan::scan_backward_packed_kernel<T, decltype(pt)::value, decltype(vt)::value, decltype(ft)::value>
                         <<<packed_blocks(pb, lanes_log2), 256, 0, (hipStream_t)stream>>>(
                             (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad_out,
                             (const T*)cached_output, (const T*)input_tokens, (T*)gate_grad_out, (const T*)h_init,
                             (T*)initial_state_grad, pb.rows, (int32_t)pb.M, (int32_t)pb.D, (int32_t)pb.L, lanes_log2);
-                });
+                }); });
             });
         });
         return launched("backward");

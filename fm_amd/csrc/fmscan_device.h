@@ -51,7 +51,12 @@ __device__ __forceinline__ void wait_for_loads() { __builtin_amdgcn_s_waitcnt(0x
 // fm/scan/fm_scan.cuh:14-40).
 template <typename T> struct Elem;
 
+// 16 bytes at the alignment of one element: the GPU takes such an access as one instruction
+typedef u32x4 u32x4_at4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_at2 __attribute__((aligned(2)));
+
 template <> struct Elem<float> {
+    using LooseVec = u32x4_at4;
     static constexpr int E = 4;
     static constexpr uint32_t kOnes = 0x3f800000u;  // 1.0f
     static __device__ __forceinline__ void unpack(u32x4 r, float (&f)[4]) {
@@ -65,6 +70,7 @@ template <> struct Elem<float> {
 };
 
 template <> struct Elem<__bf16> {
+    using LooseVec = u32x4_at2;
     static constexpr int E = 8;
     static constexpr uint32_t kOnes = 0x3f803f80u;  // two bf16 1.0
     static __device__ __forceinline__ void unpack(u32x4 r, float (&f)[8]) {
@@ -88,6 +94,7 @@ template <> struct Elem<__bf16> {
 };
 
 template <> struct Elem<_Float16> {
+    using LooseVec = u32x4_at2;
     static constexpr int E = 8;
     static constexpr uint32_t kOnes = 0x3c003c00u;  // two fp16 1.0
     static __device__ __forceinline__ void unpack(u32x4 r, float (&f)[8]) {
@@ -140,7 +147,10 @@ __device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t
         const u32x4 v = load16<T, ONCE>(row + (inside ? t0 : L - E));
         r = inside ? v : r;
     } else {
-        if (t0 < L) {
+        if (t0 + E <= L) {  // a whole chunk: one access at the alignment of an element
+            if constexpr (ONCE) r = __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::LooseVec*>(row + t0));
+            else r = *reinterpret_cast<const typename Elem<T>::LooseVec*>(row + t0);
+        } else if (t0 < L) {  // the ragged end of a row
             if constexpr (sizeof(T) == 4) {
                 const uint32_t* p = reinterpret_cast<const uint32_t*>(row);
 #pragma unroll
@@ -173,7 +183,9 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ row, int64_t t0, int
     if constexpr (VEC) {
         __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(row + t0));
     } else {
-        if constexpr (sizeof(T) == 4) {
+        if (t0 + E <= L) {
+            __builtin_nontemporal_store(r, reinterpret_cast<typename Elem<T>::LooseVec*>(row + t0));
+        } else if constexpr (sizeof(T) == 4) {
             uint32_t* p = reinterpret_cast<uint32_t*>(row);
 #pragma unroll
             for (int i = 0; i < E; ++i)

@@ -97,12 +97,12 @@ int forward(const char* who, const void* gates, const void* tokens, const void* 
         with_dtype(dtype, [&](auto tt) {
             using T = typename decltype(tt)::type;
             with_bool(pb.plain, [&](auto pt) {
-                with_bool(fold, [&](auto ft) {
-                    fmscan::scan_forward_packed_kernel<T, decltype(pt)::value, decltype(ft)::value>
+                with_bool(vec, [&](auto vt) { with_bool(fold, [&](auto ft) {
+                    fmscan::scan_forward_packed_kernel<T, decltype(pt)::value, decltype(vt)::value, decltype(ft)::value>
                         <<<packed_blocks(pb, lanes_log2), 256, 0, (hipStream_t)stream>>>(
                             (const T*)gates, (const T*)tokens, (const T*)initial_state, (T*)out, pb.rows,
                             (int32_t)pb.M, (int32_t)pb.D, (int32_t)pb.L, lanes_log2);
-                });
+                }); });
             });
         });
         return launched("forward");

@@ -255,13 +255,14 @@ inline int settle(const Problem& pb, bool backward, const void* workspace, size_
     return 0;
 }
 
-// Short rows of whole 16-byte vectors (at most 64 of them, 1 KiB) go to the kernels that put several
+// Short rows (at most 64 chunks of 16 bytes, 1 KiB) go to the kernels that put several
 // rows into a wave (fmscan_packed.h), unless the caller asks for a kernel variant by flag: measured on
 // 2^27 elements of bfloat16 with M = D = 1, fraction of 8 TB/s forward (3 streams) / backward (6 streams),
 // one row per wave -> packed: L = 32: 0.07 / 0.06 -> 0.82 / 0.75; 64: 0.13 / 0.11 -> 0.77 / 0.72;
 // 128: 0.24 / 0.22 -> 0.78 / 0.73; 256: 0.43 / 0.41 -> 0.81 / 0.76; 512: 0.73 / 0.70 -> 0.82 / 0.77.
 inline bool packs_rows(const Problem& pb, bool vec, bool backward) {
-    if (!vec || pb.L * pb.esize > 1024 || pb.waves || pb.blocks_per_cu || pb.depth || pb.segments > 1) return false;
+    (void)vec;  // rows that are not whole aligned vectors are packed too
+    if (pb.L * pb.esize > 1024 || pb.waves || pb.blocks_per_cu || pb.depth || pb.segments > 1) return false;
     // The packed backward kernel reads the saved states, which the general one makes again from gates and
     // tokens that the caches hold when rows share them: with 4-byte elements and rows of more than 32 chunks
     // the general kernel is then as fast or faster (ms, (128,32,128,256) float32: 0.349 against 0.380).
@@ -270,7 +271,7 @@ inline bool packs_rows(const Problem& pb, bool vec, bool backward) {
 }
 // log2 of the lanes a row takes: the power of two at or above its number of 16-byte chunks
 inline int32_t packed_lanes_log2(const Problem& pb) {
-    const int64_t chunks = pb.L * pb.esize / 16;
+    const int64_t chunks = (pb.L * pb.esize + 15) / 16;
     int32_t k = 0;
     while ((1 << k) < chunks) ++k;
     return k;

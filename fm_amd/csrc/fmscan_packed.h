@@ -11,8 +11,9 @@
 // neighbours' values (NaN and infinity included) and is the same bit for bit wherever the row sits in the
 // wave.
 //
-// Rows must be whole 16-byte vectors (L * sizeof(T) a multiple of 16, pointers aligned). One tile per row:
-// no loop, no LDS, no workspace. Arithmetic as in the general kernels (float32, one fma per step); the
+// Rows of whole 16-byte vectors at aligned addresses move as such (VEC); any other row of up to 64 chunks
+// with accesses at the alignment of an element and a ragged last chunk. One tile per row: no loop, no LDS,
+// no workspace. Arithmetic as in the general kernels (float32, one fma per step); the
 // backward kernel reads the saved states (a fourth stream) instead of making them again.
 #pragma once
 
@@ -39,6 +40,15 @@ __device__ __forceinline__ void group_scan_inclusive(float& a, float& b, int p) 
     segmented_level<0x118, 0xf>(a, b, p >= 8);   // row_shr:8
     segmented_level<0x142, 0xa>(a, b, p >= 16);  // row_bcast:15 into the 16-lane rows 1 and 3
     segmented_level<0x143, 0xc>(a, b, p >= 32);  // row_bcast:31 into the 16-lane rows 2 and 3
+}
+
+// The chunk at position t0 of a row. VEC: rows are whole 16-byte vectors at 16-byte aligned addresses.
+// Otherwise a row starts wherever an element may, and its last chunk may be ragged: whole chunks move as
+// one access at the alignment of an element, the ragged one element by element, positions past the end as `fill`.
+template <typename T, bool VEC, bool ONCE>
+__device__ __forceinline__ u32x4 packed_load(const T* __restrict__ row, int32_t t0, int32_t L, uint32_t fill) {
+    if constexpr (VEC) return load16<T, ONCE>(row + t0);
+    else return load_chunk<T, false, ONCE>(row, t0, L, fill);
 }
 
 // Where a lane works: its row, its place in the group, the chunk it owns.
@@ -70,18 +80,18 @@ __device__ __forceinline__ PackedLane locate_packed(int64_t rows, int32_t M, int
 }
 
 // h_t = g_t h_{t-1} + u_t,  u_t = (1 - g_t) x_t  (PLAIN: u_t = x_t); see scan_forward_kernel.
-template <typename T, bool PLAIN, bool FOLD>
+template <typename T, bool PLAIN, bool VEC, bool FOLD>
 __global__ __launch_bounds__(256) void scan_forward_packed_kernel(
     const T* __restrict__ gates, const T* __restrict__ tokens, const T* __restrict__ h0, T* __restrict__ out,
     int64_t rows, int32_t M, int32_t D, int32_t L, int32_t lpr_log2) {
     constexpr int E = Elem<T>::E;
-    const int32_t CL = L / E;  // chunks per row
+    const int32_t CL = (L + E - 1) / E;  // chunks per row (VEC: all whole)
     if ((((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) << (6 - lpr_log2)) >= rows) return;  // whole waves
     const PackedLane q = locate_packed<FOLD>(rows, M, D, lpr_log2);
     const bool active = q.has_row && q.p < CL;
     const int32_t t0 = (q.p < CL ? q.p : CL - 1) * E;
-    u32x4 gq = load16<T, FOLD>(gates + q.gate_row * L + t0);
-    u32x4 xq = load16<T, FOLD>(tokens + q.token_row * L + t0);
+    u32x4 gq = packed_load<T, VEC, FOLD>(gates + q.gate_row * L, t0, L, Elem<T>::kOnes);
+    u32x4 xq = packed_load<T, VEC, FOLD>(tokens + q.token_row * L, t0, L, 0u);
     const float hin = (h0 && q.p == 0) ? Elem<T>::widen(h0[q.row]) : 0.0f;
     if (!active) {  // identity steps
         gq = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
@@ -110,30 +120,30 @@ __global__ __launch_bounds__(256) void scan_forward_packed_kernel(
         h = __builtin_fmaf(g[i], h, u[i]);
         o[i] = h;
     }
-    if (active) store16<T>(out + q.row * L + t0, Elem<T>::pack(o));
+    if (active) store_chunk<T, VEC>(out + q.row * L, t0, L, Elem<T>::pack(o));
 }
 
 // delta_t = G_t + g_{t+1} delta_{t+1}; token_grad_t = (1 - g_t) delta_t, gate_grad_t = (h_{t-1} - x_t) delta_t
 // (PLAIN: delta_t, h_{t-1} delta_t); see scan_backward_kernel. The lanes of a group take the row's chunks
 // from the last to the first, so the suffix scan in memory order is a prefix scan in lane order.
-template <typename T, bool PLAIN, bool FOLD>
+template <typename T, bool PLAIN, bool VEC, bool FOLD>
 __global__ __launch_bounds__(256) void scan_backward_packed_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad, const T* __restrict__ h_saved, const T* __restrict__ tokens,
     T* __restrict__ gate_grad, const T* __restrict__ h0, T* __restrict__ h0_grad, int64_t rows, int32_t M,
     int32_t D, int32_t L, int32_t lpr_log2) {
     constexpr int E = Elem<T>::E;
-    const int32_t CL = L / E;
+    const int32_t CL = (L + E - 1) / E;
     if ((((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) << (6 - lpr_log2)) >= rows) return;
     const PackedLane q = locate_packed<FOLD>(rows, M, D, lpr_log2);
     const bool active = q.has_row && q.p < CL;
     const int32_t c = q.p < CL ? CL - 1 - q.p : 0;  // the chunk of this lane, counted from the row's start
     const int32_t t0 = c * E;
-    u32x4 gq = load16<T, FOLD>(gates + q.gate_row * L + t0);
-    u32x4 Gq = load16<T, true>(out_grad + q.row * L + t0);
-    const u32x4 hq = load16<T, true>(h_saved + q.row * L + t0);
+    u32x4 gq = packed_load<T, VEC, FOLD>(gates + q.gate_row * L, t0, L, Elem<T>::kOnes);
+    u32x4 Gq = packed_load<T, VEC, true>(out_grad + q.row * L, t0, L, 0u);
+    const u32x4 hq = packed_load<T, VEC, true>(h_saved + q.row * L, t0, L, 0u);
     u32x4 xq = u32x4{0u, 0u, 0u, 0u};
-    if constexpr (!PLAIN) xq = load16<T, FOLD>(tokens + q.token_row * L + t0);
+    if constexpr (!PLAIN) xq = packed_load<T, VEC, FOLD>(tokens + q.token_row * L, t0, L, 0u);
     const float cinit = (first_prop_grad && q.p == 0) ? Elem<T>::widen(first_prop_grad[q.row]) : 0.0f;
     const float hinit = (h0 && c == 0) ? Elem<T>::widen(h0[q.row]) : 0.0f;
     if (!active) {
@@ -187,8 +197,8 @@ __global__ __launch_bounds__(256) void scan_backward_packed_kernel(
         }
     }
     if (active) {
-        store16<T>(token_grad + q.row * L + t0, Elem<T>::pack(dx));
-        store16<T>(gate_grad + q.row * L + t0, Elem<T>::pack(dg));
+        store_chunk<T, VEC>(token_grad + q.row * L, t0, L, Elem<T>::pack(dx));
+        store_chunk<T, VEC>(gate_grad + q.row * L, t0, L, Elem<T>::pack(dg));
     }
 }
 

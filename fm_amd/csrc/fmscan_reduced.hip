@@ -254,11 +254,11 @@ int fmscan_reduced_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, i
 
 int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype) {
     if (B < 1 || M < 2 || D < 2 || L < 1) return 0;
-    // Rows of at most 16 chunks of 16 bytes leave three quarters of this kernel's lanes idle, and
+    // Rows of at most 256 bytes leave three quarters of this kernel's lanes idle, and
     // fmscan_backward puts several such rows into a wave (bf16, ms, against it and the two sums:
     // (512,32,128,64) 0.73 against 0.30, (256,32,128,128) 0.39 against 0.29, (128,32,128,256) 0.21 against 0.28).
     const int64_t row_bytes = L * (dtype == FMSCAN_DTYPE_F32 ? 4 : 2);
-    if (row_bytes <= 256 && row_bytes % 16 == 0) return 0;
+    if (row_bytes <= 256) return 0;
     int64_t split = 0, segments = 0;
     if (fmscan_reduced_plan(B, M, D, L, dtype, &split, &segments) != 0) return 0;
     // Measured against fmscan_backward followed by the two sums (bf16, ms): 512 blocks after split and cut

@@ -263,8 +263,8 @@ int fmscan_backward_layer(const void* gates, const void* states_n,
 int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D);
 /* 1 when fmscan_backward_reduced (split and cut as fmscan_reduced_plan below says) is expected to be at
  * least as fast as fmscan_backward followed by the two sums, 0 when even that leaves too few blocks
- * (very few batch elements with few slots and channels, rows too short to cut) and for rows of whole
- * 16-byte vectors up to 256 bytes, where fmscan_backward puts several rows into a wave and this kernel
+ * (very few batch elements with few slots and channels, rows too short to cut) and for rows of up to
+ * 256 bytes, where fmscan_backward puts several rows into a wave and this kernel
  * leaves most lanes idle. */
 int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
 int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,

@@ -156,9 +156,9 @@ def test_rejected_arguments(lib):
     pays = lib.fmscan_reduced_pays
     assert pays(32, 32, 128, 2048, 2) == 1 and pays(2, 32, 128, 16384, 2) == 1
     assert pays(1, 16, 64, 65536, 2) == 1 and pays(1, 16, 64, 2048, 2) == 0 and pays(4, 1, 64, 2048, 2) == 0
-    # rows of up to 256 bytes of whole 16-byte vectors: fmscan_backward packs several into a wave
+    # rows of up to 256 bytes: fmscan_backward packs several into a wave
     assert pays(512, 32, 128, 64, 2) == 0 and pays(256, 32, 128, 128, 2) == 0 and pays(128, 32, 128, 256, 2) == 1
-    assert pays(256, 32, 128, 64, 0) == 0 and pays(256, 32, 128, 68, 0) == 1 and pays(256, 32, 128, 100, 2) == 1
+    assert pays(256, 32, 128, 64, 0) == 0 and pays(256, 32, 128, 68, 0) == 1 and pays(256, 32, 128, 100, 2) == 0
     assert lib.fmscan_forward_normed_pays(32, 32, 128) == 1 and lib.fmscan_forward_normed_pays(2, 32, 128) == 1
     assert lib.fmscan_forward_normed_pays(1, 32, 128) == 0 and lib.fmscan_forward_normed_pays(1, 8, 2048) == 1
     # scan and norm in one kernel with the sequence cut: no cut without a workspace, no more segments than tiles

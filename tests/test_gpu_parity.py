@@ -568,14 +568,17 @@ def test_few_long_rows_are_cut_into_segments(scan, dtype, plain):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_short_rows_several_per_wave(scan, dtype):
     """Rows of at most 64 chunks of 16 bytes take the kernels that put several rows into a wave: every
-    number of chunks from 1 to 64, row counts that leave the last wave part empty, fold mapping and shared
+    number of chunks from 1 to 64, lengths that are not whole chunks, row counts that leave the last wave part empty, fold mapping and shared
     gates / tokens, both forms, non-zero initial state and first_prop_grad, the initial-state gradient;
     against the oracle, and against the one-row-per-wave kernels (asked for by flag) to rounding."""
     E = 4 if dtype == torch.float32 else 8
     shapes = [(37, 1, 1), (2, 3, 5), (1, 4, 33), (130, 1, 1)]
     n = 0
-    for chunks in range(1, 65):
-        L = chunks * E
+    # whole chunks, then lengths that leave the last chunk ragged and the rows at odd addresses
+    lengths = [(chunks, chunks * E) for chunks in range(1, 65)]
+    lengths += [(k, L) for k, L in enumerate((1, 2, 3, 5, 7, 9, 13, 31, 33, 50, 100, 101, 127, 250, 255, 500, 511))
+                if L * (16 // E) <= 1024]
+    for chunks, L in lengths:
         B, M, D = shapes[chunks % len(shapes)]
         for plain in ((False, True) if chunks % 5 == 0 else (chunks % 2 == 1,)):
             gen = torch.Generator().manual_seed(1000 + chunks)
@@ -610,7 +613,7 @@ def test_short_rows_several_per_wave(scan, dtype):
             check(tag + " token grad (reference call)", dx2, tg2, TOL[dtype])
             check(tag + " gate grad (reference call)", dg2, gg2, TOL[dtype])
             n += 1
-    assert n == 64 + 12
+    assert n == (64 + 12) + (15 + 3 if dtype == torch.float32 else 17 + 4)
 
 
 def test_short_rows_do_not_see_their_neighbours(scan):
