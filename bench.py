@@ -610,6 +610,78 @@ def layer_cpu_baseline(torch, alpha, us, osc, inp, w_out, batch=16):
 GRID_ROWS = (256, 2048, 16384, 131072)
 GRID_L = (1024, 4096, 16384, 65536)
 GRID_NATIVE = ((32, 32, 64, 2048), (8, 16, 64, 16384), (4, 32, 1024, 4096), (1, 32, 1024, 8192))  # (B, M, D, L)
+# (B, M, D, L, dtype): rows of at most 1 KiB, which the scan calls put several to a wave; fold mapping
+# (M = D = 1) of 2^27 elements at every length, lengths that are not whole 16-byte vectors, and
+# Factorization-Memory shapes of the benchmark's slots and channels with short sequences
+SHORT_ROW_SHAPES = [
+    (4194304, 1, 1, 32, "bfloat16"), (2097152, 1, 1, 64, "bfloat16"), (1048576, 1, 1, 128, "bfloat16"),
+    (524288, 1, 1, 256, "bfloat16"), (262144, 1, 1, 512, "bfloat16"), (1048576, 1, 1, 64, "float32"),
+    (524288, 1, 1, 256, "float32"), (1342177, 1, 1, 100, "bfloat16"), (262144, 1, 1, 500, "bfloat16"),
+    (1048576, 1, 1, 33, "float32"),
+    (512, 32, 128, 64, "bfloat16"), (256, 32, 128, 128, "bfloat16"), (128, 32, 128, 256, "bfloat16"),
+    (64, 32, 128, 512, "bfloat16"), (128, 32, 128, 128, "float32"),
+]
+
+
+def run_short_rows(torch, args) -> int:
+    """`--short-rows`: fmscan_forward and fmscan_backward on SHORT_ROW_SHAPES, the library's choice (several
+    rows to a wave) against the general kernels asked for by flag (a row to a wave). A table on stderr, one
+    JSON line on stdout. GB/s counts streams of the size of the (B,M,D,L) tensor: 3 forward and 6 backward in the
+    fold mapping (the metric's model), 1 and 4 where gates and tokens are shared (states written; two tensors read
+    and two written), for both columns alike."""
+    import fm.scan.fm_scan as S
+
+    dev = torch.device("cuda", 0)
+
+    def timed(call, reps):
+        for _ in range(3):
+            call()
+        best = None
+        for _ in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(reps):
+                call()
+            b.record()
+            b.synchronize()
+            ms = a.elapsed_time(b) / reps
+            best = ms if best is None else min(best, ms)
+        return best
+
+    rows = []
+    for (B, M, D, L, dtn) in SHORT_ROW_SHAPES:
+        dt = getattr(torch, dtn)
+        gen = torch.Generator(device=dev).manual_seed(1)
+        g = (0.5 + 0.5 * torch.rand(B, M, L, device=dev, generator=gen)).to(dt)
+        x = torch.randn(B, D, L, device=dev, generator=gen).to(dt)
+        G = torch.randn(B, M, D, L, device=dev, generator=gen).to(dt)
+        z = torch.zeros(B, M, D, dtype=dt, device=dev)
+        out = torch.empty(B, M, D, L, dtype=dt, device=dev)
+        dx, dg = torch.empty_like(out), torch.empty_like(out)
+        nbytes = B * M * D * L * g.element_size()
+        r = {"shape": [B, M, D, L], "storage_dtype": STORAGE[dtn]}
+        for name, kw in (("packed", {}), ("row_per_wave", {"waves_per_row": 1})):
+            f = timed(lambda: S.fm_scan_forward(g, x, z, out, **kw), 20)
+            b = timed(lambda: S.fm_scan_backward(g, G, z, dx, out, x, dg, **kw), 20)
+            fold = M == 1 and D == 1
+            r[name] = {"fwd_ms": round(f, 4), "bwd_ms": round(b, 4),
+                       "fwd_GBps": round((3 if fold else 1) * nbytes / f / 1e6, 1),
+                       "bwd_GBps": round((6 if fold else 4) * nbytes / b / 1e6, 1)}
+        rows.append(r)
+        del g, x, G, out, dx, dg
+        torch.cuda.empty_cache()
+    print(f"{'(B, M, D, L)':>26s} {'dtype':>5s} | {'fwd ms':>8s} {'GB/s':>7s} {'bwd ms':>8s} {'GB/s':>7s} | a row per wave: "
+          f"{'fwd ms':>8s} {'GB/s':>7s} {'bwd ms':>8s} {'GB/s':>7s}", file=sys.stderr)
+    for r in rows:
+        p, o = r["packed"], r["row_per_wave"]
+        print(f"{str(tuple(r['shape'])):>26s} {r['storage_dtype']:>5s} | {p['fwd_ms']:8.4f} {p['fwd_GBps']:7.0f} "
+              f"{p['bwd_ms']:8.4f} {p['bwd_GBps']:7.0f} |                 {o['fwd_ms']:8.4f} {o['fwd_GBps']:7.0f} "
+              f"{o['bwd_ms']:8.4f} {o['bwd_GBps']:7.0f}", file=sys.stderr)
+    print(json.dumps({"metric": "fmscan_forward / fmscan_backward on rows of at most 1 KiB, GB/s",
+                      "unit": "GB/s", "dtype": "f32", "data": "synthetic", "shapes": rows}), flush=True)
+    return 0
+
+
 GRID_MAX_ELEMENTS = 1 << 31  # per tensor; larger cells of the grid are left out
 GRID_DEPTHS = (2, 4)
 
@@ -722,6 +794,9 @@ def main() -> int:
     ap.add_argument("--layer-shapes", action="store_true",
                     help="the layer's step over shapes with fewer batch elements and longer rows than the "
                          "benchmark's, with the routes the library takes for each; a table on stderr")
+    ap.add_argument("--short-rows", action="store_true",
+                    help="the two scan calls on rows of at most 1 KiB (several rows to a wave) against the "
+                         "general kernels asked for by flag; a table on stderr")
     ap.add_argument("--graph", action="store_true",
                     help="also capture one step in a HIP graph and time its replays (what a launch-bound "
                          "caller, e.g. the small configuration 1, gets without the per-call Python cost)")
@@ -746,6 +821,8 @@ def main() -> int:
         return run_grid(torch, args)
     if args.layer_shapes:
         return run_layer_shapes(torch, args)
+    if args.short_rows:
+        return run_short_rows(torch, args)
     if args.workload == "layer":
         return run_layer(torch, args)
     B, Cn, T, dtn = WORKLOADS[args.workload]

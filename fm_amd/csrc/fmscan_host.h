@@ -263,10 +263,10 @@ inline int settle(const Problem& pb, bool backward, const void* workspace, size_
 inline bool packs_rows(const Problem& pb, bool vec, bool backward) {
     (void)vec;  // rows that are not whole aligned vectors are packed too
     if (pb.L * pb.esize > 1024 || pb.waves || pb.blocks_per_cu || pb.depth || pb.segments > 1) return false;
-    // The packed backward kernel reads the saved states, which the general one makes again from gates and
-    // tokens that the caches hold when rows share them: with 4-byte elements and rows of more than 32 chunks
-    // the general kernel is then as fast or faster (ms, (128,32,128,256) float32: 0.349 against 0.380).
-    if (backward && pb.esize == 4 && pb.L * pb.esize > 512 && (pb.M > 1 || pb.D > 1)) return false;
+    // The packed backward kernel reads the saved states, which the general one makes again from the gates
+    // and tokens: with 4-byte elements and rows of more than 32 chunks the general kernel is as fast or
+    // faster (ms, float32: (128,32,128,256) 0.349 against 0.380, (524288,1,1,256) 0.516 against 0.541).
+    if (backward && pb.esize == 4 && pb.L * pb.esize > 512) return false;
     return true;
 }
 // log2 of the lanes a row takes: the power of two at or above its number of 16-byte chunks
