@@ -66,6 +66,10 @@ extern "C" {
 #define FMSCAN_FLAG_SEGMENTS_SHIFT 20 /* bits 20..27: segments a row is cut into (2..255, needs the
                                          workspace); 1 = never cut; 0 = library's choice */
 #define FMSCAN_FLAG_SEGMENTS_MASK 0xFF00000u
+/* With none of the four choices above made by the caller, fmscan_forward, fmscan_forward_static and
+ * fmscan_backward put rows of at most 1 KiB several to a wave (a kernel of its own, a segmented wave scan);
+ * any of them set selects the general kernels, which give a wave one row at a time. Results agree to
+ * float32 rounding. */
 
 /* error codes (negative returns) */
 #define FMSCAN_E_NULL      (-1) /* a required pointer is NULL */
