@@ -3,6 +3,8 @@
 // operator. Everything here is written for CDNA4 wave64 directly.
 #pragma once
 
+#include <type_traits>
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -127,10 +129,15 @@ template <> struct Elem<_Float16> {
 // no other row reads again: it is loaded with the non-temporal hint so that it does
 // not displace anything from the caches on its way through (measured: worth about a
 // tenth of the bandwidth on 1 GiB tensors). Stores always carry the hint.
-template <typename T, bool ONCE>
+// ALIGNED = false: p is aligned as an element is, not to 16 bytes (still one access).
+template <typename T, bool ALIGNED> struct Vec16 { using type = u32x4; };
+template <typename T> struct Vec16<T, false> { using type = typename Elem<T>::LooseVec; };
+
+template <typename T, bool ONCE, bool ALIGNED = true>
 __device__ __forceinline__ u32x4 load16(const T* __restrict__ p) {
-    if constexpr (ONCE) return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-    else return *reinterpret_cast<const u32x4*>(p);
+    using V = typename Vec16<T, ALIGNED>::type;
+    if constexpr (ONCE) return __builtin_nontemporal_load(reinterpret_cast<const V*>(p));
+    else return *reinterpret_cast<const V*>(p);
 }
 
 // The VEC form never branches around its load: a chunk outside [0, L) reads the last
@@ -148,8 +155,7 @@ __device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t
         r = inside ? v : r;
     } else {
         if (t0 + E <= L) {  // a whole chunk: one access at the alignment of an element
-            if constexpr (ONCE) r = __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::LooseVec*>(row + t0));
-            else r = *reinterpret_cast<const typename Elem<T>::LooseVec*>(row + t0);
+            r = load16<T, ONCE, false>(row + t0);
         } else if (t0 < L) {  // the ragged end of a row
             if constexpr (sizeof(T) == 4) {
                 const uint32_t* p = reinterpret_cast<const uint32_t*>(row);
@@ -171,9 +177,10 @@ __device__ __forceinline__ u32x4 load_chunk(const T* __restrict__ row, int64_t t
     return r;
 }
 
-template <typename T>
+template <typename T, bool ALIGNED = true>
 __device__ __forceinline__ void store16(T* __restrict__ p, u32x4 r) {
-    __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(p));
+    using V = typename Vec16<T, ALIGNED>::type;
+    __builtin_nontemporal_store(r, reinterpret_cast<V*>(p));
 }
 
 template <typename T, bool VEC>
@@ -184,7 +191,7 @@ __device__ __forceinline__ void store_chunk(T* __restrict__ row, int64_t t0, int
         __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(row + t0));
     } else {
         if (t0 + E <= L) {
-            __builtin_nontemporal_store(r, reinterpret_cast<typename Elem<T>::LooseVec*>(row + t0));
+            store16<T, false>(row + t0, r);
         } else if constexpr (sizeof(T) == 4) {
             uint32_t* p = reinterpret_cast<uint32_t*>(row);
 #pragma unroll
