@@ -124,8 +124,9 @@ template <> struct Elem<_Float16> {
 // Chunk = the E consecutive elements one lane owns in a tile, starting at
 // sequence position t0 of a row. VEC: the row base and L*sizeof(T) are 16-byte
 // multiples, so a chunk is either wholly inside [0, L) or wholly outside and
-// moves as one 16-byte access. !VEC: element accesses with a bound check each;
-// `fill` is the 32-bit pattern for positions at or beyond L. ONCE marks data that
+// moves as one 16-byte access. !VEC: a chunk wholly inside moves as one access at the
+// alignment of an element, the ragged one at the end of a row as element accesses with a
+// bound check each; `fill` is the 32-bit pattern for positions at or beyond L. ONCE marks data that
 // no other row reads again: it is loaded with the non-temporal hint so that it does
 // not displace anything from the caches on its way through (measured: worth about a
 // tenth of the bandwidth on 1 GiB tensors). Stores always carry the hint.

@@ -313,7 +313,7 @@ void dispatch(int dtype, const Tuning& t, bool plain, bool vec, bool fold, F&& f
                 if (plain) f(tt, wt, rt, dt, BoolTag<true>{}, vt, ft);
                 else f(tt, wt, rt, dt, BoolTag<false>{}, vt, ft);
             };
-            if (!vec) {  // element access: the slow path gets one variant
+            if (!vec) {  // rows off the 16-byte grid: the slower path gets one variant
                 with_depth(IntTag<2>{}, BoolTag<false>{}, BoolTag<false>{});
                 return;
             }

@@ -109,8 +109,9 @@ size_t fmscan_workspace_bytes(int64_t B, int64_t M, int64_t D, int64_t L, int dt
  *   initial_state  (B, M, D)     in, may be NULL (= zeros)
  *   out            (B, M, D, L)  out; must not overlap gates or tokens
  * Any L >= 1 is accepted (the reference accepts powers of two in 32..131072,
- * fm_scan.cuh:275-329); 16-byte vector access is used when the pointers and
- * L * sizeof(element) are multiples of 16, element access otherwise.
+ * fm_scan.cuh:275-329); aligned 16-byte vector access is used when the pointers and
+ * L * sizeof(element) are multiples of 16; otherwise 16-byte accesses at the alignment of an element,
+ * and element access for the ragged end of a row (about 0.6 of the aligned rate).
  */
 int fmscan_forward(const void* gates, const void* tokens, const void* initial_state,
                    void* out,
