@@ -626,7 +626,8 @@ SHORT_ROW_SHAPES = [
 def run_short_rows(torch, args) -> int:
     """`--short-rows`: fmscan_forward and fmscan_backward on SHORT_ROW_SHAPES, the library's choice (several
     rows to a wave) against the general kernels asked for by flag (a row to a wave). A table on stderr, one
-    JSON line on stdout. GB/s counts streams of the size of the (B,M,D,L) tensor: 3 forward and 6 backward in the
+    JSON line on stdout; for the shapes with shared gates and tokens also FM_Scan.backward's two routes.
+    GB/s counts streams of the size of the (B,M,D,L) tensor: 3 forward and 6 backward in the
     fold mapping (the metric's model), 1 and 4 where gates and tokens are shared (states written; two tensors read
     and two written), for both columns alike."""
     import fm.scan.fm_scan as S
@@ -667,6 +668,16 @@ def run_short_rows(torch, args) -> int:
             r[name] = {"fwd_ms": round(f, 4), "bwd_ms": round(b, 4),
                        "fwd_GBps": round((3 if fold else 1) * nbytes / f / 1e6, 1),
                        "bwd_GBps": round((6 if fold else 4) * nbytes / b / 1e6, 1)}
+        if M > 1 and D > 1:  # FM_Scan.backward's routes: the sums inside the kernel, or two tensors and two sums
+            code = {"float32": 0, "float16": 1, "bfloat16": 2}[dtn]
+            r["sums_inside"] = ("packed" if S.module.fmscan_reduced_packed_groups(B, M, D, L, code) > 0 else "a row per wave")
+            r["sums_inside_ms"] = round(timed(lambda: S.fm_scan_backward_reduced(g, G, z, out, x), 10), 4)
+
+            def two():
+                S.fm_scan_backward(g, G, z, dx, out, x, dg)
+                return dg.sum(dim=2), dx.sum(dim=1)
+
+            r["two_tensors_and_sums_ms"] = round(timed(two, 10), 4)
         rows.append(r)
         del g, x, G, out, dx, dg
         torch.cuda.empty_cache()
@@ -677,6 +688,12 @@ def run_short_rows(torch, args) -> int:
         print(f"{str(tuple(r['shape'])):>26s} {r['storage_dtype']:>5s} | {p['fwd_ms']:8.4f} {p['fwd_GBps']:7.0f} "
               f"{p['bwd_ms']:8.4f} {p['bwd_GBps']:7.0f} |                 {o['fwd_ms']:8.4f} {o['fwd_GBps']:7.0f} "
               f"{o['bwd_ms']:8.4f} {o['bwd_GBps']:7.0f}", file=sys.stderr)
+    print("\nbackward with the sums over slots and channels (FM_Scan.backward): inside the kernel | "
+          "fmscan_backward, then two torch sums", file=sys.stderr)
+    for r in rows:
+        if "sums_inside_ms" in r:
+            print(f"{str(tuple(r['shape'])):>26s} {r['storage_dtype']:>5s} | {r['sums_inside_ms']:8.4f} ms "
+                  f"({r['sums_inside']}) | {r['two_tensors_and_sums_ms']:8.4f} ms", file=sys.stderr)
     print(json.dumps({"metric": "fmscan_forward / fmscan_backward on rows of at most 1 KiB, GB/s",
                       "unit": "GB/s", "dtype": "f32", "data": "synthetic", "shapes": rows}), flush=True)
     return 0

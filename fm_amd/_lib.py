@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint, c_void_p
 
 from . import build as _build
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 FLAG_PLAIN = 0x1
@@ -95,6 +95,10 @@ def load() -> ctypes.CDLL:
     lib.fmscan_reduced_split.argtypes = [c_int64] * 3
     lib.fmscan_reduced_pays.restype = c_int
     lib.fmscan_reduced_pays.argtypes = [c_int64] * 4 + [c_int]
+    lib.fmscan_reduced_packed_groups.restype = c_int64
+    lib.fmscan_reduced_packed_groups.argtypes = [c_int64] * 4 + [c_int]
+    lib.fmscan_backward_reduced_packed.restype = c_int
+    lib.fmscan_backward_reduced_packed.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     lib.fmscan_backward_reduced_split.restype = c_int
     lib.fmscan_backward_reduced_split.argtypes = ([c_void_p] * 9 + [c_int64] * 6 + [c_void_p, c_size_t]
                                                   + [c_int, c_uint, c_void_p])

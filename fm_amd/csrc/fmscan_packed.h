@@ -202,4 +202,158 @@ __global__ __launch_bounds__(256) void scan_backward_packed_kernel(
     }
 }
 
+// ---- backward with the sums inside, for short rows ---------------------------------------------------
+// What scan_backward_packed_kernel computes, summed as the reference sums it afterwards (fm_scan.py:76-78):
+// the token gradient over the M slots and the gate gradient over the D rows of a slot, in float32. A wave
+// is a batch element b and a tile of 64 >> lpr_log2 consecutive rows d, and walks the M slots: the token
+// gradient of its rows adds up in registers and is stored once; the gate gradient of a slot is added
+// across the wave's groups (rotations inside the 16-lane rows, then the rows change places in a copy: every
+// lane ends with the sum) and the first group stores it as one of G = ceil(D / rows of a tile) float32
+// partial sums, gate_grad_partial (B * M, G, L), which fmscan_sum_groups adds. No LDS, no barrier; the
+// loads of the next slot are in flight while a slot is worked on. Sums are taken in a fixed order.
+// v + (v of the lane 16 or 32 away): the two halves change places in a copy and meet in an add
+template <int AWAY>
+__device__ __forceinline__ float add_across(float v) {
+    uint32_t mine = f2u(v), copy;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(copy) : "v"(mine));  // a copy the compiler cannot identify with `mine`
+    if constexpr (AWAY == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(mine, copy, false, false);
+        return u2f(r[0]) + u2f(r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane16_swap(mine, copy, false, false);
+        return u2f(r[0]) + u2f(r[1]);
+    }
+}
+
+// Every lane's E values summed over the lanes that hold the same chunk in the wave's other groups
+// (groups are 1 << lpr_log2 lanes, at most 16): rotations inside the 16-lane rows, then the two exchanges
+// across them. Every lane ends with the sum.
+template <int E>
+__device__ __forceinline__ void sum_over_groups(float (&v)[E], int32_t lpr_log2) {
+    if (lpr_log2 <= 3) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] += dpp<0x128, 0xf>(v[e], v[e]);  // row_ror:8
+    }
+    if (lpr_log2 <= 2) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] += dpp<0x124, 0xf>(v[e], v[e]);  // row_ror:4
+    }
+    if (lpr_log2 <= 1) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] += dpp<0x122, 0xf>(v[e], v[e]);  // row_ror:2
+    }
+    if (lpr_log2 <= 0) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] += dpp<0x121, 0xf>(v[e], v[e]);  // row_ror:1
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = add_across<32>(add_across<16>(v[e]));
+}
+
+template <typename T, bool PLAIN>
+__global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
+    const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
+    T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved, const T* __restrict__ tokens,
+    float* __restrict__ gate_grad_partial /* (B * M, G, L) */, const T* __restrict__ h0, T* __restrict__ h0_grad,
+    int32_t B, int32_t M, int32_t D, int32_t L, int32_t lpr_log2, int32_t G) {
+    constexpr int E = Elem<T>::E;
+    const int32_t CL = L / E;  // rows are whole 16-byte vectors
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + uniform((int)(threadIdx.x >> 6));
+    if (wave >= (int64_t)B * G) return;  // whole waves
+    const int32_t b = uniform((int)(wave / G));
+    const int32_t tile = uniform((int)(wave - (int64_t)b * G));
+    const int32_t p = lane & ((1 << lpr_log2) - 1);
+    const int32_t group = lane >> lpr_log2;
+    const int32_t d_mine = (tile << (6 - lpr_log2)) + group;
+    const bool active = d_mine < D && p < CL;
+    const int32_t d = d_mine < D ? d_mine : D - 1;            // lanes without a row load the last one and drop it
+    const int32_t c = p < CL ? CL - 1 - p : 0;                // the chunk of this lane, counted from the row's start
+    const int32_t t0 = c * E;
+    const int64_t token_row = (int64_t)b * D + d;
+
+    float x[E];
+    if constexpr (!PLAIN) Elem<T>::unpack(load16<T, false>(tokens + token_row * L + t0), x);
+    float dtok[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) dtok[e] = 0.0f;
+
+    struct In {
+        u32x4 g, G, h;
+        float cinit, hinit;
+    };
+    auto fetch = [&](In& n, int32_t m) {
+        const int64_t gate_row = (int64_t)b * M + m;
+        const int64_t row = gate_row * D + d;
+        n.g = load16<T, false>(gates + gate_row * L + t0);
+        n.G = load16<T, true>(out_grad + row * L + t0);
+        n.h = load16<T, true>(h_saved + row * L + t0);
+        n.cinit = (first_prop_grad && p == 0) ? Elem<T>::widen(first_prop_grad[row]) : 0.0f;
+        n.hinit = (h0 && c == 0) ? Elem<T>::widen(h0[row]) : 0.0f;
+    };
+    In cur, next;
+    fetch(cur, 0);
+    for (int32_t m = 0; m < M; ++m) {
+        fetch(next, m + 1 < M ? m + 1 : m);
+        const int64_t gate_row = (int64_t)b * M + m;
+        u32x4 gq = cur.g, Gq = cur.G;
+        if (!active) {  // identity steps
+            gq = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
+            Gq = u32x4{0u, 0u, 0u, 0u};
+        }
+        float g[E], Gv[E], pr[E], h[E];
+        Elem<T>::unpack(gq, g);
+        Elem<T>::unpack(Gq, Gv);
+        Elem<T>::unpack(cur.h, h);
+#pragma unroll
+        for (int e = 0; e < E; ++e) pr[e] = g[e] * Gv[e];
+        float a = g[E - 1], bb = pr[E - 1];
+#pragma unroll
+        for (int e = E - 2; e >= 0; --e) {
+            bb = __builtin_fmaf(g[e], bb, pr[e]);
+            a *= g[e];
+        }
+        if (p == 0) bb = __builtin_fmaf(a, cur.cinit, bb);  // what arrives at the end of the row
+        group_scan_inclusive(a, bb, p);
+        const float before = dpp<kWaveShr1>(0.0f, bb);
+        float cc = p == 0 ? cur.cinit : before;
+        if (h0_grad && active && c == 0) {  // g_0 * delta_0: the gradient of the state before the row
+            float v[E] = {bb};
+            const u32x4 packed = Elem<T>::pack(v);
+            const int64_t row = gate_row * D + d;
+            if constexpr (sizeof(T) == 4) reinterpret_cast<uint32_t*>(h0_grad)[row] = packed.x;
+            else reinterpret_cast<uint16_t*>(h0_grad)[row] = (uint16_t)(packed.x & 0xffffu);
+        }
+        const float behind = dpp<kWaveShl1>(0.0f, h[E - 1]);
+        float hp[E];
+        hp[0] = c == 0 ? cur.hinit : behind;
+#pragma unroll
+        for (int e = 1; e < E; ++e) hp[e] = h[e - 1];
+        float dg[E];
+#pragma unroll
+        for (int e = E - 1; e >= 0; --e) {
+            const float delta = Gv[e] + cc;
+            cc = __builtin_fmaf(g[e], cc, pr[e]);
+            float mine;
+            if constexpr (PLAIN) {
+                dtok[e] += delta;
+                mine = hp[e] * delta;
+            } else {
+                dtok[e] = __builtin_fmaf(-g[e], delta, dtok[e] + delta);
+                mine = (hp[e] - x[e]) * delta;
+            }
+            dg[e] = active ? mine : 0.0f;
+        }
+        sum_over_groups<E>(dg, lpr_log2);
+        if (group == 0 && p < CL) {
+            float* dst = gate_grad_partial + (gate_row * G + tile) * L + t0;
+#pragma unroll
+            for (int e = 0; e < E; e += 4)
+                *reinterpret_cast<float4*>(dst + e) = make_float4(dg[e], dg[e + 1], dg[e + 2], dg[e + 3]);
+        }
+        cur = next;
+    }
+    if (active) store16<T>(token_grad + token_row * L + t0, Elem<T>::pack(dtok));
+}
+
 }  // namespace fmscan

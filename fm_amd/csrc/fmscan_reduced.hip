@@ -2,6 +2,7 @@
 // D and M inside. Contract: include/fmscan.h.
 #include "fmscan_host.h"
 #include "fmscan_reduced.h"
+#include "fmscan_packed.h"
 
 using namespace fmscan::host;
 
@@ -254,8 +255,9 @@ int fmscan_reduced_plan(int64_t B, int64_t M, int64_t D, int64_t L, int dtype, i
 
 int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype) {
     if (B < 1 || M < 2 || D < 2 || L < 1) return 0;
-    // Rows of at most 256 bytes leave three quarters of this kernel's lanes idle, and
-    // fmscan_backward puts several such rows into a wave (bf16, ms, against it and the two sums:
+    // Rows of at most 256 bytes leave three quarters of this kernel's lanes idle; fmscan_backward_reduced_packed
+    // (where fmscan_reduced_packed_groups is not 0) and fmscan_backward put several such rows into a wave
+    // (bf16, ms, this kernel against fmscan_backward and the two sums:
     // (512,32,128,64) 0.73 against 0.30, (256,32,128,128) 0.39 against 0.29, (128,32,128,256) 0.21 against 0.28).
     const int64_t row_bytes = L * (dtype == FMSCAN_DTYPE_F32 ? 4 : 2);
     if (row_bytes <= 256) return 0;
@@ -290,6 +292,78 @@ int fmscan_backward_layer_split(const void* gates, const void* states_n, const f
                             input_tokens, gate_grad_partial, initial_state, initial_state_grad, coef_out, coef_self,
                             out_grad, rms, B, M, D, L, dtype, flags, stream, token_grad_partial, split, true, segments,
                             workspace, workspace_bytes);
+}
+
+// Rows of at most 256 bytes of whole 16-byte vectors, and enough (b, tile of rows) pairs to fill the GPU:
+// the kernel that puts several rows into a wave and walks the slots (fmscan_packed.h). 0: not for this shape.
+int64_t fmscan_reduced_packed_groups(int64_t B, int64_t M, int64_t D, int64_t L, int dtype) {
+    if (B < 1 || M < 1 || D < 1 || L < 1) return 0;
+    if (dtype != FMSCAN_DTYPE_F32 && dtype != FMSCAN_DTYPE_F16 && dtype != FMSCAN_DTYPE_BF16) return 0;
+    const int64_t row_bytes = L * (dtype == FMSCAN_DTYPE_F32 ? 4 : 2);
+    if (row_bytes > 256 || row_bytes % 16 != 0) return 0;
+    int lanes_log2 = 0;
+    while ((16 << lanes_log2) < row_bytes) ++lanes_log2;
+    const int64_t per_tile = 64 >> lanes_log2;
+    const int64_t groups = (D + per_tile - 1) / per_tile;
+    // a wave per (b, tile): below about four waves per SIMD of the whole GPU fmscan_backward and the two sums
+    // are faster (they spread over rows, not over (b, tile) pairs)
+    if ((__int128)B * groups < 4096) return 0;
+    return groups;
+}
+
+int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, const void* first_prop_grad,
+                                   void* token_grad, const void* cached_output, const void* input_tokens,
+                                   float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                                   void* stream) {
+    const char* who = "fmscan_backward_reduced_packed";
+    Problem pb;
+    if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
+    if (flags & ~FMSCAN_FLAG_PLAIN) return fail(FMSCAN_E_FLAGS, "%s: only FMSCAN_FLAG_PLAIN is understood here", who);
+    const int64_t groups = fmscan_reduced_packed_groups(B, M, D, L, dtype);
+    if (groups < 1)
+        return fail(FMSCAN_E_SHAPE, "%s: not for this shape (fmscan_reduced_packed_groups is 0): rows of whole "
+                    "16-byte vectors up to 256 bytes, 4096 (b, tile of rows) pairs or more", who);
+    if (!gates || !out_grad || !token_grad || !cached_output || !gate_grad_partial)
+        return fail(FMSCAN_E_NULL, "%s: gates, out_grad, token_grad, cached_output and gate_grad_partial must not "
+                    "be NULL", who);
+    if (!pb.plain && !input_tokens)
+        return fail(FMSCAN_E_NULL, "%s: input_tokens must not be NULL without FMSCAN_FLAG_PLAIN", who);
+    if (B > INT32_MAX || (__int128)B * groups > (__int128)INT32_MAX)
+        return fail(FMSCAN_E_SHAPE, "%s: B * groups must be < 2^31", who);
+    const int64_t full = pb.rows * L * pb.esize;
+    const Range outs[] = {{"token_grad", token_grad, B * D * L * pb.esize},
+                          {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
+                          {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
+    const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
+                         {"out_grad", out_grad, full},
+                         {"first_prop_grad", first_prop_grad, pb.rows * pb.esize},
+                         {"cached_output", cached_output, full},
+                         {"input_tokens", pb.plain ? nullptr : input_tokens, B * D * L * pb.esize},
+                         {"initial_state", initial_state, pb.rows * pb.esize}};
+    for (const Range& o : outs)
+        for (const Range& in : ins)
+            if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
+    for (int i = 0; i < 3; ++i)
+        for (int j = i + 1; j < 3; ++j)
+            if (overlap(outs[i], outs[j])) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, outs[i].name, outs[j].name);
+    if (!(aligned16(gates) && aligned16(out_grad) && aligned16(token_grad) && aligned16(cached_output) &&
+          (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial)))
+        return fail(FMSCAN_E_UNALIGNED, "%s: pointers must be multiples of 16 bytes", who);
+    // NULL initial_state reproduces the reference kernel: h[-1] := first_prop_grad
+    const void* h_init = initial_state ? initial_state : first_prop_grad;
+    const int32_t lanes_log2 = packed_lanes_log2(pb);
+    const unsigned grid = (unsigned)((B * groups + 3) / 4);
+    with_dtype(dtype, [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        with_bool(pb.plain, [&](auto pt) {
+            fmscan::scan_backward_reduced_packed_kernel<T, decltype(pt)::value><<<grid, 256, 0, (hipStream_t)stream>>>(
+                (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad, (const T*)cached_output,
+                (const T*)input_tokens, gate_grad_partial, (const T*)h_init, (T*)initial_state_grad, (int32_t)B,
+                (int32_t)M, (int32_t)D, (int32_t)L, lanes_log2, (int32_t)groups);
+        });
+    });
+    return launched(who);
 }
 
 int fmscan_sum_groups(const float* partial, int64_t G, void* out, int64_t rows, int64_t L, int dtype,

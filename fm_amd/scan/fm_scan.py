@@ -200,6 +200,11 @@ def _reduced_ok(gates, tokens, states, grad_output) -> bool:
     return all(t.data_ptr() % 16 == 0 for t in (gates, tokens, states, grad_output))
 
 
+def _packed_reduced_ok(*tensors):
+    """fmscan_backward_reduced_packed needs 16-byte aligned pointers (the rows' length is the library's to judge)."""
+    return all(t.data_ptr() % 16 == 0 for t in tensors)
+
+
 def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input_tokens, *,
                              initial_state=None, initial_state_grad=None, plain=False):
     """Backward scan that returns the summed gradients (d_gates (B, M, L), d_tokens (B, D, L))
@@ -227,6 +232,19 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
         if t is not None:
             _require(t.numel() == B * M * D, f"{name} must hold {B * M * D} elements")
     code = _dtype_code(gates)
+    flags = _lib.FLAG_PLAIN if plain else 0
+    # short rows: the kernel that puts several rows into a wave, where the library says it applies
+    packed_groups = _raw.fmscan_reduced_packed_groups(B, M, D, L, code) if _packed_reduced_ok(
+        gates, outGrad, cached_output, input_tokens) else 0
+    if packed_groups > 0:
+        partial = torch.empty((B, M, packed_groups, L), dtype=torch.float32, device=dev)
+        d_tokens = torch.empty((B, D, L), dtype=gates.dtype, device=dev)
+        with _on_device(dev):
+            _lib.check(_raw.fmscan_backward_reduced_packed(
+                gates.data_ptr(), outGrad.data_ptr(), firstPropGrad.data_ptr(), d_tokens.data_ptr(),
+                cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state),
+                _ptr(initial_state_grad), B, M, D, L, code, flags, torch.cuda.current_stream(dev).cuda_stream))
+        return _sum_groups(partial, gates.dtype), d_tokens
     # few batch elements: the rows are cut into segments (not in the plain form) and the slots of a batch
     # element dealt to `split` blocks, as the library plans it; those blocks' token gradients are summed after
     split, segments = _reduced_plan(B, M, D, L, code) if cached_output.numel() else (1, 1)
@@ -234,7 +252,6 @@ def fm_scan_backward_reduced(gates, outGrad, firstPropGrad, cached_output, input
         split, segments = max(1, _raw.fmscan_reduced_split(B, M, D)), 1
     groups = _raw.fmscan_reduced_groups(B * split, D)
     partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
-    flags = _lib.FLAG_PLAIN if plain else 0
     common = (cached_output.data_ptr(), input_tokens.data_ptr(), partial.data_ptr(), _ptr(initial_state),
               _ptr(initial_state_grad), B, M, D, L)
     if split > 1 or segments > 1:
@@ -322,7 +339,9 @@ def _scan_gradients(gates, tokens, states, initial_state, grad_output, want_init
     # is returned here when autograd asks for it, as its per-timestep PyTorch path would.
     d_initial_state = torch.empty_like(first_prop_grad) if want_initial_state_grad else None
 
-    if _reduced_ok(gates, tokens, states, grad_output) and _raw.fmscan_reduced_pays(B, M, D, L, _dtype_code(gates)):
+    code = _dtype_code(gates)
+    if _reduced_ok(gates, tokens, states, grad_output) and (
+            _raw.fmscan_reduced_pays(B, M, D, L, code) or _raw.fmscan_reduced_packed_groups(B, M, D, L, code) > 0):
         # both sums are real: one kernel produces d_gates and d_tokens directly (unless the shape leaves
         # it too few blocks: very few batch elements, slots and channels, rows too short to cut)
         d_gates, d_tokens = fm_scan_backward_reduced(

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FMSCAN_ABI_VERSION 6
+#define FMSCAN_ABI_VERSION 7
 
 /* element type of every tensor in one call (reference fm_scan.cuh:333-342) */
 #define FMSCAN_DTYPE_F32  0
@@ -272,6 +272,20 @@ int64_t fmscan_reduced_split(int64_t B, int64_t M, int64_t D);
  * 256 bytes, where fmscan_backward puts several rows into a wave and this kernel
  * leaves most lanes idle. */
 int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
+/* fmscan_backward_reduced for short rows: rows of whole 16-byte vectors up to 256 bytes, which
+ * fmscan_backward_reduced gives a wave instruction each (most lanes idle). Several rows share a wave, a wave
+ * takes one batch element and a tile of rows d and walks the M slots: token_grad (B, D, L) is complete,
+ * gate_grad_partial is (B, M, G, L) float32 with G = fmscan_reduced_packed_groups(B, M, D, L, dtype), to be
+ * added by fmscan_sum_groups. That query returns 0 where the call does not apply (longer or unaligned rows,
+ * fewer than 4096 (b, tile) pairs): then the call returns FMSCAN_E_SHAPE. Arguments, flags (FMSCAN_FLAG_PLAIN
+ * only) and results otherwise as fmscan_backward_reduced; results agree with it to float32 rounding.
+ * No counterpart in the reference (fm_scan.py:70-78 writes two (B, M, D, L) tensors and sums them). */
+int64_t fmscan_reduced_packed_groups(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
+int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, const void* first_prop_grad,
+                                   void* token_grad, const void* cached_output, const void* input_tokens,
+                                   float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                                   void* stream);
 int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,
                                   float* token_grad_partial,
                                   const void* cached_output, const void* input_tokens,

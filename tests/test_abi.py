@@ -25,14 +25,15 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
                                     "fmscan_backward_layer_split", "fmscan_backward_reduced",
-                                    "fmscan_backward_reduced_split", "fmscan_build_id", "fmscan_forward",
+                                    "fmscan_backward_reduced_packed", "fmscan_backward_reduced_split",
+                                    "fmscan_build_id", "fmscan_forward",
                                     "fmscan_forward_normed", "fmscan_forward_normed_cut",
                                     "fmscan_forward_normed_max_d", "fmscan_forward_normed_pays",
                                     "fmscan_forward_normed_segments", "fmscan_forward_static",
                                     "fmscan_forward_sumsq", "fmscan_last_error", "fmscan_layer_finish",
                                     "fmscan_layer_prepare", "fmscan_readout_backward", "fmscan_readout_dot",
                                     "fmscan_readout_forward", "fmscan_readout_inv_rms", "fmscan_reduced_groups",
-                                    "fmscan_reduced_pays", "fmscan_reduced_plan", "fmscan_reduced_split",
+                                    "fmscan_reduced_packed_groups", "fmscan_reduced_pays", "fmscan_reduced_plan", "fmscan_reduced_split",
                                     "fmscan_sum_groups", "fmscan_sumsq_finish", "fmscan_sumsq_groups",
                                     "fmscan_swap_last_two", "fmscan_workspace_bytes"]
 
@@ -78,8 +79,8 @@ def bwd(lib, g=P, G=2 * P, fpg=None, dx=3 * P, h=4 * P, x=5 * P, dg=6 * P, h0=No
 
 
 def test_rejected_arguments(lib):
-    E_NULL, E_SHAPE, E_DTYPE, E_FLAGS, E_ALIAS, E_WORKSPACE = (
-        _const("FMSCAN_E_" + n) for n in ("NULL", "SHAPE", "DTYPE", "FLAGS", "ALIAS", "WORKSPACE"))
+    E_NULL, E_SHAPE, E_DTYPE, E_FLAGS, E_ALIAS, E_WORKSPACE, E_UNALIGNED = (
+        _const("FMSCAN_E_" + n) for n in ("NULL", "SHAPE", "DTYPE", "FLAGS", "ALIAS", "WORKSPACE", "UNALIGNED"))
     assert fwd(lib, g=None) == E_NULL
     assert b"NULL" in lib.fmscan_last_error()
     assert fwd(lib, out=None) == E_NULL
@@ -159,6 +160,19 @@ def test_rejected_arguments(lib):
     # rows of up to 256 bytes: fmscan_backward packs several into a wave
     assert pays(512, 32, 128, 64, 2) == 0 and pays(256, 32, 128, 128, 2) == 0 and pays(128, 32, 128, 256, 2) == 1
     assert pays(256, 32, 128, 64, 0) == 0 and pays(256, 32, 128, 68, 0) == 1 and pays(256, 32, 128, 100, 2) == 0
+    # the kernel with the sums inside for such rows: groups of the rows a wave holds, 0 where it does not apply
+    pg = lib.fmscan_reduced_packed_groups
+    assert pg(512, 32, 128, 64, 2) == 16 and pg(256, 32, 128, 128, 2) == 32 and pg(2048, 32, 128, 16, 2) == 4
+    assert pg(512, 32, 128, 64, 0) == 32 and pg(128, 32, 128, 256, 2) == 0 and pg(512, 32, 128, 100, 2) == 0
+    assert pg(8, 32, 128, 64, 2) == 0 and pg(0, 32, 128, 64, 2) == 0 and pg(512, 32, 128, 64, 9) == 0
+    assert lib.fmscan_backward_reduced_packed(P, 2 * P, None, 3 * P, 4 * P, 5 * P, 6 * P, None, None,
+                                              8, 32, 128, 64, 2, 0, None) == E_SHAPE   # too few rows for it
+    assert lib.fmscan_backward_reduced_packed(P, 2 * P, None, 3 * P, 4 * P, 5 * P, 6 * P, None, None,
+                                              512, 32, 128, 64, 2, 2, None) == E_FLAGS
+    assert lib.fmscan_backward_reduced_packed(P, 2 * P, None, None, 4 * P, 5 * P, 6 * P, None, None,
+                                              512, 32, 128, 64, 2, 0, None) == E_NULL
+    assert lib.fmscan_backward_reduced_packed(P + 2, 2 * P, None, 3 * P, 4 * P, 5 * P, 6 * P, None, None,
+                                              512, 32, 128, 64, 2, 0, None) == E_UNALIGNED
     assert lib.fmscan_forward_normed_pays(32, 32, 128) == 1 and lib.fmscan_forward_normed_pays(2, 32, 128) == 1
     assert lib.fmscan_forward_normed_pays(1, 32, 128) == 0 and lib.fmscan_forward_normed_pays(1, 8, 2048) == 1
     # scan and norm in one kernel with the sequence cut: no cut without a workspace, no more segments than tiles

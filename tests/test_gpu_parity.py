@@ -616,6 +616,58 @@ def test_short_rows_several_per_wave(scan, dtype):
     assert n == (64 + 12) + (15 + 3 if dtype == torch.float32 else 17 + 4)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_short_rows_backward_with_the_sums_inside(scan, dtype):
+    """fmscan_backward_reduced_packed (rows of up to 256 bytes, through fm_scan_backward_reduced, which asks the
+    library whether it applies): groups of 1 to 16 lanes, numbers of chunks that are not powers of two, D that is
+    not a multiple of the rows of a wave and D below them, both forms, initial state, first_prop_grad and the
+    initial-state gradient; against the oracle's sums, and against fmscan_backward followed by torch.sum."""
+    E = 4 if dtype == torch.float32 else 8
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    lib = scan.module
+    n = 0
+    for chunks, M, D, plain in ((1, 2, 5, False), (2, 3, 70, False), (3, 2, 9, True), (4, 2, 16, False), (5, 3, 20, False),
+                                (8, 2, 24, True), (13, 2, 6, False), (16, 3, 10, False)):
+        L = chunks * E
+        lanes = 1
+        while lanes < chunks:
+            lanes *= 2
+        G = -(-D // (64 // lanes))
+        B = -(-4096 // G) + 3
+        assert lib.fmscan_reduced_packed_groups(B, M, D, L, code) == G, (B, M, D, L)
+        gen = torch.Generator().manual_seed(77 + chunks)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        G_out = torch.randn(B, M, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        fpg = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV)
+        out = torch.empty(B, M, D, L, dtype=dtype, device=DEV)
+        scan.fm_scan_forward(g, x, h0, out, plain=plain)
+        dh0 = torch.empty_like(h0)
+        d_g, d_x = scan.fm_scan_backward_reduced(g, G_out, fpg, out, x, initial_state=h0, initial_state_grad=dh0,
+                                                 plain=plain)
+        assert d_g.shape == (B, M, L) and d_x.shape == (B, D, L) and d_g.dtype == dtype
+        tag = f"{(B, M, D, L)} {dtype} plain={plain}"
+        tg, gg, delta = O.backward_per_row(g, G_out, out, x, fpg, h0, plain)
+        check(tag + " d_gates", d_g, gg.sum(axis=2), TOL[dtype])
+        check(tag + " d_tokens", d_x, tg.sum(axis=1), TOL[dtype])
+        check(tag + " d_initial_state", dh0, O.to_f64(g)[:, :, 0][:, :, None] * delta[..., 0], TOL[dtype])
+        dx, dg, dh1 = torch.empty_like(out), torch.empty_like(out), torch.empty_like(h0)
+        scan.fm_scan_backward(g, G_out, fpg, dx, out, x, dg, initial_state=h0, initial_state_grad=dh1, plain=plain)
+        check(tag + " vs two-tensor route (gates)", d_g, dg.float().sum(dim=2).double().cpu().numpy(), 2 * TOL[dtype])
+        check(tag + " vs two-tensor route (tokens)", d_x, dx.float().sum(dim=1).double().cpu().numpy(), 2 * TOL[dtype])
+        assert torch.equal(dh0, dh1), tag + ": the initial-state gradient is the same arithmetic in both"
+        # the reference's call: no initial state (first_prop_grad stands in for it in the gate gradient)
+        d_g2, d_x2 = scan.fm_scan_backward_reduced(g, G_out, fpg, out, x, plain=plain)
+        tg2, gg2 = C.backward_f64(g, G_out, out, x, fpg, None, plain)
+        check(tag + " d_gates (reference call)", d_g2, gg2.sum(axis=2), TOL[dtype])
+        check(tag + " d_tokens (reference call)", d_x2, tg2.sum(axis=1), TOL[dtype])
+        again = scan.fm_scan_backward_reduced(g, G_out, fpg, out, x, plain=plain)
+        assert torch.equal(again[0], d_g2) and torch.equal(again[1], d_x2), tag + ": not deterministic"
+        n += 1
+    assert n == 8
+
+
 def test_short_rows_do_not_see_their_neighbours(scan):
     """Several rows share a wave, and the wave scan runs across all of its lanes: a row's results must be
     the same bits wherever it sits and whatever its neighbours hold, NaN and infinity included."""
