@@ -99,6 +99,8 @@ def load() -> ctypes.CDLL:
     lib.fmscan_reduced_packed_groups.argtypes = [c_int64] * 4 + [c_int]
     lib.fmscan_backward_reduced_packed.restype = c_int
     lib.fmscan_backward_reduced_packed.argtypes = [c_void_p] * 9 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
+    lib.fmscan_backward_layer_packed.restype = c_int
+    lib.fmscan_backward_layer_packed.argtypes = [c_void_p] * 13 + [c_int64] * 4 + [c_int, c_uint, c_void_p]
     lib.fmscan_backward_reduced_split.restype = c_int
     lib.fmscan_backward_reduced_split.argtypes = ([c_void_p] * 9 + [c_int64] * 6 + [c_void_p, c_size_t]
                                                   + [c_int, c_uint, c_void_p])

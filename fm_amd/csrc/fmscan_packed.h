@@ -250,12 +250,18 @@ __device__ __forceinline__ void sum_over_groups(float (&v)[E], int32_t lpr_log2)
     for (int e = 0; e < E; ++e) v[e] = add_across<32>(add_across<16>(v[e]));
 }
 
-template <typename T, bool PLAIN>
+// LAYER (as in scan_backward_reduced_kernel): the gradient that arrives at the states is made on the spot,
+//   G[b,m,d,t] = coef_out[b,m,t] * layer_out_grad[b,d,t] - coef_self[b,m,t] * out_grad[b,m,d,t],
+// `out_grad` then carrying the normalised states; LAYER == 2: the scanned states are not read either but
+// taken back from the normalised ones, h = out_grad * rms (h_saved is NULL). coef_out, coef_self, rms: float32.
+template <typename T, bool PLAIN, int LAYER>
 __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
     const T* __restrict__ gates, const T* __restrict__ out_grad, const T* __restrict__ first_prop_grad,
     T* __restrict__ token_grad /* (B, D, L) */, const T* __restrict__ h_saved, const T* __restrict__ tokens,
     float* __restrict__ gate_grad_partial /* (B * M, G, L) */, const T* __restrict__ h0, T* __restrict__ h0_grad,
-    int32_t B, int32_t M, int32_t D, int32_t L, int32_t lpr_log2, int32_t G) {
+    const float* __restrict__ coef_out, const float* __restrict__ coef_self, const T* __restrict__ layer_out_grad,
+    const float* __restrict__ rms, int32_t B, int32_t M, int32_t D, int32_t L, int32_t lpr_log2, int32_t G) {
+    static_assert(LAYER == 0 || !PLAIN, "the layer's scan is the Factorization-Memory form");
     constexpr int E = Elem<T>::E;
     const int32_t CL = L / E;  // rows are whole 16-byte vectors
     const int lane = threadIdx.x & 63;
@@ -274,12 +280,16 @@ __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
 
     float x[E];
     if constexpr (!PLAIN) Elem<T>::unpack(load16<T, false>(tokens + token_row * L + t0), x);
+    [[maybe_unused]] float y[E];  // LAYER: the gradient of the layer's output at this row
+    if constexpr (LAYER != 0) Elem<T>::unpack(load16<T, false>(layer_out_grad + token_row * L + t0), y);
     float dtok[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) dtok[e] = 0.0f;
 
     struct In {
-        u32x4 g, G, h;
+        u32x4 g, G;
+        u32x4 h;                    // LAYER != 2: the saved states
+        FloatChunk<E> co, cs, rr;   // LAYER; rr: LAYER == 2
         float cinit, hinit;
     };
     auto fetch = [&](In& n, int32_t m) {
@@ -287,7 +297,12 @@ __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
         const int64_t row = gate_row * D + d;
         n.g = load16<T, false>(gates + gate_row * L + t0);
         n.G = load16<T, true>(out_grad + row * L + t0);
-        n.h = load16<T, true>(h_saved + row * L + t0);
+        if constexpr (LAYER != 2) n.h = load16<T, true>(h_saved + row * L + t0);
+        if constexpr (LAYER != 0) {
+            n.co = load_float_chunk<E>(coef_out + gate_row * L + t0);
+            n.cs = load_float_chunk<E>(coef_self + gate_row * L + t0);
+        }
+        if constexpr (LAYER == 2) n.rr = load_float_chunk<E>(rms + gate_row * L + t0);
         n.cinit = (first_prop_grad && p == 0) ? Elem<T>::widen(first_prop_grad[row]) : 0.0f;
         n.hinit = (h0 && c == 0) ? Elem<T>::widen(h0[row]) : 0.0f;
     };
@@ -296,15 +311,29 @@ __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
     for (int32_t m = 0; m < M; ++m) {
         fetch(next, m + 1 < M ? m + 1 : m);
         const int64_t gate_row = (int64_t)b * M + m;
-        u32x4 gq = cur.g, Gq = cur.G;
-        if (!active) {  // identity steps
-            gq = u32x4{Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes, Elem<T>::kOnes};
-            Gq = u32x4{0u, 0u, 0u, 0u};
-        }
         float g[E], Gv[E], pr[E], h[E];
-        Elem<T>::unpack(gq, g);
-        Elem<T>::unpack(Gq, Gv);
-        Elem<T>::unpack(cur.h, h);
+        Elem<T>::unpack(cur.g, g);
+        Elem<T>::unpack(cur.G, Gv);
+        if constexpr (LAYER == 2) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) h[e] = Gv[e];  // the normalised states; their factor follows below
+        } else {
+            Elem<T>::unpack(cur.h, h);
+        }
+        if constexpr (LAYER != 0) {
+            float co[E], cs[E];
+            spread<E>(cur.co, co);
+            spread<E>(cur.cs, cs);
+#pragma unroll
+            for (int e = 0; e < E; ++e) Gv[e] = __builtin_fmaf(-cs[e], Gv[e], co[e] * y[e]);
+        }
+        if (!active) {  // identity steps
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                g[e] = 1.0f;
+                Gv[e] = 0.0f;
+            }
+        }
 #pragma unroll
         for (int e = 0; e < E; ++e) pr[e] = g[e] * Gv[e];
         float a = g[E - 1], bb = pr[E - 1];
@@ -324,11 +353,22 @@ __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
             if constexpr (sizeof(T) == 4) reinterpret_cast<uint32_t*>(h0_grad)[row] = packed.x;
             else reinterpret_cast<uint16_t*>(h0_grad)[row] = (uint16_t)(packed.x & 0xffffu);
         }
+        // hp[e] = the state before element e: the last element of the chunk before this one in memory is with
+        // the next lane; the row's first chunk takes the state before the row
         const float behind = dpp<kWaveShl1>(0.0f, h[E - 1]);
         float hp[E];
-        hp[0] = c == 0 ? cur.hinit : behind;
+        hp[0] = behind;
 #pragma unroll
         for (int e = 1; e < E; ++e) hp[e] = h[e - 1];
+        if constexpr (LAYER == 2) {  // h = normalised state * rms, each at the step before
+            float rr[E];
+            spread<E>(cur.rr, rr);
+            const float rr_behind = dpp<kWaveShl1>(1.0f, rr[E - 1]);
+            hp[0] *= rr_behind;
+#pragma unroll
+            for (int e = 1; e < E; ++e) hp[e] *= rr[e - 1];
+        }
+        if (c == 0) hp[0] = cur.hinit;  // the state before the row, as it is
         float dg[E];
 #pragma unroll
         for (int e = E - 1; e >= 0; --e) {

@@ -311,22 +311,31 @@ int64_t fmscan_reduced_packed_groups(int64_t B, int64_t M, int64_t D, int64_t L,
     return groups;
 }
 
-int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, const void* first_prop_grad,
-                                   void* token_grad, const void* cached_output, const void* input_tokens,
-                                   float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
-                                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
-                                   void* stream) {
-    const char* who = "fmscan_backward_reduced_packed";
+// Shared by fmscan_backward_reduced_packed and fmscan_backward_layer_packed (coef_out != NULL: `out_grad`
+// carries the normalised states and the gradient of the states is made in the kernel).
+static int backward_reduced_packed(const char* who, const void* gates, const void* out_grad,
+                                   const void* first_prop_grad, void* token_grad, const void* cached_output,
+                                   const void* input_tokens, float* gate_grad_partial, const void* initial_state,
+                                   void* initial_state_grad, const float* coef_out, const float* coef_self,
+                                   const void* layer_out_grad, const float* rms, int64_t B, int64_t M, int64_t D,
+                                   int64_t L, int dtype, unsigned flags, void* stream) {
     Problem pb;
     if (int rc = parse(B, M, D, L, dtype, flags & FMSCAN_FLAG_PLAIN, &pb)) return rc;
     if (flags & ~FMSCAN_FLAG_PLAIN) return fail(FMSCAN_E_FLAGS, "%s: only FMSCAN_FLAG_PLAIN is understood here", who);
+    const bool layer = coef_out != nullptr;
+    const bool recover = layer && !cached_output;  // the states come back from states_n * rms
+    if (layer && pb.plain) return fail(FMSCAN_E_FLAGS, "%s: the layer's scan has no FMSCAN_FLAG_PLAIN form", who);
     const int64_t groups = fmscan_reduced_packed_groups(B, M, D, L, dtype);
     if (groups < 1)
         return fail(FMSCAN_E_SHAPE, "%s: not for this shape (fmscan_reduced_packed_groups is 0): rows of whole "
                     "16-byte vectors up to 256 bytes, 4096 (b, tile of rows) pairs or more", who);
-    if (!gates || !out_grad || !token_grad || !cached_output || !gate_grad_partial)
-        return fail(FMSCAN_E_NULL, "%s: gates, out_grad, token_grad, cached_output and gate_grad_partial must not "
-                    "be NULL", who);
+    if (!gates || !out_grad || !token_grad || (!cached_output && !recover) || !gate_grad_partial)
+        return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
+                    "be NULL", who, layer ? "states_n" : "out_grad");
+    if (recover && !rms)
+        return fail(FMSCAN_E_NULL, "%s: without cached_output the states are states_n * rms: rms must not be NULL", who);
+    if (layer && (!coef_self || !layer_out_grad))
+        return fail(FMSCAN_E_NULL, "%s: coef_self and out_grad must not be NULL", who);
     if (!pb.plain && !input_tokens)
         return fail(FMSCAN_E_NULL, "%s: input_tokens must not be NULL without FMSCAN_FLAG_PLAIN", who);
     if (B > INT32_MAX || (__int128)B * groups > (__int128)INT32_MAX)
@@ -336,11 +345,15 @@ int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, cons
                           {"gate_grad_partial", gate_grad_partial, B * M * groups * L * 4},
                           {"initial_state_grad", initial_state_grad, pb.rows * pb.esize}};
     const Range ins[] = {{"gates", gates, B * M * L * pb.esize},
-                         {"out_grad", out_grad, full},
+                         {layer ? "states_n" : "out_grad", out_grad, full},
                          {"first_prop_grad", first_prop_grad, pb.rows * pb.esize},
                          {"cached_output", cached_output, full},
                          {"input_tokens", pb.plain ? nullptr : input_tokens, B * D * L * pb.esize},
-                         {"initial_state", initial_state, pb.rows * pb.esize}};
+                         {"initial_state", initial_state, pb.rows * pb.esize},
+                         {"coef_out", coef_out, B * M * L * 4},
+                         {"coef_self", layer ? coef_self : nullptr, B * M * L * 4},
+                         {"out_grad", layer ? layer_out_grad : nullptr, B * D * L * pb.esize},
+                         {"rms", recover ? rms : nullptr, B * M * L * 4}};
     for (const Range& o : outs)
         for (const Range& in : ins)
             if (overlap(o, in)) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, o.name, in.name);
@@ -348,7 +361,8 @@ int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, cons
         for (int j = i + 1; j < 3; ++j)
             if (overlap(outs[i], outs[j])) return fail(FMSCAN_E_ALIAS, "%s: %s overlaps %s", who, outs[i].name, outs[j].name);
     if (!(aligned16(gates) && aligned16(out_grad) && aligned16(token_grad) && aligned16(cached_output) &&
-          (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial)))
+          (pb.plain || aligned16(input_tokens)) && aligned16(gate_grad_partial) && (!recover || aligned16(rms)) &&
+          (!layer || (aligned16(coef_out) && aligned16(coef_self) && aligned16(layer_out_grad)))))
         return fail(FMSCAN_E_UNALIGNED, "%s: pointers must be multiples of 16 bytes", who);
     // NULL initial_state reproduces the reference kernel: h[-1] := first_prop_grad
     const void* h_init = initial_state ? initial_state : first_prop_grad;
@@ -356,14 +370,42 @@ int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, cons
     const unsigned grid = (unsigned)((B * groups + 3) / 4);
     with_dtype(dtype, [&](auto tt) {
         using T = typename decltype(tt)::type;
-        with_bool(pb.plain, [&](auto pt) {
-            fmscan::scan_backward_reduced_packed_kernel<T, decltype(pt)::value><<<grid, 256, 0, (hipStream_t)stream>>>(
-                (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad, (const T*)cached_output,
-                (const T*)input_tokens, gate_grad_partial, (const T*)h_init, (T*)initial_state_grad, (int32_t)B,
-                (int32_t)M, (int32_t)D, (int32_t)L, lanes_log2, (int32_t)groups);
-        });
+        auto go = [&](auto pt, auto lt) {
+            fmscan::scan_backward_reduced_packed_kernel<T, decltype(pt)::value, decltype(lt)::value>
+                <<<grid, 256, 0, (hipStream_t)stream>>>(
+                    (const T*)gates, (const T*)out_grad, (const T*)first_prop_grad, (T*)token_grad,
+                    (const T*)cached_output, (const T*)input_tokens, gate_grad_partial, (const T*)h_init,
+                    (T*)initial_state_grad, coef_out, coef_self, (const T*)layer_out_grad, recover ? rms : nullptr,
+                    (int32_t)B, (int32_t)M, (int32_t)D, (int32_t)L, lanes_log2, (int32_t)groups);
+        };
+        if (recover) go(BoolTag<false>{}, IntTag<2>{});
+        else if (layer) go(BoolTag<false>{}, IntTag<1>{});
+        else if (pb.plain) go(BoolTag<true>{}, IntTag<0>{});
+        else go(BoolTag<false>{}, IntTag<0>{});
     });
     return launched(who);
+}
+
+int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, const void* first_prop_grad,
+                                   void* token_grad, const void* cached_output, const void* input_tokens,
+                                   float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
+                                   int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
+                                   void* stream) {
+    return backward_reduced_packed("fmscan_backward_reduced_packed", gates, out_grad, first_prop_grad, token_grad,
+                                   cached_output, input_tokens, gate_grad_partial, initial_state, initial_state_grad,
+                                   nullptr, nullptr, nullptr, nullptr, B, M, D, L, dtype, flags, stream);
+}
+
+int fmscan_backward_layer_packed(const void* gates, const void* states_n, const float* coef_out,
+                                 const float* coef_self, const void* out_grad, const void* first_prop_grad,
+                                 void* token_grad, const void* cached_output, const float* rms,
+                                 const void* input_tokens, float* gate_grad_partial, const void* initial_state,
+                                 void* initial_state_grad, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                                 unsigned flags, void* stream) {
+    if (!coef_out) return fail(FMSCAN_E_NULL, "fmscan_backward_layer_packed: coef_out must not be NULL");
+    return backward_reduced_packed("fmscan_backward_layer_packed", gates, states_n, first_prop_grad, token_grad,
+                                   cached_output, input_tokens, gate_grad_partial, initial_state, initial_state_grad,
+                                   coef_out, coef_self, out_grad, rms, B, M, D, L, dtype, flags, stream);
 }
 
 int fmscan_sum_groups(const float* partial, int64_t G, void* out, int64_t rows, int64_t L, int dtype,

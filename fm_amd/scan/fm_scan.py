@@ -594,8 +594,12 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
         # few batch elements: the rows are cut into segments and the slots of a batch element dealt to
         # `split` blocks, as the library plans it; the token gradients of those blocks are summed after
         split, segments = _reduced_plan(B, M, D, L, code)
+        # short rows: the kernel that puts several rows into a wave, where the library says it applies
+        packed_groups = _raw.fmscan_reduced_packed_groups(B, M, D, L, code)
+        if packed_groups > 0:
+            split, segments = 1, 1
         divided = split > 1 or segments > 1
-        groups = _raw.fmscan_reduced_groups(B * split, D)
+        groups = packed_groups if packed_groups > 0 else _raw.fmscan_reduced_groups(B * split, D)
         partial = torch.empty((B, M, groups, L), dtype=torch.float32, device=dev)
         d_h0 = torch.empty((B, M, D), dtype=dtype, device=dev) if want_initial_state_grad else None
         if divided:
@@ -616,6 +620,8 @@ def _layer_gradients(gates, tokens, states, initial_state, read, normed, inv_rms
                 _lib.check(_raw.fmscan_backward_layer_split(
                     *head, token_partial.data_ptr(), *tail, split, segments,
                     pairs.data_ptr() if segments > 1 else None, pairs.numel(), code, 0, stream))
+            elif packed_groups > 0:
+                _lib.check(_raw.fmscan_backward_layer_packed(*head, d_tokens.data_ptr(), *tail, code, 0, stream))
             else:
                 _lib.check(_raw.fmscan_backward_layer(*head, d_tokens.data_ptr(), *tail, code, 0, stream))
         if divided:

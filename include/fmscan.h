@@ -286,6 +286,15 @@ int fmscan_backward_reduced_packed(const void* gates, const void* out_grad, cons
                                    float* gate_grad_partial, const void* initial_state, void* initial_state_grad,
                                    int64_t B, int64_t M, int64_t D, int64_t L, int dtype, unsigned flags,
                                    void* stream);
+/* The same for the layer's form: arguments and results as fmscan_backward_layer (both of its forms: the
+ * saved states in cached_output, or NULL there and rms), gate_grad_partial as above. No counterpart in the
+ * reference. */
+int fmscan_backward_layer_packed(const void* gates, const void* states_n, const float* coef_out,
+                                 const float* coef_self, const void* out_grad, const void* first_prop_grad,
+                                 void* token_grad, const void* cached_output, const float* rms,
+                                 const void* input_tokens, float* gate_grad_partial, const void* initial_state,
+                                 void* initial_state_grad, int64_t B, int64_t M, int64_t D, int64_t L, int dtype,
+                                 unsigned flags, void* stream);
 int fmscan_backward_reduced_split(const void* gates, const void* out_grad, const void* first_prop_grad,
                                   float* token_grad_partial,
                                   const void* cached_output, const void* input_tokens,

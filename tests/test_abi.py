@@ -24,7 +24,7 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["fmscan_abi_version", "fmscan_backward", "fmscan_backward_layer",
-                                    "fmscan_backward_layer_split", "fmscan_backward_reduced",
+                                    "fmscan_backward_layer_packed", "fmscan_backward_layer_split", "fmscan_backward_reduced",
                                     "fmscan_backward_reduced_packed", "fmscan_backward_reduced_split",
                                     "fmscan_build_id", "fmscan_forward",
                                     "fmscan_forward_normed", "fmscan_forward_normed_cut",

@@ -88,6 +88,9 @@ LAYER_SHAPES = [
     ((16, 264, 4, 24), 1e-4, "64 slots: scan and norm in one kernel, 8 waves of 4 rows"),
     ((1, 1032, 16, 20), 1e-4, "one batch element: separate kernels forward, slots dealt to four blocks backward"),
     ((1, 4104, 8, 24), 1e-4, "few slots, long rows: the sequence cut in 2 (4 in float32), in scan + norm and in backward"),
+    ((2060, 24, 2, 20), 1e-4, "rows of at most 256 bytes, many batch elements: several rows to a wave in backward "
+                              "(4 lanes a row in bfloat16, 8 in float32; D not a multiple of the rows of a wave)"),
+    ((1030, 32, 3, 70), 1e-4, "the same with 4 / 8 lanes a row and three slots"),
 ]
 
 
