@@ -396,4 +396,125 @@ __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
     if (active) store16<T>(token_grad + token_row * L + t0, Elem<T>::pack(dtok));
 }
 
+// ---- scan and norm in one kernel, for short rows ---------------------------------------------------
+// What scan_forward_normed_kernel computes (fmscan_normed.h: the states scanned, rounded as stored states
+// are, their mean square over the D rows of a slot, states_n = state * inv_rms and inv_rms itself), with
+// several rows to a wave. A wave is a slot (b, m): it walks the slot's rows in NT tiles of 64 >> lpr_log2
+// rows, keeps every tile's rounded states packed in registers (NT <= NT_MAX), adds up their squares per
+// lane, sums those over the wave's groups (every lane ends with the sum over all D rows at its steps),
+// and scales and stores what it holds. The gates are the same for all rows of a slot: their half of the
+// segmented scan is done once, a tile scans the other half only. No LDS, no barrier.
+template <typename T, int NT_MAX>
+__global__ __launch_bounds__(256) void scan_forward_normed_packed_kernel(
+    const T* __restrict__ gates, const T* __restrict__ tokens, const T* __restrict__ h0,
+    T* __restrict__ states_n /* (B, M, D, L) */, float* __restrict__ inv_rms /* (B, M, L) */, int64_t slots,
+    int32_t M, int32_t D, int32_t L, float eps, int32_t lpr_log2, int32_t NT) {
+    constexpr int E = Elem<T>::E;
+    const int32_t CL = L / E;  // rows are whole 16-byte vectors
+    const int lane = threadIdx.x & 63;
+    const int64_t bm = (int64_t)blockIdx.x * (blockDim.x >> 6) + uniform((int)(threadIdx.x >> 6));
+    if (bm >= slots) return;  // whole waves
+    const int64_t b = (int64_t)uniform((int)((uint32_t)bm / (uint32_t)M));
+    const int32_t p = lane & ((1 << lpr_log2) - 1);
+    const int32_t group = lane >> lpr_log2;
+    const int32_t per_tile = 64 >> lpr_log2;
+    const bool in_row = p < CL;
+    const int32_t t0 = (in_row ? p : CL - 1) * E;
+
+    // the gates' half of the scan, once: the product of the chunk's gates before each of the four steps
+    // inside a group (groups are at most 16 lanes here)
+    float g[E];
+    Elem<T>::unpack(load16<T, false>(gates + bm * L + t0), g);
+    if (!in_row) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) g[e] = 1.0f;
+    }
+    float a_chunk = g[0];
+#pragma unroll
+    for (int e = 1; e < E; ++e) a_chunk *= g[e];
+    float a_before[4];
+    {
+        float a = a_chunk;
+        a_before[0] = a;
+        a = p >= 1 ? a * dpp<0x111, 0xf>(1.0f, a) : a;
+        a_before[1] = a;
+        a = p >= 2 ? a * dpp<0x112, 0xf>(1.0f, a) : a;
+        a_before[2] = a;
+        a = p >= 4 ? a * dpp<0x114, 0xf>(1.0f, a) : a;
+        a_before[3] = a;
+    }
+
+    auto row_of = [&](int32_t i) {  // the row of this lane in tile i (clamped: lanes without one load the last)
+        const int32_t d = i * per_tile + group;
+        return d < D ? d : D - 1;
+    };
+    constexpr int RING = 4;  // token tiles in flight
+    u32x4 xq[RING];
+#pragma unroll
+    for (int i = 0; i < RING; ++i)
+        xq[i] = load16<T, false>(tokens + (b * D + row_of(i < NT ? i : 0)) * L + t0);
+
+    u32x4 held[NT_MAX];
+    float sumsq[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) sumsq[e] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NT_MAX; ++i) {
+        if (i >= NT) continue;  // the whole wave
+        const int32_t d = row_of(i);
+        const bool active = i * per_tile + group < D && in_row;
+        float u[E];
+        Elem<T>::unpack(xq[i % RING], u);
+        if (i + RING < NT_MAX) xq[i % RING] = load16<T, false>(tokens + (b * D + row_of(i + RING < NT ? i + RING : i)) * L + t0);
+        const float hin = (h0 && p == 0) ? Elem<T>::widen(h0[bm * D + d]) : 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) u[e] = in_row ? __builtin_fmaf(-g[e], u[e], u[e]) : 0.0f;  // (1 - g) x, one rounding
+        float bb = u[0];
+#pragma unroll
+        for (int e = 1; e < E; ++e) bb = __builtin_fmaf(g[e], bb, u[e]);
+        if (p == 0) bb = __builtin_fmaf(a_chunk, hin, bb);  // the state before the row enters the group's first chunk
+        {
+            float nb = __builtin_fmaf(dpp<0x111, 0xf>(0.0f, bb), a_before[0], bb);
+            bb = p >= 1 ? nb : bb;
+            nb = __builtin_fmaf(dpp<0x112, 0xf>(0.0f, bb), a_before[1], bb);
+            bb = p >= 2 ? nb : bb;
+            nb = __builtin_fmaf(dpp<0x114, 0xf>(0.0f, bb), a_before[2], bb);
+            bb = p >= 4 ? nb : bb;
+            nb = __builtin_fmaf(dpp<0x118, 0xf>(0.0f, bb), a_before[3], bb);
+            bb = p >= 8 ? nb : bb;
+        }
+        const float before = dpp<kWaveShr1>(0.0f, bb);
+        float h = p == 0 ? hin : before;
+        float o[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            h = __builtin_fmaf(g[e], h, u[e]);
+            o[e] = h;
+        }
+        held[i] = Elem<T>::pack(o);
+        Elem<T>::unpack(held[i], o);  // the norm sees the states as they would be stored
+#pragma unroll
+        for (int e = 0; e < E; ++e) sumsq[e] = active ? __builtin_fmaf(o[e], o[e], sumsq[e]) : sumsq[e];
+    }
+    sum_over_groups<E>(sumsq, lpr_log2);
+    float r[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) r[e] = 1.0f / __builtin_sqrtf(sumsq[e] / (float)D + eps);
+    if (group == 0 && in_row) {
+        float* dst = inv_rms + bm * L + t0;
+#pragma unroll
+        for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(dst + e) = make_float4(r[e], r[e + 1], r[e + 2], r[e + 3]);
+    }
+#pragma unroll
+    for (int i = 0; i < NT_MAX; ++i) {
+        if (i < NT && i * per_tile + group < D && in_row) {
+            float o[E];
+            Elem<T>::unpack(held[i], o);
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] *= r[e];
+            store16<T>(states_n + (bm * D + i * per_tile + group) * L + t0, Elem<T>::pack(o));
+        }
+    }
+}
+
 }  // namespace fmscan

@@ -90,7 +90,7 @@ LAYER_SHAPES = [
     ((1, 4104, 8, 24), 1e-4, "few slots, long rows: the sequence cut in 2 (4 in float32), in scan + norm and in backward"),
     ((2060, 24, 2, 20), 1e-4, "rows of at most 256 bytes, many batch elements: several rows to a wave in backward "
                               "(4 lanes a row in bfloat16, 8 in float32; D not a multiple of the rows of a wave)"),
-    ((1030, 32, 3, 70), 1e-4, "the same with 4 / 8 lanes a row and three slots"),
+    ((1400, 32, 3, 70), 1e-4, "the same with 4 / 8 lanes a row and three slots"),
 ]
 
 
@@ -349,6 +349,45 @@ def test_forward_scan_and_norm_in_one_kernel(scan, dtype):
                                      1e-6, st) == -2
     assert lib.fmscan_forward_normed(g.data_ptr(), x.data_ptr(), None, n.data_ptr(), r.data_ptr(), 1, 1, 4, 63, 0,
                                      1e-6, st) == -7
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_scan_and_norm_several_rows_to_a_wave(scan, dtype):
+    """fmscan_forward_normed on rows of at most 256 bytes with 4096 slots or more: the kernel that puts several
+    rows into a wave and gives a slot a wave. Groups of 1 to 16 lanes, D that is not a multiple of the rows of
+    a wave, 2 to 32 tiles a slot (the three register budgets), with and without initial state; against the
+    three separate calls on everything, and against the float64 oracle on the first and last batch elements."""
+    lib, st = scan.module, torch.cuda.current_stream().cuda_stream
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    E = 4 if dtype == torch.float32 else 8
+    for chunks, M, D, with_h0 in ((1, 2, 70, True), (3, 3, 40, False), (5, 2, 128, True), (8, 4, 33, False),
+                                  (16, 2, 100, True), (12, 3, 128, False)):
+        L = chunks * E
+        B = -(-4096 // M) + 1
+        gen = torch.Generator().manual_seed(500 + chunks)
+        g = torch.sigmoid(torch.randn(B, M, L, generator=gen) + 2).to(dtype).to(DEV)
+        x = torch.randn(B, D, L, generator=gen).to(dtype).to(DEV)
+        h0 = torch.randn(B, M, D, generator=gen).to(dtype).to(DEV) if with_h0 else None
+        eps = 1e-5
+        normed = torch.full((B, M, D, L), float("nan"), dtype=dtype, device=DEV)
+        inv = torch.full((B, M, L), float("nan"), device=DEV)
+        rc = lib.fmscan_forward_normed(g.data_ptr(), x.data_ptr(), None if h0 is None else h0.data_ptr(),
+                                       normed.data_ptr(), inv.data_ptr(), B, M, D, L, code, eps, st)
+        assert rc == 0, lib.fmscan_last_error()
+        tag = f"{(B, M, D, L)} {dtype}"
+        tol = FWD_TOL[dtype]
+        z = torch.zeros(B, M, D, dtype=dtype, device=DEV)
+        out = torch.empty_like(normed)
+        scan.fm_scan_forward(g, x, z if h0 is None else h0, out)
+        _, n3, r3 = scan.fm_readout_forward(out, torch.ones(B, M, L, dtype=dtype, device=DEV), True, eps)
+        check_all(tag + " vs three calls", {"normalised states": normed, "inv_rms": inv},
+                  {"normalised states": n3.double().cpu().numpy(), "inv_rms": r3.double().cpu().numpy()},
+                  {"normalised states": tol, "inv_rms": 1e-5})
+        sel = torch.tensor([0, 1, 2, B - 2, B - 1], device=DEV)
+        states = O.forward(g[sel], x[sel], None if h0 is None else h0[sel])
+        _, o_normed, o_inv = O.readout_forward(states, np.ones((len(sel), M, L)), True, eps)
+        check_all(tag, {"normalised states": normed[sel], "inv_rms": inv[sel]},
+                  {"normalised states": o_normed, "inv_rms": o_inv}, {"normalised states": tol, "inv_rms": tol})
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
