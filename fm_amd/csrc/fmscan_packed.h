@@ -517,4 +517,120 @@ __global__ __launch_bounds__(256) void scan_forward_normed_packed_kernel(
     }
 }
 
+// ---- the layer's read-out and its dot, for short rows ------------------------------------------------
+// output[b,d,t] = sum_m read[b,m,t] * states[b,m,d,t] (readout_forward_kernel without the norm,
+// fmscan_readout.h; reference fm/scan/fm_scan.py:130-131). A wave is a batch element and a tile of
+// 64 >> lpr_log2 rows d and walks the M slots, the next slot's loads in flight.
+template <typename T>
+__global__ __launch_bounds__(256) void readout_forward_packed_kernel(
+    const T* __restrict__ states /* (B, M, D, L) */, const T* __restrict__ read /* (B, M, L) */,
+    T* __restrict__ output /* (B, D, L) */, int32_t B, int32_t M, int32_t D, int32_t L, int32_t lpr_log2, int32_t G) {
+    constexpr int E = Elem<T>::E;
+    const int32_t CL = L / E;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + uniform((int)(threadIdx.x >> 6));
+    if (wave >= (int64_t)B * G) return;  // whole waves
+    const int32_t b = uniform((int)(wave / G));
+    const int32_t tile = uniform((int)(wave - (int64_t)b * G));
+    const int32_t p = lane & ((1 << lpr_log2) - 1);
+    const int32_t d_mine = (tile << (6 - lpr_log2)) + (lane >> lpr_log2);
+    const bool active = d_mine < D && p < CL;
+    const int32_t d = d_mine < D ? d_mine : D - 1;
+    const int32_t t0 = (p < CL ? p : CL - 1) * E;
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+    struct In {
+        u32x4 h, wr;
+    };
+    auto fetch = [&](In& n, int32_t m) {
+        const int64_t bm = (int64_t)b * M + m;
+        n.h = load16<T, true>(states + (bm * D + d) * L + t0);
+        n.wr = load16<T, false>(read + bm * L + t0);
+    };
+    In cur, next;
+    fetch(cur, 0);
+    for (int32_t m = 0; m < M; ++m) {
+        fetch(next, m + 1 < M ? m + 1 : m);
+        float h[E], wr[E];
+        Elem<T>::unpack(cur.h, h);
+        Elem<T>::unpack(cur.wr, wr);
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[e] = __builtin_fmaf(wr[e], h[e], acc[e]);
+        cur = next;
+    }
+    if (active) store16<T>(output + ((int64_t)b * D + d) * L + t0, Elem<T>::pack(acc));
+}
+
+// q[b,m,t] = sum_d out_grad[b,d,t] * states_n[b,m,d,t] and what the layer's backward kernel takes with it
+// (rowdot_kernel in its dot form, fmscan_readout.h). A wave is a slot and walks its rows in tiles; the
+// lanes' sums meet across the wave's groups.
+template <typename T>
+__global__ __launch_bounds__(256) void readout_dot_packed_kernel(
+    const T* __restrict__ states_n /* (B, M, D, L) */, const T* __restrict__ out_grad /* (B, D, L) */,
+    float* __restrict__ q /* (B, M, L) */, const float* __restrict__ inv_rms, const T* __restrict__ read,
+    float* __restrict__ coef_out, float* __restrict__ coef_self, float* __restrict__ rms_out, int64_t slots,
+    int32_t M, int32_t D, int32_t L, int32_t lpr_log2, int32_t NT) {
+    constexpr int E = Elem<T>::E;
+    const int32_t CL = L / E;
+    const int lane = threadIdx.x & 63;
+    const int64_t bm = (int64_t)blockIdx.x * (blockDim.x >> 6) + uniform((int)(threadIdx.x >> 6));
+    if (bm >= slots) return;  // whole waves
+    const int64_t b = (int64_t)uniform((int)((uint32_t)bm / (uint32_t)M));
+    const int32_t p = lane & ((1 << lpr_log2) - 1);
+    const int32_t group = lane >> lpr_log2;
+    const int32_t per_tile = 64 >> lpr_log2;
+    const bool in_row = p < CL;
+    const int32_t t0 = (in_row ? p : CL - 1) * E;
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+    struct In {
+        u32x4 h, y;
+    };
+    auto fetch = [&](In& n, int32_t i) {
+        const int32_t d_mine = i * per_tile + group;
+        const int32_t d = d_mine < D ? d_mine : D - 1;
+        n.h = load16<T, true>(states_n + (bm * D + d) * L + t0);
+        n.y = load16<T, false>(out_grad + (b * D + d) * L + t0);
+    };
+    In cur, next;
+    fetch(cur, 0);
+    for (int32_t i = 0; i < NT; ++i) {
+        fetch(next, i + 1 < NT ? i + 1 : i);
+        const bool active = i * per_tile + group < D && in_row;
+        float h[E], y[E];
+        Elem<T>::unpack(cur.h, h);
+        Elem<T>::unpack(cur.y, y);
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[e] = active ? __builtin_fmaf(h[e], y[e], acc[e]) : acc[e];
+        cur = next;
+    }
+    sum_over_groups<E>(acc, lpr_log2);
+    if (group == 0 && in_row) {
+        const int64_t at = bm * L + t0;
+#pragma unroll
+        for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(q + at + e) = make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+        if (coef_out != nullptr || rms_out != nullptr) {
+            float r[E], wr[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e) r[e] = 1.0f;
+            if (inv_rms != nullptr) spread<E>(load_float_chunk<E>(inv_rms + at), r);
+            if (coef_out != nullptr) {
+                Elem<T>::unpack(load16<T, false>(read + at), wr);
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const float c = r[e] * wr[e];
+                    coef_out[at + e] = c;
+                    coef_self[at + e] = inv_rms != nullptr ? c * acc[e] / (float)D : 0.0f;
+                }
+            }
+            if (rms_out != nullptr) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) rms_out[at + e] = 1.0f / r[e];
+            }
+        }
+    }
+}
+
 }  // namespace fmscan
