@@ -385,7 +385,9 @@ def layer_step(torch, dev):
 # fewer batch elements and longer rows, where the fused kernels' blocks (one per batch element and group of
 # channels, or per slot, for the whole sequence) become few
 LAYER_SHAPES = [(32, 2048, 32, 128), (8, 8192, 32, 128), (4, 8192, 32, 128), (2, 16384, 32, 128), (1, 32768, 32, 128),
-                (1, 65536, 16, 64), (1, 8192, 32, 2048), (64, 1024, 16, 64)]
+                (1, 65536, 16, 64), (1, 8192, 32, 2048), (64, 1024, 16, 64),
+                # short sequences, many batch elements: rows of at most 256 bytes go several to a wave
+                (256, 256, 32, 128), (256, 128, 32, 128), (512, 64, 32, 128), (1024, 32, 32, 128), (2048, 16, 32, 128)]
 
 
 def run_layer_shapes(torch, args) -> int:
@@ -447,7 +449,8 @@ def run_layer_shapes(torch, args) -> int:
                      "scan_and_norm_in_one_kernel": bool(lib.fmscan_forward_normed_segments(B, M, D, L, 2) > 1
                                                          or lib.fmscan_forward_normed_pays(B, M, D)),
                      "slots_dealt_to_blocks": plan[0], "backward_cut_into": plan[1],
-                     "groups_of_d": int(lib.fmscan_reduced_groups(B * plan[0], D))})
+                     "groups_of_d": int(lib.fmscan_reduced_groups(B * plan[0], D)),
+                     "several_rows_to_a_wave": bool(lib.fmscan_reduced_packed_groups(B, M, D, L, 2) > 0)})
         del alpha, us, osc, inp, w_out
         torch.cuda.empty_cache()
     print(f"{'(B, L, M, D)':>24s} {'elements':>11s} {'step ms':>8s} {'fwd':>7s} {'bwd':>7s} {'Gelem/s':>8s}  routes",
@@ -458,7 +461,10 @@ def run_layer_shapes(torch, args) -> int:
               f"{'scan + norm in one kernel' if r['scan_and_norm_in_one_kernel'] else 'scan, norm, read-out apart'}"
               f"{', sequence cut in %d' % r['sequence_cut_into'] if r['sequence_cut_into'] > 1 else ''}; "
               f"backward: slots of a batch element in {r['slots_dealt_to_blocks']} block(s), "
-              f"{'rows cut in %d, ' % r['backward_cut_into'] if r['backward_cut_into'] > 1 else ''}{r['groups_of_d']} groups of d",
+              f"{'rows cut in %d, ' % r['backward_cut_into'] if r['backward_cut_into'] > 1 else ''}{r['groups_of_d']} groups of d"
+              if not r["several_rows_to_a_wave"] else
+              f"{str(tuple(r['shape'])):>24s} {r['elements']:11d} {r['ms_per_step']:8.3f} {r['fwd_ms']:7.3f} "
+              f"{r['bwd_ms']:7.3f} {r['Gelem_per_s']:8.1f}  short rows: several to a wave in scan + norm, read-out, dot and backward",
               file=sys.stderr)
     print(json.dumps({"metric": "fm_memory layer forward+backward, elements of the (B,M,D,L) states per second",
                       "unit": "Gelem/s", "dtype": "f32", "storage_dtype": "bf16", "data": "synthetic",
