@@ -565,10 +565,12 @@ __global__ __launch_bounds__(256) void readout_forward_packed_kernel(
 // q[b,m,t] = sum_d out_grad[b,d,t] * states_n[b,m,d,t] and what the layer's backward kernel takes with it
 // (rowdot_kernel in its dot form, fmscan_readout.h). A wave is a slot and walks its rows in tiles; the
 // lanes' sums meet across the wave's groups.
-template <typename T>
+template <typename T, bool EXT>
 __global__ __launch_bounds__(256) void readout_dot_packed_kernel(
     const T* __restrict__ states_n /* (B, M, D, L) */, const T* __restrict__ out_grad /* (B, D, L) */,
-    float* __restrict__ q /* (B, M, L) */, const float* __restrict__ inv_rms, const T* __restrict__ read,
+    const T* __restrict__ ext_grad /* (B, M, D, L); EXT */, float* __restrict__ q /* (B, M, L) */,
+    float* __restrict__ qe /* (B, M, L); EXT: sum_d ext_grad * states_n */, const float* __restrict__ inv_rms,
+    const T* __restrict__ read,
     float* __restrict__ coef_out, float* __restrict__ coef_self, float* __restrict__ rms_out, int64_t slots,
     int32_t M, int32_t D, int32_t L, int32_t lpr_log2, int32_t NT) {
     constexpr int E = Elem<T>::E;
@@ -582,17 +584,18 @@ __global__ __launch_bounds__(256) void readout_dot_packed_kernel(
     const int32_t per_tile = 64 >> lpr_log2;
     const bool in_row = p < CL;
     const int32_t t0 = (in_row ? p : CL - 1) * E;
-    float acc[E];
+    float acc[E], acc_ext[E];
 #pragma unroll
-    for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+    for (int e = 0; e < E; ++e) acc[e] = acc_ext[e] = 0.0f;
     struct In {
-        u32x4 h, y;
+        u32x4 h, y, x;
     };
     auto fetch = [&](In& n, int32_t i) {
         const int32_t d_mine = i * per_tile + group;
         const int32_t d = d_mine < D ? d_mine : D - 1;
         n.h = load16<T, true>(states_n + (bm * D + d) * L + t0);
         n.y = load16<T, false>(out_grad + (b * D + d) * L + t0);
+        if constexpr (EXT) n.x = load16<T, true>(ext_grad + (bm * D + d) * L + t0);
     };
     In cur, next;
     fetch(cur, 0);
@@ -604,13 +607,23 @@ __global__ __launch_bounds__(256) void readout_dot_packed_kernel(
         Elem<T>::unpack(cur.y, y);
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[e] = active ? __builtin_fmaf(h[e], y[e], acc[e]) : acc[e];
+        if constexpr (EXT) {
+            Elem<T>::unpack(cur.x, y);
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc_ext[e] = active ? __builtin_fmaf(h[e], y[e], acc_ext[e]) : acc_ext[e];
+        }
         cur = next;
     }
     sum_over_groups<E>(acc, lpr_log2);
+    if constexpr (EXT) sum_over_groups<E>(acc_ext, lpr_log2);
     if (group == 0 && in_row) {
         const int64_t at = bm * L + t0;
 #pragma unroll
-        for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(q + at + e) = make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+        for (int e = 0; e < E; e += 4) {
+            *reinterpret_cast<float4*>(q + at + e) = make_float4(acc[e], acc[e + 1], acc[e + 2], acc[e + 3]);
+            if constexpr (EXT)
+                *reinterpret_cast<float4*>(qe + at + e) = make_float4(acc_ext[e], acc_ext[e + 1], acc_ext[e + 2], acc_ext[e + 3]);
+        }
         if (coef_out != nullptr || rms_out != nullptr) {
             float r[E], wr[E];
 #pragma unroll
@@ -630,6 +643,81 @@ __global__ __launch_bounds__(256) void readout_dot_packed_kernel(
                 for (int e = 0; e < E; ++e) rms_out[at + e] = 1.0f / r[e];
             }
         }
+    }
+}
+
+// dn = read * out_grad (+ ext_grad); with the norm  d h = inv_rms * (dn - states_n * s / D), s = read * q (+ qe)
+// (readout_backward_kernel, fmscan_readout.h). A wave is a batch element and a tile of rows and walks the slots.
+// state_grad may be ext_grad itself: a lane reads its chunk before it writes it.
+template <typename T, bool NORM, bool EXT>
+__global__ __launch_bounds__(256) void readout_backward_packed_kernel(
+    const T* __restrict__ states_n, const float* __restrict__ inv_rms, const T* __restrict__ read,
+    const T* __restrict__ out_grad /* (B, D, L) */, const T* ext_grad /* (B, M, D, L) */, const float* __restrict__ q,
+    const float* __restrict__ qe, T* state_grad /* (B, M, D, L) */, int32_t B, int32_t M, int32_t D, int32_t L,
+    int32_t lpr_log2, int32_t G) {
+    constexpr int E = Elem<T>::E;
+    const int32_t CL = L / E;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + uniform((int)(threadIdx.x >> 6));
+    if (wave >= (int64_t)B * G) return;  // whole waves
+    const int32_t b = uniform((int)(wave / G));
+    const int32_t tile = uniform((int)(wave - (int64_t)b * G));
+    const int32_t p = lane & ((1 << lpr_log2) - 1);
+    const int32_t d_mine = (tile << (6 - lpr_log2)) + (lane >> lpr_log2);
+    const bool active = d_mine < D && p < CL;
+    const int32_t d = d_mine < D ? d_mine : D - 1;
+    const int32_t t0 = (p < CL ? p : CL - 1) * E;
+    float dout[E];
+    Elem<T>::unpack(load16<T, false>(out_grad + ((int64_t)b * D + d) * L + t0), dout);
+    const float inv_d = 1.0f / (float)D;
+    struct In {
+        u32x4 wr, x, hn;
+        FloatChunk<E> r, s, se;
+    };
+    auto fetch = [&](In& n, int32_t m) {
+        const int64_t bm = (int64_t)b * M + m;
+        const int64_t row = (bm * D + d) * L + t0;
+        n.wr = load16<T, false>(read + bm * L + t0);
+        if constexpr (EXT) n.x = load16<T, true>(ext_grad + row);
+        if constexpr (NORM) {
+            n.hn = load16<T, true>(states_n + row);
+            n.r = load_float_chunk<E>(inv_rms + bm * L + t0);
+            n.s = load_float_chunk<E>(q + bm * L + t0);
+            if constexpr (EXT) n.se = load_float_chunk<E>(qe + bm * L + t0);
+        }
+    };
+    In cur, next;
+    fetch(cur, 0);
+    for (int32_t m = 0; m < M; ++m) {
+        fetch(next, m + 1 < M ? m + 1 : m);
+        float wr[E], g[E];
+        Elem<T>::unpack(cur.wr, wr);
+#pragma unroll
+        for (int e = 0; e < E; ++e) g[e] = wr[e] * dout[e];
+        if constexpr (EXT) {
+            float x[E];
+            Elem<T>::unpack(cur.x, x);
+#pragma unroll
+            for (int e = 0; e < E; ++e) g[e] += x[e];
+        }
+        if constexpr (NORM) {
+            float r[E], sv[E], hn[E];
+            spread<E>(cur.r, r);
+            spread<E>(cur.s, sv);
+            Elem<T>::unpack(cur.hn, hn);
+#pragma unroll
+            for (int e = 0; e < E; ++e) sv[e] *= wr[e];
+            if constexpr (EXT) {
+                float se[E];
+                spread<E>(cur.se, se);
+#pragma unroll
+                for (int e = 0; e < E; ++e) sv[e] += se[e];
+            }
+#pragma unroll
+            for (int e = 0; e < E; ++e) g[e] = r[e] * __builtin_fmaf(-hn[e], sv[e] * inv_d, g[e]);
+        }
+        if (active) store16<T>(state_grad + (((int64_t)b * M + m) * D + d) * L + t0, Elem<T>::pack(g));
+        cur = next;
     }
 }
 

@@ -169,17 +169,21 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
             if (overlap(outs[i], outs[j]))
                 return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", outs[i].name, outs[j].name);
     const bool vec = vector_path(rs, {states_n, out_grad, ext_grad});
-    // Rows of at most 256 bytes, many slots, no second gradient: several rows to a wave, a wave per slot
-    if (vec && !ext_grad && L * rs.esize <= 256 && (__int128)B * M >= 4096 && aligned16(q) && aligned16(inv_rms) &&
+    // Rows of at most 256 bytes, many slots: several rows to a wave, a wave per slot
+    if (vec && L * rs.esize <= 256 && (__int128)B * M >= 4096 && aligned16(q) && aligned16(qe) && aligned16(inv_rms) &&
         aligned16(read) && aligned16(coef_out) && aligned16(coef_self) && aligned16(rms_out)) {
         int32_t lanes_log2 = 0;
         while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
         const int64_t per_tile = 64 >> lanes_log2, tiles = (D + per_tile - 1) / per_tile, slots = B * M;
         with_dtype(dtype, [&](auto tt) {
             using T = typename decltype(tt)::type;
-            fmscan::readout_dot_packed_kernel<T><<<(unsigned)((slots + 3) / 4), 256, 0, (hipStream_t)stream>>>(
-                (const T*)states_n, (const T*)out_grad, q, inv_rms, (const T*)read, coef_out, coef_self, rms_out, slots,
-                (int32_t)M, (int32_t)D, (int32_t)L, lanes_log2, (int32_t)tiles);
+            with_bool(ext_grad != nullptr, [&](auto et) {
+                fmscan::readout_dot_packed_kernel<T, decltype(et)::value>
+                    <<<(unsigned)((slots + 3) / 4), 256, 0, (hipStream_t)stream>>>(
+                        (const T*)states_n, (const T*)out_grad, (const T*)ext_grad, q, qe, inv_rms, (const T*)read,
+                        coef_out, coef_self, rms_out, slots, (int32_t)M, (int32_t)D, (int32_t)L, lanes_log2,
+                        (int32_t)tiles);
+            });
         });
         return launched("read-out (dot)");
     }
@@ -227,6 +231,27 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
     const bool vec = vector_path(rs, {norm ? states_n : nullptr, inv_rms, read, out_grad, ext_grad,
                                       norm ? (const void*)q : nullptr, norm && ext_grad ? (const void*)qe : nullptr,
                                       state_grad});
+    // Rows of at most 256 bytes, enough (b, tile of rows) pairs: several rows to a wave (fmscan_packed.h)
+    if (vec && L * rs.esize <= 256) {
+        int32_t lanes_log2 = 0;
+        while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
+        const int64_t per_tile = 64 >> lanes_log2, groups = (D + per_tile - 1) / per_tile;
+        if ((__int128)B * groups >= 4096 && (__int128)B * groups <= (__int128)INT32_MAX && B <= INT32_MAX) {
+            with_dtype(dtype, [&](auto tt) {
+                using T = typename decltype(tt)::type;
+                with_bool(norm, [&](auto nt) {
+                    with_bool(ext_grad != nullptr, [&](auto et) {
+                        fmscan::readout_backward_packed_kernel<T, decltype(nt)::value, decltype(et)::value>
+                            <<<(unsigned)((B * groups + 3) / 4), 256, 0, (hipStream_t)stream>>>(
+                                (const T*)states_n, inv_rms, (const T*)read, (const T*)out_grad, (const T*)ext_grad, q, qe,
+                                (T*)state_grad, (int32_t)B, (int32_t)M, (int32_t)D, (int32_t)L, lanes_log2,
+                                (int32_t)groups);
+                    });
+                });
+            });
+            return launched("read-out (backward)");
+        }
+    }
     const dim3 grid((unsigned)(B * rs.tiles), (unsigned)((D + 4 * kReadoutRows - 1) / (4 * kReadoutRows)));
     int rc = 0;
     with_dtype(dtype, [&](auto tt) {
