@@ -207,8 +207,8 @@ __global__ __launch_bounds__(256) void scan_backward_packed_kernel(
 // the token gradient over the M slots and the gate gradient over the D rows of a slot, in float32. A wave
 // is a batch element b and a tile of 64 >> lpr_log2 consecutive rows d, and walks the M slots: the token
 // gradient of its rows adds up in registers and is stored once; the gate gradient of a slot is added
-// across the wave's groups (rotations inside the 16-lane rows, then the rows change places in a copy: every
-// lane ends with the sum) and the first group stores it as one of G = ceil(D / rows of a tile) float32
+// across the wave's groups (the halves of the wave, then the 16-lane rows, trade the values the other is
+// to keep; rotations inside the rows finish) and stored as one of G = ceil(D / rows of a tile) float32
 // partial sums, gate_grad_partial (B * M, G, L), which fmscan_sum_groups adds. No LDS, no barrier; the
 // loads of the next slot are in flight while a slot is worked on. Sums are taken in a fixed order.
 // v + (v of the lane 16 or 32 away): the two halves change places in a copy and meet in an add
@@ -384,12 +384,36 @@ __global__ __launch_bounds__(256) void scan_backward_reduced_packed_kernel(
             }
             dg[e] = active ? mine : 0.0f;
         }
-        sum_over_groups<E>(dg, lpr_log2);
-        if (group == 0 && p < CL) {
-            float* dst = gate_grad_partial + (gate_row * G + tile) * L + t0;
+        // The sum over the wave's groups, each quarter of the wave ending with a quarter of the values: the
+        // halves of the wave, then the 16-lane rows of a half, trade what the other is to keep (one exchange
+        // and one add per pair of values), and only what is left is summed inside the 16-lane rows.
+        float kept[E / 4];
+        {
+            float half[E / 2];
 #pragma unroll
-            for (int e = 0; e < E; e += 4)
-                *reinterpret_cast<float4*>(dst + e) = make_float4(dg[e], dg[e + 1], dg[e + 2], dg[e + 3]);
+            for (int e = 0; e < E / 2; ++e) {
+                const auto r = __builtin_amdgcn_permlane32_swap(f2u(dg[e]), f2u(dg[e + E / 2]), false, false);
+                half[e] = u2f(r[0]) + u2f(r[1]);  // lanes 0-31: value e, lanes 32-63: value e + E/2
+            }
+#pragma unroll
+            for (int e = 0; e < E / 4; ++e) {
+                const auto r = __builtin_amdgcn_permlane16_swap(f2u(half[e]), f2u(half[e + E / 4]), false, false);
+                kept[e] = u2f(r[0]) + u2f(r[1]);  // even 16-lane rows: value e of the half, odd ones: e + E/4
+            }
+#pragma unroll
+            for (int e = 0; e < E / 4; ++e) {
+                if (lpr_log2 <= 3) kept[e] += dpp<0x128, 0xf>(kept[e], kept[e]);  // row_ror:8
+                if (lpr_log2 <= 2) kept[e] += dpp<0x124, 0xf>(kept[e], kept[e]);  // row_ror:4
+                if (lpr_log2 <= 1) kept[e] += dpp<0x122, 0xf>(kept[e], kept[e]);  // row_ror:2
+                if (lpr_log2 <= 0) kept[e] += dpp<0x121, 0xf>(kept[e], kept[e]);  // row_ror:1
+            }
+        }
+        // the first group of every 16-lane row stores its quarter: values (half * E/2 + odd row * E/4) onwards
+        if ((lane & 15) < (1 << lpr_log2) && p < CL) {
+            const int32_t first = (lane >> 5) * (E / 2) + ((lane >> 4) & 1) * (E / 4);
+            float* dst = gate_grad_partial + (gate_row * G + tile) * L + t0 + first;
+            if constexpr (E == 8) *reinterpret_cast<float2*>(dst) = make_float2(kept[0], kept[1]);
+            else dst[0] = kept[0];
         }
         cur = next;
     }
