@@ -283,6 +283,17 @@ inline unsigned packed_blocks(const Problem& pb, int32_t lanes_log2) {
     return (unsigned)((waves + 3) / 4);
 }
 
+// The kernels of the layer and of the backward scan with the sums inside that put several rows into a wave
+// (fmscan_packed.h) give a wave a slot, or a batch element and a tile of rows, for the whole of its loop:
+// they are taken from this many waves on. Measured on the backward kernel with the sums inside (bf16, us, the
+// general routes against the packed kernel): (B,M,D,L) = (64,32,128,64), 1024 waves, 98 against 52;
+// (128,32,128,64) 187 / 62; (256,16,64,32), 1024 waves, 105 / 31; (128,16,64,32), 512 waves, 56 / 32;
+// (32,32,128,64), 512 waves, 53 / 49; (16,32,128,128), 512 waves, 44 / 49; with 256 waves 43-47 either way.
+#ifndef FMSCAN_PACKED_MIN_WAVES
+#define FMSCAN_PACKED_MIN_WAVES 512
+#endif
+constexpr int64_t kPackedMinWaves = FMSCAN_PACKED_MIN_WAVES;
+
 // Expands run-time choices into template arguments: F is a generic lambda called with tags.
 template <typename T> struct TypeTag { using type = T; };
 template <int V> struct IntTag { static constexpr int value = V; };

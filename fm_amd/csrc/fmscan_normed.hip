@@ -113,7 +113,7 @@ static int forward_normed(const char* who, const void* gates, const void* tokens
     }
     // Rows of at most 256 bytes, many slots: several rows to a wave, a wave per slot (fmscan_packed.h), where
     // a slot's rows fit the tiles a wave holds; the layer's forward at (B,L,M,D) = (512,64,32,128) bf16: 0.60 -> 0.25 ms.
-    if (segments == 1 && L * pb.esize <= 256 && aligned16(inv_rms) && (__int128)B * M >= 4096) {
+    if (segments == 1 && L * pb.esize <= 256 && aligned16(inv_rms) && (__int128)B * M >= kPackedMinWaves) {
         const int32_t lanes_log2 = packed_lanes_log2(pb);
         const int64_t per_tile = 64 >> lanes_log2, tiles = (D + per_tile - 1) / per_tile;
         if (tiles <= 32) {

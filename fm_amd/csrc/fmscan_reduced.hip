@@ -305,9 +305,8 @@ int64_t fmscan_reduced_packed_groups(int64_t B, int64_t M, int64_t D, int64_t L,
     while ((16 << lanes_log2) < row_bytes) ++lanes_log2;
     const int64_t per_tile = 64 >> lanes_log2;
     const int64_t groups = (D + per_tile - 1) / per_tile;
-    // a wave per (b, tile): below about four waves per SIMD of the whole GPU fmscan_backward and the two sums
-    // are faster (they spread over rows, not over (b, tile) pairs)
-    if ((__int128)B * groups < 4096) return 0;
+    // a wave per (b, tile): with few of them the routes that spread over rows are as fast or faster
+    if ((__int128)B * groups < kPackedMinWaves) return 0;
     return groups;
 }
 
@@ -328,7 +327,7 @@ static int backward_reduced_packed(const char* who, const void* gates, const voi
     const int64_t groups = fmscan_reduced_packed_groups(B, M, D, L, dtype);
     if (groups < 1)
         return fail(FMSCAN_E_SHAPE, "%s: not for this shape (fmscan_reduced_packed_groups is 0): rows of whole "
-                    "16-byte vectors up to 256 bytes, 4096 (b, tile of rows) pairs or more", who);
+                    "16-byte vectors up to 256 bytes, 512 (b, tile of rows) pairs or more", who);
     if (!gates || !out_grad || !token_grad || (!cached_output && !recover) || !gate_grad_partial)
         return fail(FMSCAN_E_NULL, "%s: gates, %s, token_grad, cached_output and gate_grad_partial must not "
                     "be NULL", who, layer ? "states_n" : "out_grad");

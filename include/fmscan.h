@@ -277,7 +277,7 @@ int fmscan_reduced_pays(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
  * takes one batch element and a tile of rows d and walks the M slots: token_grad (B, D, L) is complete,
  * gate_grad_partial is (B, M, G, L) float32 with G = fmscan_reduced_packed_groups(B, M, D, L, dtype), to be
  * added by fmscan_sum_groups. That query returns 0 where the call does not apply (longer or unaligned rows,
- * fewer than 4096 (b, tile) pairs): then the call returns FMSCAN_E_SHAPE. Arguments, flags (FMSCAN_FLAG_PLAIN
+ * fewer than 512 (b, tile) pairs): then the call returns FMSCAN_E_SHAPE. Arguments, flags (FMSCAN_FLAG_PLAIN
  * only) and results otherwise as fmscan_backward_reduced; results agree with it to float32 rounding.
  * No counterpart in the reference (fm_scan.py:70-78 writes two (B, M, D, L) tensors and sums them). */
 int64_t fmscan_reduced_packed_groups(int64_t B, int64_t M, int64_t D, int64_t L, int dtype);
