@@ -293,6 +293,12 @@ inline unsigned packed_blocks(const Problem& pb, int32_t lanes_log2) {
 #define FMSCAN_PACKED_MIN_WAVES 512
 #endif
 constexpr int64_t kPackedMinWaves = FMSCAN_PACKED_MIN_WAVES;
+// The read-out's kernels and the dot have less to do per wave and general forms that hold up longer: four
+// times as many (us, general / packed, bf16: read-out (B,M,D,L) = (32,32,128,64), 512 waves, 15 / 18,
+// (128,32,128,64), 2048 waves, 30 / 22, (64,32,128,128), 2048 waves, 18 / 22, (128,32,128,128) 34 / 25;
+// dot (16,32,128,64), 512 waves, 8 / 11, (32,32,128,64) 14 / 12, (64,32,128,128), 2048 waves, 27 / 22;
+// scan + norm (16,32,128,64), 512 waves, 16 / 9, (16,32,128,128) 15 / 15, (8,32,128,128), 256 waves, 8 / 15).
+constexpr int64_t kPackedMinWavesReadout = 4 * kPackedMinWaves;
 
 // Expands run-time choices into template arguments: F is a generic lambda called with tags.
 template <typename T> struct TypeTag { using type = T; };

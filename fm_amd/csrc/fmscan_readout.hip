@@ -114,7 +114,7 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
         int32_t lanes_log2 = 0;
         while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
         const int64_t per_tile = 64 >> lanes_log2, groups = (D + per_tile - 1) / per_tile;
-        if ((__int128)B * groups >= kPackedMinWaves && (__int128)B * groups <= (__int128)INT32_MAX && B <= INT32_MAX) {
+        if ((__int128)B * groups >= kPackedMinWavesReadout && (__int128)B * groups <= (__int128)INT32_MAX && B <= INT32_MAX) {
             with_dtype(dtype, [&](auto tt) {
                 using T = typename decltype(tt)::type;
                 fmscan::readout_forward_packed_kernel<T><<<(unsigned)((B * groups + 3) / 4), 256, 0, (hipStream_t)stream>>>(
@@ -170,7 +170,7 @@ int fmscan_readout_dot(const void* states_n, const void* out_grad, const void* e
                 return fail(FMSCAN_E_ALIAS, "fmscan_readout_dot: %s overlaps %s", outs[i].name, outs[j].name);
     const bool vec = vector_path(rs, {states_n, out_grad, ext_grad});
     // Rows of at most 256 bytes, many slots: several rows to a wave, a wave per slot
-    if (vec && L * rs.esize <= 256 && (__int128)B * M >= kPackedMinWaves && aligned16(q) && aligned16(qe) && aligned16(inv_rms) &&
+    if (vec && L * rs.esize <= 256 && (__int128)B * M >= kPackedMinWavesReadout && aligned16(q) && aligned16(qe) && aligned16(inv_rms) &&
         aligned16(read) && aligned16(coef_out) && aligned16(coef_self) && aligned16(rms_out)) {
         int32_t lanes_log2 = 0;
         while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
@@ -236,7 +236,7 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
         int32_t lanes_log2 = 0;
         while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
         const int64_t per_tile = 64 >> lanes_log2, groups = (D + per_tile - 1) / per_tile;
-        if ((__int128)B * groups >= kPackedMinWaves && (__int128)B * groups <= (__int128)INT32_MAX && B <= INT32_MAX) {
+        if ((__int128)B * groups >= kPackedMinWavesReadout && (__int128)B * groups <= (__int128)INT32_MAX && B <= INT32_MAX) {
             with_dtype(dtype, [&](auto tt) {
                 using T = typename decltype(tt)::type;
                 with_bool(norm, [&](auto nt) {
