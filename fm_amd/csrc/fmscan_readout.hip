@@ -4,6 +4,14 @@
 #include "fmscan_readout.h"
 #include "fmscan_packed.h"
 
+// Rows up to this many bytes take the packed forms of the read-out's two kernels, which have no sum across
+// lanes and so no limit on the lanes of a group (bf16, us, general / packed, forward and backward:
+// (256,32,128,192) 85 / 67 and 272 / 208, (256,32,128,256) 96 / 91 and 278 / 239, (128,32,128,512) 89 / 108 and
+// 217 / 311).
+#ifndef FMSCAN_READOUT_PACKED_BYTES
+#define FMSCAN_READOUT_PACKED_BYTES 512
+#endif
+
 using namespace fmscan::host;
 
 namespace {
@@ -110,7 +118,7 @@ int fmscan_readout_forward(const void* states, const float* inv_rms, const void*
     const bool vec = vector_path(rs, {states, inv_rms, read, inv_rms ? states_out : nullptr, output});
     // Rows of at most 256 bytes without the norm (the layer's read-out of normalised states), enough
     // (b, tile of rows) pairs: several rows to a wave (fmscan_packed.h)
-    if (vec && !inv_rms && L * rs.esize <= 256) {
+    if (vec && !inv_rms && L * rs.esize <= FMSCAN_READOUT_PACKED_BYTES) {
         int32_t lanes_log2 = 0;
         while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
         const int64_t per_tile = 64 >> lanes_log2, groups = (D + per_tile - 1) / per_tile;
@@ -232,7 +240,7 @@ int fmscan_readout_backward(const void* states_n, const float* inv_rms, const vo
                                       norm ? (const void*)q : nullptr, norm && ext_grad ? (const void*)qe : nullptr,
                                       state_grad});
     // Rows of at most 256 bytes, enough (b, tile of rows) pairs: several rows to a wave (fmscan_packed.h)
-    if (vec && L * rs.esize <= 256) {
+    if (vec && L * rs.esize <= FMSCAN_READOUT_PACKED_BYTES) {
         int32_t lanes_log2 = 0;
         while ((16 << lanes_log2) < L * rs.esize) ++lanes_log2;
         const int64_t per_tile = 64 >> lanes_log2, groups = (D + per_tile - 1) / per_tile;

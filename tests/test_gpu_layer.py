@@ -91,6 +91,7 @@ LAYER_SHAPES = [
     ((2060, 24, 2, 20), 1e-4, "rows of at most 256 bytes, many batch elements: several rows to a wave in backward "
                               "(4 lanes a row in bfloat16, 8 in float32; D not a multiple of the rows of a wave)"),
     ((1400, 32, 3, 70), 1e-4, "the same with 4 / 8 lanes a row and three slots"),
+    ((420, 200, 2, 20), 1e-4, "rows of 400 bytes in bfloat16: the read-out's kernels alone put two rows into a wave"),
 ]
 
 
