@@ -69,7 +69,9 @@ extern "C" {
 /* With none of the four choices above made by the caller, fmscan_forward, fmscan_forward_static and
  * fmscan_backward put rows of at most 1 KiB several to a wave (a kernel of its own, a segmented wave scan);
  * any of them set selects the general kernels, which give a wave one row at a time. Results agree to
- * float32 rounding. */
+ * float32 rounding. The layer's calls (fmscan_forward_normed, fmscan_readout_forward, fmscan_readout_backward,
+ * fmscan_readout_dot) do the same by themselves for rows of at most 256 bytes (512 for the read-out's two)
+ * when there is enough work for it; their results do not change shape. */
 
 /* error codes (negative returns) */
 #define FMSCAN_E_NULL      (-1) /* a required pointer is NULL */
